@@ -1,0 +1,259 @@
+/*
+ * mi355_moe.h -- C ABI of the MI355X (gfx950) MoE-block kernels.
+ *
+ * Every entry point takes plain device pointers, sizes and a HIP stream
+ * (passed as void*; NULL = the null stream) and returns 0 on success or a
+ * negative MI355_E* code; mi355_moe_last_error() then describes the failure
+ * (thread-local text).  No entry point synchronises the host with the device and
+ * none allocates device memory: outputs and workspaces are caller-owned.
+ * All kernels of one call run on the given stream in program order.
+ *
+ * The reference (TorchLLMTuner) has no FFI: its MoE block is a composition of
+ * PyTorch ops.  Each declaration therefore cites the reference lines whose
+ * arithmetic it replaces (paths relative to the reference checkout).
+ *
+ * Shape legend: T tokens, D model dim, E experts, K experts per token, N = T*K
+ * assignment slots (flat index t*K + k), F expert hidden dim, R rows of the
+ * expert-major buffer, El = number of local experts (hi - lo).
+ */
+#ifndef MI355_MOE_H
+#define MI355_MOE_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI355_MOE_ABI_VERSION 1
+
+/* element types of activation / weight buffers */
+#define MI355_F32 0
+#define MI355_BF16 1
+
+/* score functions: llmtuner/models/common/moe/routing.py:270-277 */
+#define MI355_SCORE_SIGMOID 0
+#define MI355_SCORE_SOFTMAX 1
+#define MI355_SCORE_SQRTSOFTPLUS 2
+
+/* selection modes: routing.py:291-303 */
+#define MI355_SELECT_TOPK 0     /* biased top-k, optionally group-limited   */
+#define MI355_SELECT_FIXED 1    /* fixed_router: (t + k) % E, weights 1/K   */
+#define MI355_SELECT_BALANCED 2 /* _debug_force_load_balance: (t*K + k) % E */
+
+/* error codes */
+#define MI355_OK 0
+#define MI355_EINVAL (-1)  /* bad argument (shape, dtype, alignment, null)  */
+#define MI355_ELAUNCH (-2) /* a HIP launch or runtime call failed           */
+#define MI355_EUNSUP (-3)  /* valid request this build does not implement   */
+
+int mi355_moe_abi_version(void);
+const char* mi355_moe_last_error(void);
+
+/* ------------------------------------------------------------------ router */
+
+/*
+ * logits_TE[t][e] = sum_d x[t][d] * w[e][d]  (+ logit_bias[e]), fp32 output and
+ * fp32 accumulation whatever the storage types.
+ * Replaces RouterGateLinearFunction.forward and RouterGateLinear.forward,
+ * llmtuner/models/common/linear.py:107-131,179-183.
+ * x: (T,D) x_dtype row-major; w: (E,D) w_dtype; logit_bias: (E) fp32 or NULL.
+ */
+int mi355_router_gate_fwd(const void* x, int x_dtype, const void* w, int w_dtype,
+                          const float* logit_bias, float* logits_TE,
+                          int64_t T, int64_t D, int64_t E, void* stream);
+
+/*
+ * dx[t][d] = sum_e dlogits[t][e] * w[e][d]   (written in x_dtype; NULL = skip)
+ * dw[e][d] = sum_t dlogits[t][e] * x[t][d]   (written in w_dtype; NULL = skip)
+ * both accumulated in fp32.  Replaces RouterGateLinearFunction.backward,
+ * linear.py:133-151.  workspace: mi355_router_gate_bwd_workspace_bytes() bytes
+ * (split-K partial sums for dw), may be NULL when dw is NULL.
+ */
+int64_t mi355_router_gate_bwd_workspace_bytes(int64_t T, int64_t D, int64_t E);
+int mi355_router_gate_bwd(const float* dlogits_TE, const void* x, int x_dtype,
+                          const void* w, int w_dtype, void* dx, void* dw,
+                          void* workspace, int64_t T, int64_t D, int64_t E,
+                          void* stream);
+
+/*
+ * Scores, expert choice, gather, norm and scale in one pass over the logits.
+ * Replaces TokenChoiceTopKRouter.forward after the gate, routing.py:270-324:
+ * score function (:270-277), biased top-k (:168-192) or group-limited top-k
+ * (:194-239; group score = sum of the group's top-2, top num_limited groups kept,
+ * the rest masked to -inf), unbiased gather, route_norm with +1e-20, route_scale
+ * (:311-315), and the fixed / balanced debug routings (:291-309, :146-166).
+ * Selection order is "higher choice score first, ties to the lower expert id";
+ * ids are emitted in that order.
+ * expert_bias: (E) fp32 or NULL.  num_groups = 0 disables grouping.
+ * scores_TE: optional (T,E) fp32 output of the score function (NULL = skip).
+ */
+int mi355_router_select_fwd(const float* logits_TE, const float* expert_bias,
+                            float* weights_TK, int64_t* ids_TK, float* scores_TE,
+                            int64_t T, int64_t E, int64_t K, int score_func,
+                            int route_norm, float route_scale, int num_groups,
+                            int num_limited, int select_mode, void* stream);
+
+/*
+ * dlogits_TE from dweights_TK (and, optionally, a dense gradient dscores_TE on the
+ * full score map, e.g. from an auxiliary loss; NULL = none): the backward of the
+ * gather / norm / scale / score chain that autograd derives for routing.py:270-315.
+ * For MI355_SELECT_FIXED the weights are constants and only dscores_TE flows.
+ */
+int mi355_router_select_bwd(const float* logits_TE, const int64_t* ids_TK,
+                            const float* dweights_TK, const float* dscores_TE,
+                            float* dlogits_TE, int64_t T, int64_t E, int64_t K,
+                            int score_func, int route_norm, float route_scale,
+                            int select_mode, void* stream);
+
+/* ------------------------------------------------------- permutation plan */
+
+/*
+ * Expert-major layout of the N = T*K assignment slots, stable in the flat slot
+ * index (bit-identical to argsort(ids.flatten(), stable=True)).
+ * Replaces LocalTokenDispatcher._local_reorder's index work,
+ * llmtuner/parallel/expert_parallel/token_dispatch.py:180-186, the routing-map
+ * count layer.py:278, GroupedExperts' cumsum experts.py:204, and -- with
+ * align > 1 -- the padded layout of TorchAOTokenDispatcher._permute,
+ * torchao_dispatch.py:143-175 (contract:
+ * tests/unit_tests/cpu/models/test_moe_token_dispatch.py:154-179): each local
+ * expert's segment is padded up to a multiple of `align` rows; an empty expert gets
+ * no padding.
+ *
+ * Only experts in [local_lo, local_hi) receive rows (one rank's share of an
+ * expert-parallel layout, token_dispatch.py:367-371); other slots get row -1 but
+ * are still counted.
+ *
+ * Outputs (all caller-allocated, int32):
+ *   counts_E      (E)     slots per expert, over all experts
+ *   seg_offsets   (El+1)  first row of each local segment; [El] = total rows used
+ *   seg_counts    (El)    real (unpadded) rows per local segment
+ *   row_of_slot   (N)     row of slot t*K+k, or -1 when not local
+ *   slot_of_row   (row_capacity) slot held by each row, -1 for padding / unused
+ *   tile_expert, tile_row0 (tile_capacity each) and num_tiles (1): the list of
+ *       tile_m-row tiles covering the real rows of every segment (local expert
+ *       index and first row of each tile)
+ * row_capacity  >= N + El*(align-1) is always enough;
+ * tile_capacity >= N/tile_m + El + 1 is always enough.
+ * workspace: mi355_permute_plan_workspace_bytes(T,K,E) bytes.
+ * ids outside [0,E) make the result undefined but never write out of bounds.
+ */
+int64_t mi355_permute_plan_workspace_bytes(int64_t T, int64_t K, int64_t E);
+int mi355_permute_plan(const int64_t* ids_TK, int64_t T, int64_t K, int64_t E,
+                       int64_t local_lo, int64_t local_hi, int64_t align,
+                       int64_t tile_m, int32_t* counts_E, int32_t* seg_offsets,
+                       int32_t* seg_counts, int32_t* row_of_slot,
+                       int32_t* slot_of_row, int64_t row_capacity,
+                       int32_t* tile_expert, int32_t* tile_row0, int32_t* num_tiles,
+                       int64_t tile_capacity, void* workspace, void* stream);
+
+/*
+ * Segment offsets, counts and the tile list for rows that are ALREADY expert-major
+ * with `counts[e]` rows per local expert (no padding): the layout
+ * GroupedExperts.forward receives, llmtuner/models/common/moe/experts.py:152-204
+ * (offsets_E = cumsum(counts), :204).  counts: (El) int32; negative counts are
+ * treated as 0 and segments are clamped to the row_capacity rows that exist.
+ * tile_capacity >= row_capacity/tile_m + El is always enough.
+ */
+int mi355_segments_from_counts(const int32_t* counts, int64_t El, int64_t tile_m,
+                               int64_t row_capacity, int32_t* seg_offsets, int32_t* seg_counts,
+                               int32_t* tile_expert, int32_t* tile_row0,
+                               int32_t* num_tiles, int64_t tile_capacity, void* stream);
+
+/*
+ * rows[r] = x[slot_of_row[r] / K], zero for padding rows; rows at or beyond
+ * seg_offsets[El] are left untouched.  Replaces the gather x[token_indices],
+ * token_dispatch.py:197-199, and the sentinel-row padding of the padded layout.
+ * total_rows points at seg_offsets[El] on the device.
+ */
+int mi355_permute_rows_fwd(const void* x, int dtype, const int32_t* slot_of_row,
+                           const int32_t* total_rows, void* rows, int64_t T,
+                           int64_t D, int64_t K, int64_t row_capacity,
+                           void* stream);
+
+/*
+ * dx[t] = sum_k drows[row_of_slot[t*K+k]] (slots with row -1 contribute nothing),
+ * summed in fp32 in ascending k, written in `dtype`.  This is the backward of the
+ * row gather (autograd's index_put accumulate for token_dispatch.py:199; the
+ * duplicate-row contract is tests/unit_tests/cpu/kernel/test_kernel_contracts.py:
+ * 114-127).
+ */
+int mi355_permute_rows_bwd(const void* drows, int dtype, const int32_t* row_of_slot,
+                           void* dx, int64_t T, int64_t D, int64_t K, void* stream);
+
+/* ------------------------------------------------------------------ combine */
+
+/*
+ * out[t] = sum_k weights[t][k] * y[row_of_slot[t*K+k]], contributions taken in
+ * ascending row order (the order index_add visits them in).  Replaces
+ * LocalTokenDispatcher.combine, token_dispatch.py:255-275, and the padding strip
+ * of TorchAOTokenDispatcher._unpermute, torchao_dispatch.py:177-185.
+ * round_terms != 0 reproduces the reference's default rounding (each weighted row
+ * rounded to the y dtype before the sum, accumulate_in_fp32 = False); 0 keeps the
+ * products in fp32 (accumulate_in_fp32 = True).  The sum itself is always fp32 and
+ * rounded once to `dtype`.
+ */
+int mi355_combine_fwd(const void* y, int dtype, const float* weights_TK,
+                      const int32_t* row_of_slot, void* out, int64_t T, int64_t D,
+                      int64_t K, int round_terms, void* stream);
+
+/*
+ * dy[row] = weights[t][k] * dout[t]   for every slot with a row (rows that hold
+ *           padding are zeroed up to *total_rows)
+ * dweights[t][k] = sum_d y[row][d] * dout[t][d]   (0 for slots without a row)
+ * The autograd-derived backward of token_dispatch.py:263-274.
+ */
+int mi355_combine_bwd(const void* dout, const void* y, int dtype,
+                      const float* weights_TK, const int32_t* row_of_slot,
+                      const int32_t* slot_of_row, const int32_t* total_rows,
+                      void* dy, float* dweights_TK, int64_t T, int64_t D, int64_t K,
+                      int64_t row_capacity, void* stream);
+
+/* ---------------------------------------------------- grouped SwiGLU experts */
+
+/*
+ * For every tile-listed row r of local expert e:
+ *   gate[r] = rows[r] . w1[e]^T,  up[r] = rows[r] . w3[e]^T      (R,F)
+ *   h[r]    = silu(gate[r]) * up[r]                              (R,F)
+ *   y[r]    = h[r] . w2[e]^T                                     (R,D)
+ * with gate, up, the SiLU value, the product and y each rounded to `dtype`
+ * (the reference's rounding points).  Replaces GroupedExperts._compute,
+ * llmtuner/models/common/moe/experts.py:204-209, its _grouped_mm (:211-285) and
+ * SwiGLU.forward, llmtuner/models/common/activation.py:36-37.
+ * w1,w3: (El,F,D); w2: (El,D,F), all `dtype`, row-major.
+ * gate/up/h are saved for the backward (each (row_capacity,F)).
+ * bf16 uses MFMA tiles of tile_m rows (the plan's tile list must have been built
+ * with the value mi355_grouped_tile_m(dtype) returns).
+ */
+int64_t mi355_grouped_tile_m(int dtype);
+int mi355_grouped_swiglu_fwd(const void* rows, const void* w1, const void* w3,
+                             const void* w2, int dtype, const int32_t* seg_offsets,
+                             const int32_t* seg_counts, const int32_t* tile_expert,
+                             const int32_t* tile_row0, const int32_t* num_tiles,
+                             int64_t tile_capacity, void* gate, void* up, void* h,
+                             void* y, int64_t El, int64_t D, int64_t F,
+                             int64_t row_capacity, void* stream);
+
+/*
+ * Backward of the above (autograd-derived in the reference):
+ *   dh = dy . w2[e];  dgate = dh * up * silu'(gate);  dup = dh * silu(gate)
+ *   drows = dgate . w1[e] + dup . w3[e]
+ *   dw2[e] = dy_e^T . h_e;  dw1[e] = dgate_e^T . rows_e;  dw3[e] = dup_e^T . rows_e
+ * dgate/dup are caller-provided scratch of (row_capacity,F) each.  Weight
+ * gradients are written (not accumulated) in `dtype`; experts with no rows get
+ * zeros.  Any of drows/dw1/dw3/dw2 may be NULL to skip it.
+ */
+int mi355_grouped_swiglu_bwd(const void* dy, const void* rows, const void* w1,
+                             const void* w3, const void* w2, const void* gate,
+                             const void* up, const void* h, int dtype,
+                             const int32_t* seg_offsets, const int32_t* seg_counts,
+                             const int32_t* tile_expert, const int32_t* tile_row0,
+                             const int32_t* num_tiles, int64_t tile_capacity,
+                             void* dgate, void* dup, void* drows, void* dw1,
+                             void* dw3, void* dw2, int64_t El, int64_t D, int64_t F,
+                             int64_t row_capacity, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355_MOE_H */

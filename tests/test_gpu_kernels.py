@@ -1,0 +1,302 @@
+"""GPU parity of every kernel, called through the C ABI (torchllmtuner_amd.ops),
+against the CPU oracle on identical seeded inputs.
+
+Bars: routing ids, counts and permutation order bit-exact (on tokens whose decision
+is not a few-ulp near tie, see helpers.stable_tokens); fp32 values within 1e-5
+relative; bf16 values within 2e-2 relative L2.
+"""
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import moe_ref as R
+from tests.helpers import rel_l2, rel_max, stable_tokens
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+FP32_TOL = 1e-5
+BF16_TOL = 2e-2
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from torchllmtuner_amd import ops as _ops
+
+    return _ops
+
+
+# ---------------------------------------------------------------- router gate
+@pytest.mark.parametrize("T,D,E,xdt", [(3, 8, 4, torch.float32), (512, 256, 8, torch.float32),
+                                       (1000, 320, 72, torch.bfloat16), (0, 16, 4, torch.float32)])
+def test_router_gate_fwd_bwd(ops, T, D, E, xdt):
+    print(f"router_gate T={T} D={D} E={E} {xdt}", flush=True)
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(T, D, generator=g).to(xdt)
+    w = torch.randn(E, D, generator=g) * 0.05
+    b = torch.randn(E, generator=g)
+    gout = torch.randn(T, E, generator=g)
+    xr, wr = x.clone().requires_grad_(), w.clone().requires_grad_()
+    ref = R.router_gate(xr, wr, b)
+    got = ops.router_gate_fwd(x.to(DEV), w.to(DEV), b.to(DEV))
+    assert got.dtype == torch.float32 and got.shape == (T, E)
+    if T == 0:
+        return
+    assert rel_max(got, ref) < FP32_TOL
+    ref.backward(gout)
+    dx, dw = ops.router_gate_bwd(gout.to(DEV), x.to(DEV), w.to(DEV))
+    assert dx.dtype == xdt and dw.dtype == torch.float32
+    assert rel_max(dx, xr.grad) < (FP32_TOL if xdt == torch.float32 else 1e-2)
+    assert rel_max(dw, wr.grad) < FP32_TOL
+
+
+# ---------------------------------------------------------------- router select
+SELECT_CASES = [
+    dict(T=512, E=8, K=2, score_func="softmax", route_norm=True),
+    dict(T=2048, E=128, K=8, score_func="softmax", route_norm=True),
+    dict(T=1024, E=256, K=8, score_func="sigmoid", route_norm=True, route_scale=2.5,
+         num_expert_groups=8, num_limited_groups=4, bias=True),
+    dict(T=300, E=64, K=6, score_func="sigmoid", bias=True),
+    dict(T=300, E=24, K=3, score_func="sqrtsoftplus", route_norm=True, route_scale=0.5),
+    dict(T=257, E=320, K=5, score_func="softmax", num_expert_groups=5, num_limited_groups=2),
+    dict(T=10, E=4, K=2, score_func="sigmoid", fixed_router=True, route_scale=7.0),
+    dict(T=10, E=4, K=2, score_func="sigmoid", debug_force_load_balance=True, route_norm=True, route_scale=2.0),
+]
+
+
+@pytest.mark.parametrize("case", SELECT_CASES, ids=lambda c: f"E{c['E']}K{c['K']}{c['score_func']}")
+def test_router_select_fwd_bwd(ops, case):
+    print(f"router_select {case}", flush=True)
+    c = dict(case)
+    T, E, K = c.pop("T"), c.pop("E"), c.pop("K")
+    use_bias = c.pop("bias", False)
+    spec = R.RouterSpec(E, K, **c)
+    g = torch.Generator().manual_seed(7)
+    logits = torch.randn(T, E, generator=g) * 1.5
+    bias = (torch.rand(E, generator=g) * 0.2 - 0.1) if use_bias else None
+    lr = logits.clone().requires_grad_()
+    w_ref, ids_ref, _ = R.route(lr, spec, bias)
+    mode = 1 if spec.fixed_router else (2 if spec.debug_force_load_balance else 0)
+    w, ids, scores = ops.router_select_fwd(
+        logits.to(DEV), None if bias is None else bias.to(DEV), K, spec.score_func, spec.route_norm,
+        spec.route_scale, spec.num_expert_groups or 0, spec.num_limited_groups or 0, mode, True)
+    assert ids.dtype == torch.int64
+    ok = torch.ones(T, dtype=torch.bool) if mode else stable_tokens(logits, spec, bias)
+    assert ok.float().mean() > 0.98, "too many near-tie tokens for a meaningful check"
+    assert torch.equal(ids.cpu()[ok], ids_ref[ok]), "routing ids differ on tokens that are not near ties"
+    assert rel_max(scores, R.score(logits, spec.score_func)) < FP32_TOL
+    assert rel_max(w.cpu()[ok], w_ref[ok]) < FP32_TOL
+    # backward given the oracle's ids (same inputs on both sides)
+    gw = torch.randn(T, K, generator=g)
+    if not spec.fixed_router:
+        w_ref.backward(gw)
+        dl = ops.router_select_bwd(logits.to(DEV), ids_ref.to(DEV), gw.to(DEV), None, spec.score_func,
+                                   spec.route_norm, spec.route_scale, mode)
+        assert rel_max(dl, lr.grad) < 2e-5
+    # dense score gradient path (aux-loss hook)
+    lr2 = logits.clone().requires_grad_()
+    gs = torch.randn(T, E, generator=g)
+    R.score(lr2, spec.score_func).backward(gs)
+    dl2 = ops.router_select_bwd(logits.to(DEV), ids_ref.to(DEV), None, gs.to(DEV), spec.score_func,
+                                spec.route_norm, spec.route_scale, mode)
+    assert rel_max(dl2, lr2.grad) < 2e-5
+
+
+def test_router_select_exact_ties_go_to_lower_index(ops):
+    logits = torch.zeros(5, 16)
+    logits[1, 3] = logits[1, 9] = 1.0
+    for fn in ("softmax", "sigmoid"):
+        w, ids, _ = ops.router_select_fwd(logits.to(DEV), None, 4, fn, False, 1.0)
+        assert ids[0].tolist() == [0, 1, 2, 3]
+        assert ids[1].tolist() == [3, 9, 0, 1]
+    # grouped known answer: tests/unit_tests/cpu/models/test_models_common.py:157-165
+    s = torch.tensor([[0.80, 0.70, 0.00, 0.00, 0.90, 0.20, 0.00, 0.00]])
+    lg = torch.log(s.clamp_min(1e-6) / (1 - s).clamp_min(1e-6))  # sigmoid^-1
+    _, ids, _ = ops.router_select_fwd(lg.to(DEV), None, 2, "sigmoid", False, 1.0, 2, 1)
+    assert ids.tolist() == [[0, 1]]
+
+
+# ---------------------------------------------------------------- permutation plan
+@pytest.mark.parametrize("T,K,E,align,local", [
+    (3, 2, 3, 1, None), (6, 2, 4, 4, None), (700, 8, 128, 1, None), (700, 8, 128, 128, None),
+    (5000, 8, 256, 1, (0, 32)), (5000, 6, 64, 16, (8, 24)), (0, 2, 4, 1, None), (1, 1, 1, 1, None),
+    (8192, 8, 128, 1, None),
+])
+def test_permute_plan_is_the_stable_argsort(ops, T, K, E, align, local):
+    print(f"plan T={T} K={K} E={E} align={align} local={local}", flush=True)
+    g = torch.Generator().manual_seed(11)
+    ids = torch.randint(0, E, (T, K), generator=g)  # duplicates inside a token allowed
+    lo, hi = (0, E) if local is None else local
+    plan = ops.permute_plan(ids.to(DEV), E, lo, hi, align)
+    counts = torch.bincount(ids.reshape(-1), minlength=E)
+    assert torch.equal(plan.counts_E.cpu().long(), counts)
+    perm = torch.argsort(ids.reshape(-1), stable=True)
+    start = int(counts[:lo].sum()); stop = int(counts[:hi].sum())
+    local_perm = perm[start:stop]
+    lc = counts[lo:hi]
+    padded = lc + (-lc % align)
+    seg_off = torch.cat([torch.zeros(1, dtype=torch.long), padded.cumsum(0)])
+    assert torch.equal(plan.seg_offsets.cpu().long(), seg_off)
+    assert torch.equal(plan.seg_counts.cpu().long(), lc)
+    total = int(seg_off[-1])
+    # expected slot_of_row: each segment's slots then -1 padding
+    exp = torch.full((plan.row_capacity,), -1, dtype=torch.long)
+    pos = 0
+    for j in range(hi - lo):
+        c = int(lc[j]); o = int(seg_off[j])
+        exp[o:o + c] = local_perm[pos:pos + c]; pos += c
+    assert torch.equal(plan.slot_of_row.cpu().long(), exp)
+    row_of_slot = plan.row_of_slot.cpu().long()
+    exp_r = torch.full((T * K,), -1, dtype=torch.long)
+    valid = exp >= 0
+    exp_r[exp[valid]] = torch.nonzero(valid).squeeze(-1)
+    assert torch.equal(row_of_slot, exp_r)
+    # tile list covers exactly the real rows
+    nt = int(plan.num_tiles.item()); tm = plan.tile_m
+    te, tr = plan.tile_expert.cpu()[:nt].long(), plan.tile_row0.cpu()[:nt].long()
+    exp_tiles = [(j, int(seg_off[j]) + i * tm) for j in range(hi - lo) for i in range((int(lc[j]) + tm - 1) // tm)]
+    assert list(zip(te.tolist(), tr.tolist())) == exp_tiles
+    assert total <= plan.row_capacity
+
+
+def test_permute_rows_known_answer_and_duplicate_backward(ops):
+    # tests/unit_tests/cpu/kernel/test_kernel_contracts.py:114-127
+    x = torch.arange(12, dtype=torch.float32).reshape(3, 4)
+    experts = torch.tensor([[2, 0], [0, 0], [2, 1]])
+    plan = ops.permute_plan(experts.to(DEV), 3)
+    rows = ops.permute_rows_fwd(x.to(DEV), plan)
+    assert torch.equal(rows.cpu(), x[[0, 1, 1, 2, 0, 2]])
+    wts = torch.arange(1, 25, dtype=torch.float32).reshape(6, 4)
+    dx = ops.permute_rows_bwd(wts.to(DEV), plan)
+    want = torch.stack([wts[0] + wts[4], wts[1] + wts[2], wts[3] + wts[5]])
+    assert torch.equal(dx.cpu(), want)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T,K,E,D,align,local", [(300, 4, 16, 96, 1, None), (300, 4, 16, 100, 8, None),
+                                                 (513, 8, 32, 256, 1, (4, 12)), (0, 2, 4, 8, 1, None)])
+def test_permute_rows_fwd_bwd_match_oracle(ops, dtype, T, K, E, D, align, local):
+    print(f"rows {dtype} T={T} K={K} E={E} D={D} align={align} local={local}", flush=True)
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(T, D, generator=g).to(dtype)
+    sc = torch.rand(T, K, generator=g)
+    # distinct experts per token, like a real top-k
+    ids = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(T)]) if T else torch.empty(0, K, dtype=torch.long)
+    lo, hi = (0, E) if local is None else local
+    plan = ops.permute_plan(ids.to(DEV), E, lo, hi, align)
+    rows = ops.permute_rows_fwd(x.to(DEV), plan)
+    total = int(plan.total_rows.item())
+    xr = x.clone().float().requires_grad_()
+    rows_ref, tok, _, _ = R.local_reorder(xr, sc, ids)
+    counts = torch.bincount(ids.reshape(-1), minlength=E)
+    start, stop = int(counts[:lo].sum()), int(counts[:hi].sum())
+    rows_ref = rows_ref[start:stop]
+    _, padded_ref, pidx, _ = R.permute_and_pad(rows_ref, counts[lo:hi], align)
+    assert total == padded_ref.shape[0]
+    assert torch.equal(rows.cpu()[:total].float(), padded_ref.detach().to(dtype).float())
+    grows = torch.randn(total, D, generator=g).to(dtype)
+    padded_ref.backward(grows.float())
+    buf = torch.zeros(plan.row_capacity, D, dtype=dtype)
+    buf[:total] = grows
+    dx = ops.permute_rows_bwd(buf.to(DEV), plan)
+    tol = FP32_TOL if dtype == torch.float32 else 1e-2
+    if T:
+        assert rel_max(dx, xr.grad) < tol
+
+
+# ---------------------------------------------------------------- combine
+def test_combine_literals(ops):
+    # tests/unit_tests/cpu/models/test_qwen_operator_contracts.py:54-68
+    tokens = torch.tensor([[1.0, 3.0], [5.0, 7.0], [11.0, 13.0]])
+    experts = torch.tensor([[2, 0], [1, 2], [0, 1]])
+    scores = torch.tensor([[0.1, 0.9], [0.2, 0.8], [0.7, 0.3]])
+    plan = ops.permute_plan(experts.to(DEV), 3)
+    rows = ops.permute_rows_fwd(tokens.to(DEV), plan)
+    gains = (experts.reshape(-1)[plan.slot_of_row.cpu().long()] + 1).unsqueeze(1).float()
+    out = ops.combine_fwd(rows * gains.to(DEV), scores.to(DEV), plan, round_terms=False)
+    want = tokens * (scores * (experts + 1)).sum(1, keepdim=True)
+    torch.testing.assert_close(out.cpu(), want)
+    dy, dw = ops.combine_bwd(torch.ones(3, 2, device=DEV), rows * gains.to(DEV), scores.to(DEV), plan)
+    # d out.sum / d score[t,k] = sum_d tokens[t,d] * (expert+1)
+    torch.testing.assert_close(dw.cpu(), tokens.sum(1, keepdim=True) * (experts + 1))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("top_k", [2, 8])
+@pytest.mark.parametrize("tokens", [0, 64, 1000])
+@pytest.mark.parametrize("fp32acc", [False, True])
+def test_combine_matches_oracle(ops, dtype, top_k, tokens, fp32acc):
+    # mirrors tests/integration_tests/routed_combine_equivalence.py:22-81
+    print(f"combine {dtype} k={top_k} T={tokens} fp32acc={fp32acc}", flush=True)
+    torch.manual_seed(91)
+    hidden = 160
+    ids = torch.randint(0, 16, (tokens, top_k))
+    values = (torch.randn(tokens * top_k, hidden) * 0.1).to(dtype)
+    scores = torch.rand(tokens, top_k)
+    probe = torch.randn(tokens, hidden).to(dtype)
+    order = ids.flatten().argsort(stable=True)
+    vr, sr = values.clone().requires_grad_(), scores.clone().requires_grad_()
+    ref = R.combine(vr, order // top_k, sr.flatten()[order], values.new_empty(tokens, hidden), fp32acc)
+    plan = ops.permute_plan(ids.to(DEV), 16)
+    got = ops.combine_fwd(values.to(DEV), scores.to(DEV), plan, round_terms=not fp32acc)
+    if tokens == 0:
+        assert got.shape == (0, hidden)
+        return
+    tol = 2e-3 if dtype == torch.bfloat16 else 2e-6
+    torch.testing.assert_close(got.cpu().float(), ref.detach().float(), atol=tol, rtol=0)
+    ref.backward(probe)
+    dy, dw = ops.combine_bwd(probe.to(DEV), values.to(DEV), scores.to(DEV), plan)
+    torch.testing.assert_close(dy.cpu().float(), vr.grad.float(), atol=tol, rtol=0)
+    torch.testing.assert_close(dw.cpu(), sr.grad, atol=2e-3 if dtype == torch.bfloat16 else 2e-5, rtol=1e-5)
+
+
+# ---------------------------------------------------------------- grouped experts
+def _experts_case(ops, dtype, counts, D, Fd, std=0.1, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    El = len(counts)
+    Rn = sum(counts)
+    x = torch.randn(Rn, D, generator=g).to(dtype)
+    w1 = (torch.randn(El, Fd, D, generator=g) * std).to(dtype)
+    w3 = (torch.randn(El, Fd, D, generator=g) * std).to(dtype)
+    w2 = (torch.randn(El, D, Fd, generator=g) * std).to(dtype)
+    gy = torch.randn(Rn, D, generator=g).to(dtype)
+    ref_in = [t.clone().requires_grad_() for t in (x, w1, w3, w2)]
+    ref = R.grouped_experts(ref_in[0], torch.tensor(counts), *ref_in[1:])
+    plan = ops.segments_from_counts(torch.tensor(counts, dtype=torch.int32, device=DEV), Rn)
+    dx_, dw1_, dw3_, dw2_ = (t.to(DEV) for t in (x, w1, w3, w2))
+    y, gate, up, h = ops.grouped_swiglu_fwd(dx_, dw1_, dw3_, dw2_, plan)
+    tol = FP32_TOL if dtype == torch.float32 else BF16_TOL
+    metric = rel_max if dtype == torch.float32 else rel_l2
+    if Rn:
+        assert metric(y, ref) < tol, f"forward {metric(y, ref)}"
+        ref.backward(gy)
+    else:
+        ref.sum().backward()
+    drows, dw1, dw3, dw2 = ops.grouped_swiglu_bwd(gy.to(DEV), dx_, dw1_, dw3_, dw2_, gate, up, h, plan)
+    for name, got, want in (("drows", drows, ref_in[0].grad), ("dw1", dw1, ref_in[1].grad),
+                            ("dw3", dw3, ref_in[2].grad), ("dw2", dw2, ref_in[3].grad)):
+        if want.abs().max() == 0:
+            assert got.abs().max() == 0, name
+        else:
+            assert metric(got, want) < tol, f"{name} {metric(got, want)}"
+
+
+@pytest.mark.parametrize("counts", [(5, 6, 4, 7), (2, 0, 3), (0, 5, 0), (0, 0, 0), (130, 1, 64, 300)])
+def test_grouped_experts_fp32(ops, counts):
+    print(f"experts fp32 {counts}", flush=True)
+    _experts_case(ops, torch.float32, counts, 16 if len(counts) == 4 else 4, 32 if len(counts) == 4 else 8)
+
+
+@pytest.mark.parametrize("counts,D,Fd", [((5, 6, 4, 7), 16, 32), ((100, 0, 29), 72, 40)])
+def test_grouped_experts_bf16_generic_shapes(ops, counts, D, Fd):
+    print(f"experts bf16 generic {counts} D={D} F={Fd}", flush=True)
+    _experts_case(ops, torch.bfloat16, counts, D, Fd)
+
+
+@pytest.mark.parametrize("counts,D,Fd", [
+    ((128, 128), 64, 64), ((5, 6, 4, 7), 128, 64), ((200, 0, 129, 1, 300), 256, 192),
+    ((0, 0, 0), 64, 128), ((513, 77), 512, 320), ((1000,), 256, 768),
+])
+def test_grouped_experts_bf16_mfma(ops, counts, D, Fd):
+    print(f"experts bf16 mfma {counts} D={D} F={Fd}", flush=True)
+    _experts_case(ops, torch.bfloat16, counts, D, Fd, std=0.05)

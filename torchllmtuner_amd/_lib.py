@@ -1,0 +1,83 @@
+"""ctypes binding of ``libmi355moe.so`` (the C ABI declared in include/mi355_moe.h).
+
+The library is the only implementation of the MoE hot path: if it is missing or
+lacks a symbol the import of the ops fails loudly -- there is no eager PyTorch or
+CPU fallback behind it.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmi355moe.so")
+CSRC_DIR = os.path.join(_HERE, "csrc")
+
+P = c_void_p
+I = c_int
+L = c_int64
+F = c_float
+
+# name -> (restype, argtypes); mirrors include/mi355_moe.h declaration by declaration
+SIGNATURES = {
+    "mi355_moe_abi_version": (I, []),
+    "mi355_moe_last_error": (c_char_p, []),
+    "mi355_router_gate_fwd": (I, [P, I, P, I, P, P, L, L, L, P]),
+    "mi355_router_gate_bwd_workspace_bytes": (L, [L, L, L]),
+    "mi355_router_gate_bwd": (I, [P, P, I, P, I, P, P, P, L, L, L, P]),
+    "mi355_router_select_fwd": (I, [P, P, P, P, P, L, L, L, I, I, F, I, I, I, P]),
+    "mi355_router_select_bwd": (I, [P, P, P, P, P, L, L, L, I, I, F, I, P]),
+    "mi355_permute_plan_workspace_bytes": (L, [L, L, L]),
+    "mi355_permute_plan": (I, [P, L, L, L, L, L, L, L, P, P, P, P, P, L, P, P, P, L, P, P]),
+    "mi355_segments_from_counts": (I, [P, L, L, L, P, P, P, P, P, L, P]),
+    "mi355_permute_rows_fwd": (I, [P, I, P, P, P, L, L, L, L, P]),
+    "mi355_permute_rows_bwd": (I, [P, I, P, P, L, L, L, P]),
+    "mi355_combine_fwd": (I, [P, I, P, P, P, L, L, L, I, P]),
+    "mi355_combine_bwd": (I, [P, P, I, P, P, P, P, P, P, L, L, L, L, P]),
+    "mi355_grouped_tile_m": (L, [I]),
+    "mi355_grouped_swiglu_fwd": (I, [P, P, P, P, I, P, P, P, P, P, L, P, P, P, P, L, L, L, L, P]),
+    "mi355_grouped_swiglu_bwd": (
+        I,
+        [P, P, P, P, P, P, P, P, I, P, P, P, P, P, L, P, P, P, P, P, P, L, L, L, L, P],
+    ),
+}
+
+_lib = None
+
+
+class MI355LibraryError(RuntimeError):
+    """The HIP library is missing, stale or failed a call."""
+
+
+def load():
+    """Load the shared library once and attach the prototypes."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise MI355LibraryError(
+            f"{LIB_PATH} is not built. Run `make -C {CSRC_DIR}` (or "
+            "`python -c 'import __graft_entry__ as g; g.build()'`); the MoE block has no "
+            "fallback implementation."
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (restype, argtypes) in SIGNATURES.items():
+        try:
+            fn = getattr(lib, name)
+        except AttributeError as exc:
+            raise MI355LibraryError(f"{LIB_PATH} does not export {name}; rebuild it") from exc
+        fn.restype = restype
+        fn.argtypes = argtypes
+    if lib.mi355_moe_abi_version() != 1:
+        raise MI355LibraryError("libmi355moe.so ABI version mismatch; rebuild it")
+    _lib = lib
+    return lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = load().mi355_moe_last_error().decode(errors="replace")
+        err = ValueError if rc == -1 else MI355LibraryError
+        raise err(f"{what} failed ({rc}): {msg}")

@@ -1,0 +1,220 @@
+// Weighted unpermute-combine and its backward (which also yields the router's
+// score gradient).  Both are bandwidth kernels: one wavefront per token, 16-byte
+// lanes along D, the K row indices and weights held in lanes 0..K-1 and broadcast
+// by shuffles.  No atomics: every output element has exactly one writer, so the
+// result is deterministic.
+#include "common.h"
+
+namespace mi355 {
+namespace {
+
+template <typename T>
+struct Vec {
+  static constexpr int N = 16 / sizeof(T);
+  __device__ static void unpack(const uint4& v, float (&f)[N]);
+  __device__ static uint4 pack(const float (&f)[N]);
+};
+template <>
+__device__ inline void Vec<float>::unpack(const uint4& v, float (&f)[4]) {
+  f[0] = __uint_as_float(v.x); f[1] = __uint_as_float(v.y);
+  f[2] = __uint_as_float(v.z); f[3] = __uint_as_float(v.w);
+}
+template <>
+__device__ inline uint4 Vec<float>::pack(const float (&f)[4]) {
+  return make_uint4(__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]),
+                    __float_as_uint(f[3]));
+}
+template <>
+__device__ inline void Vec<uint16_t>::unpack(const uint4& v, float (&f)[8]) {
+  f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
+  f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
+  f[4] = __uint_as_float(v.z << 16); f[5] = __uint_as_float(v.z & 0xffff0000u);
+  f[6] = __uint_as_float(v.w << 16); f[7] = __uint_as_float(v.w & 0xffff0000u);
+}
+template <>
+__device__ inline uint4 Vec<uint16_t>::pack(const float (&f)[8]) {
+  return make_uint4(f32_to_bf16(f[0]) | (uint32_t)f32_to_bf16(f[1]) << 16,
+                    f32_to_bf16(f[2]) | (uint32_t)f32_to_bf16(f[3]) << 16,
+                    f32_to_bf16(f[4]) | (uint32_t)f32_to_bf16(f[5]) << 16,
+                    f32_to_bf16(f[6]) | (uint32_t)f32_to_bf16(f[7]) << 16);
+}
+
+template <typename T>
+__device__ __forceinline__ float round_to(float v);
+template <>
+__device__ __forceinline__ float round_to<float>(float v) { return v; }
+template <>
+__device__ __forceinline__ float round_to<uint16_t>(float v) { return round_bf16(v); }
+
+template <typename T>
+__global__ __launch_bounds__(256) void combine_fwd_kernel(
+    const T* __restrict__ y, const float* __restrict__ weights,
+    const int32_t* __restrict__ row_of_slot, T* __restrict__ out, int T_, int D, int K,
+    int round_terms) {
+  const int lane = threadIdx.x & 63;
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= T_) return;
+  const int64_t s0 = static_cast<int64_t>(t) * K;
+  const int row = lane < K ? row_of_slot[s0 + lane] : -1;
+  const float w = lane < K ? weights[s0 + lane] : 0.0f;
+  // ascending-row visiting order (index_add's order): position of each valid slot
+  int pos = 0;
+  for (int j = 0; j < K; ++j) {
+    const int rj = __shfl(row, j, kWave);
+    pos += (rj >= 0 && (rj < row || (rj == row && j < lane))) ? 1 : 0;
+  }
+  const int nvalid = __popcll(__ballot(row >= 0));
+  int o_row = -1;
+  float o_w = 0.0f;  // lane p holds the p-th visited slot
+  for (int p = 0; p < nvalid; ++p) {
+    const unsigned long long m = __ballot(row >= 0 && pos == p);
+    const int src = __ffsll(static_cast<long long>(m)) - 1;
+    const int r = __shfl(row, src, kWave);
+    const float ww = __shfl(w, src, kWave);
+    if (lane == p) { o_row = r; o_w = ww; }
+  }
+
+  constexpr int V = Vec<T>::N;
+  T* dst = out + static_cast<int64_t>(t) * D;
+  if (D % V == 0) {
+    const int nv = D / V;
+    for (int i = lane; i < nv; i += kWave) {
+      float a[V];
+#pragma unroll
+      for (int q = 0; q < V; ++q) a[q] = 0.0f;
+      for (int p = 0; p < nvalid; ++p) {
+        const int r = __shfl(o_row, p, kWave);
+        const float ww = __shfl(o_w, p, kWave);
+        float f[V];
+        Vec<T>::unpack(reinterpret_cast<const uint4*>(y + static_cast<int64_t>(r) * D)[i], f);
+#pragma unroll
+        for (int q = 0; q < V; ++q) {
+          const float term = f[q] * ww;
+          a[q] += round_terms ? round_to<T>(term) : term;
+        }
+      }
+      reinterpret_cast<uint4*>(dst)[i] = Vec<T>::pack(a);
+    }
+  } else {
+    for (int i = lane; i < D; i += kWave) {
+      float a = 0.0f;
+      for (int p = 0; p < nvalid; ++p) {
+        const int r = __shfl(o_row, p, kWave);
+        const float ww = __shfl(o_w, p, kWave);
+        const float term = load_as_f32(y + static_cast<int64_t>(r) * D + i) * ww;
+        a += round_terms ? round_to<T>(term) : term;
+      }
+      store_from_f32(dst + i, a);
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void combine_bwd_kernel(
+    const T* __restrict__ dout, const T* __restrict__ y, const float* __restrict__ weights,
+    const int32_t* __restrict__ row_of_slot, const int32_t* __restrict__ slot_of_row,
+    const int32_t* __restrict__ total_rows, T* __restrict__ dy, float* __restrict__ dweights,
+    int T_, int D, int K, int token_blocks, int row_capacity) {
+  const int lane = threadIdx.x & 63;
+  constexpr int V = Vec<T>::N;
+  if (static_cast<int>(blockIdx.x) >= token_blocks) {
+    // padding rows of dy get zeros
+    const int r = (blockIdx.x - token_blocks) * 4 + (threadIdx.x >> 6);
+    if (r >= row_capacity || r >= *total_rows || slot_of_row[r] >= 0) return;
+    T* dst = dy + static_cast<int64_t>(r) * D;
+    for (int i = lane; i < D; i += kWave) dst[i] = T(0);
+    return;
+  }
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= T_) return;
+  const int64_t s0 = static_cast<int64_t>(t) * K;
+  const int row = lane < K ? row_of_slot[s0 + lane] : -1;
+  const float w = lane < K ? weights[s0 + lane] : 0.0f;
+  const T* g = dout + static_cast<int64_t>(t) * D;
+  float my_dot = 0.0f;  // lane k keeps slot k's dot product
+  for (int k = 0; k < K; ++k) {
+    const int r = __shfl(row, k, kWave);
+    const float ww = __shfl(w, k, kWave);
+    if (r < 0) continue;
+    const T* yr = y + static_cast<int64_t>(r) * D;
+    T* dr = dy + static_cast<int64_t>(r) * D;
+    float dot = 0.0f;
+    if (D % V == 0) {
+      const int nv = D / V;
+      for (int i = lane; i < nv; i += kWave) {
+        float gf[V], yf[V], o[V];
+        Vec<T>::unpack(reinterpret_cast<const uint4*>(g)[i], gf);
+        Vec<T>::unpack(reinterpret_cast<const uint4*>(yr)[i], yf);
+#pragma unroll
+        for (int q = 0; q < V; ++q) {
+          dot += yf[q] * gf[q];
+          o[q] = gf[q] * ww;
+        }
+        reinterpret_cast<uint4*>(dr)[i] = Vec<T>::pack(o);
+      }
+    } else {
+      for (int i = lane; i < D; i += kWave) {
+        const float gf = load_as_f32(g + i);
+        dot += load_as_f32(yr + i) * gf;
+        store_from_f32(dr + i, gf * ww);
+      }
+    }
+    dot = wave_sum(dot);
+    if (lane == k) my_dot = dot;
+  }
+  if (lane < K && dweights) dweights[s0 + lane] = my_dot;
+}
+
+}  // namespace
+}  // namespace mi355
+
+using namespace mi355;
+
+extern "C" int mi355_combine_fwd(const void* y, int dtype, const float* weights,
+                                 const int32_t* row_of_slot, void* out, int64_t T, int64_t D,
+                                 int64_t K, int round_terms, void* stream) {
+  MI355_REQUIRE(T >= 0 && D >= 1 && K >= 1 && K <= 64 && T < (1ll << 31) && D < (1ll << 31),
+                "combine_fwd: bad shape (K must be <= 64)");
+  if (T == 0) return MI355_OK;
+  MI355_REQUIRE(weights && row_of_slot && out, "combine_fwd: null pointer");
+  const dim3 grid((unsigned)((T + 3) / 4));
+  if (dtype == MI355_F32)
+    hipLaunchKernelGGL(combine_fwd_kernel<float>, grid, dim3(256), 0, as_stream(stream),
+                       static_cast<const float*>(y), weights, row_of_slot, static_cast<float*>(out),
+                       (int)T, (int)D, (int)K, round_terms);
+  else if (dtype == MI355_BF16)
+    hipLaunchKernelGGL(combine_fwd_kernel<uint16_t>, grid, dim3(256), 0, as_stream(stream),
+                       static_cast<const uint16_t*>(y), weights, row_of_slot,
+                       static_cast<uint16_t*>(out), (int)T, (int)D, (int)K, round_terms);
+  else
+    return fail(MI355_EINVAL, "combine_fwd: unknown dtype %d", dtype);
+  return check_launch("combine_fwd");
+}
+
+extern "C" int mi355_combine_bwd(const void* dout, const void* y, int dtype, const float* weights,
+                                 const int32_t* row_of_slot, const int32_t* slot_of_row,
+                                 const int32_t* total_rows, void* dy, float* dweights, int64_t T,
+                                 int64_t D, int64_t K, int64_t row_capacity, void* stream) {
+  MI355_REQUIRE(T >= 0 && D >= 1 && K >= 1 && K <= 64 && T < (1ll << 31) && D < (1ll << 31) &&
+                    row_capacity >= 0 && row_capacity < (1ll << 31),
+                "combine_bwd: bad shape (K must be <= 64)");
+  const int token_blocks = (int)((T + 3) / 4);
+  const int pad_blocks = slot_of_row ? (int)((row_capacity + 3) / 4) : 0;
+  if (token_blocks + pad_blocks == 0) return MI355_OK;
+  MI355_REQUIRE(T == 0 || (dout && weights && row_of_slot && dy), "combine_bwd: null pointer");
+  MI355_REQUIRE(!slot_of_row || total_rows, "combine_bwd: total_rows required with slot_of_row");
+  const dim3 grid((unsigned)(token_blocks + pad_blocks));
+  if (dtype == MI355_F32)
+    hipLaunchKernelGGL(combine_bwd_kernel<float>, grid, dim3(256), 0, as_stream(stream),
+                       static_cast<const float*>(dout), static_cast<const float*>(y), weights,
+                       row_of_slot, slot_of_row, total_rows, static_cast<float*>(dy), dweights,
+                       (int)T, (int)D, (int)K, token_blocks, (int)row_capacity);
+  else if (dtype == MI355_BF16)
+    hipLaunchKernelGGL(combine_bwd_kernel<uint16_t>, grid, dim3(256), 0, as_stream(stream),
+                       static_cast<const uint16_t*>(dout), static_cast<const uint16_t*>(y), weights,
+                       row_of_slot, slot_of_row, total_rows, static_cast<uint16_t*>(dy), dweights,
+                       (int)T, (int)D, (int)K, token_blocks, (int)row_capacity);
+  else
+    return fail(MI355_EINVAL, "combine_bwd: unknown dtype %d", dtype);
+  return check_launch("combine_bwd");
+}

@@ -1,0 +1,191 @@
+// Generic strided GEMM on the fp32 matrix cores (see gemm_generic.h).
+//
+// Workgroup = 256 lanes = 4 waves, output tile 64x64, each wave owns one 32x32
+// quadrant as a single v_mfma_f32_32x32x2_f32 accumulator (16 VGPRs).  K is
+// consumed in slabs of 16 staged through LDS as As[k][m] / Bs[k][n], so the
+// per-lane operand of the MFMA (one A(m,k), one B(k,n)) is a conflict-free
+// ds_read_b32 whatever the global layout was.  Global loads pick the lane mapping
+// that walks the operand's contiguous axis.
+#include "gemm_generic.h"
+
+namespace mi355 {
+
+namespace {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int TM = 64, TN = 64, TK = 16, PITCH = 65;
+
+template <typename TA, typename TB, typename TC>
+__global__ __launch_bounds__(256) void ggemm_kernel(GemmArgs g) {
+  __shared__ float As[TK][PITCH];
+  __shared__ float Bs[TK][PITCH];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
+
+  const TA* A = static_cast<const TA*>(g.A);
+  const TB* B = static_cast<const TB*>(g.B);
+  TC* C = static_cast<TC*>(g.C);
+
+  int m0, n0 = blockIdx.y * TN;
+  int m_valid;          // rows of this tile that exist
+  int64_t row_base = 0; // ROWSEG: first global row of the tile
+  int k_begin = 0, k_end = g.K;
+  float* Cpartial = nullptr;
+
+  if (g.mode == GEMM_ROWSEG) {
+    const int subs = g.tile_m / TM;
+    const int tile = blockIdx.x / subs, sub = blockIdx.x % subs;
+    if (tile >= *g.num_tiles) return;
+    const int e = g.tile_expert[tile];
+    const int r0 = g.tile_row0[tile] + sub * TM;
+    const int seg_end = g.seg_offsets[e] + g.seg_counts[e];
+    m_valid = min(TM, seg_end - r0);
+    if (m_valid <= 0) return;
+    row_base = r0;
+    m0 = 0;
+    B += static_cast<int64_t>(e) * g.b_es;
+  } else if (g.mode == GEMM_KSEG) {
+    const int e = blockIdx.z;
+    m0 = blockIdx.x * TM;
+    m_valid = min(TM, g.M - m0);
+    k_begin = g.seg_offsets[e];
+    k_end = k_begin + g.seg_counts[e];
+    C += static_cast<int64_t>(e) * g.c_es;
+  } else {
+    m0 = blockIdx.x * TM;
+    m_valid = min(TM, g.M - m0);
+    if (g.ksplit > 1) {
+      const int chunk = ((g.K + g.ksplit - 1) / g.ksplit + TK - 1) / TK * TK;
+      k_begin = blockIdx.z * chunk;
+      k_end = min(g.K, k_begin + chunk);
+      Cpartial = reinterpret_cast<float*>(g.C) + static_cast<int64_t>(blockIdx.z) * g.M * g.ldc;
+    }
+  }
+  const int n_valid = min(TN, g.N - n0);
+  const int64_t a_row0 = row_base + m0;
+
+  // lane mappings for the global->LDS copy: walk the contiguous axis with lanes
+  const bool a_kc = (g.a_cs == 1);
+  const bool b_nc = (g.b_cs == 1);
+  int am[4], ak[4], bk[4], bn[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int i = tid + j * 256;
+    if (a_kc) { ak[j] = i % TK; am[j] = i / TK; } else { am[j] = i % TM; ak[j] = i / TM; }
+    if (b_nc) { bn[j] = i % TN; bk[j] = i / TN; } else { bk[j] = i % TK; bn[j] = i / TK; }
+  }
+
+  float ra[4], rb[4];
+  auto load_slab = [&](int k0) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int k = k0 + ak[j];
+      ra[j] = (am[j] < m_valid && k < k_end)
+                  ? load_as_f32(A + (a_row0 + am[j]) * g.a_rs + static_cast<int64_t>(k) * g.a_cs)
+                  : 0.0f;
+      const int kb = k0 + bk[j];
+      rb[j] = (bn[j] < n_valid && kb < k_end)
+                  ? load_as_f32(B + static_cast<int64_t>(kb) * g.b_rs + static_cast<int64_t>(n0 + bn[j]) * g.b_cs)
+                  : 0.0f;
+    }
+  };
+
+  f32x16 acc;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+
+  if (k_begin < k_end) load_slab(k_begin);
+  for (int k0 = k_begin; k0 < k_end; k0 += TK) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      As[ak[j]][am[j]] = ra[j];
+      Bs[bk[j]][bn[j]] = rb[j];
+    }
+    __syncthreads();
+    if (k0 + TK < k_end) load_slab(k0 + TK);
+#pragma unroll
+    for (int kk = 0; kk < TK; kk += 2) {
+      const float a = As[kk + (lane >> 5)][wm + (lane & 31)];
+      const float b = Bs[kk + (lane >> 5)][wn + (lane & 31)];
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc, 0, 0, 0);
+    }
+    __syncthreads();
+  }
+
+  const int n = wn + (lane & 31);
+  if (n >= n_valid) return;
+  const float bias = g.bias ? g.bias[n0 + n] : 0.0f;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int m = wm + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3);
+    if (m >= m_valid) continue;
+    const int64_t off = (a_row0 + m) * g.ldc + n0 + n;
+    if (Cpartial) {
+      Cpartial[off] = acc[i];
+    } else {
+      float v = acc[i] + bias;
+      if (g.accumulate) v += load_as_f32(C + off);
+      store_from_f32(C + off, v);
+    }
+  }
+}
+
+template <typename TC>
+__global__ void splitk_reduce_kernel(const float* __restrict__ partial, TC* __restrict__ out,
+                                     int64_t MN, int ksplit) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= MN) return;
+  float s = 0.0f;
+  for (int z = 0; z < ksplit; ++z) s += partial[z * MN + i];
+  store_from_f32(out + i, s);
+}
+
+template <typename TA, typename TB>
+int launch_c(const GemmArgs& a, int c_dtype, dim3 grid, hipStream_t s) {
+  if (c_dtype == MI355_F32 || a.ksplit > 1)
+    hipLaunchKernelGGL((ggemm_kernel<TA, TB, float>), grid, dim3(256), 0, s, a);
+  else
+    hipLaunchKernelGGL((ggemm_kernel<TA, TB, uint16_t>), grid, dim3(256), 0, s, a);
+  return check_launch("ggemm");
+}
+
+}  // namespace
+
+int launch_gemm(const GemmArgs& a, int a_dtype, int b_dtype, int c_dtype, dim3 grid,
+                hipStream_t s) {
+  if (grid.x == 0 || grid.y == 0 || grid.z == 0) return MI355_OK;
+  if (a_dtype == MI355_F32 && b_dtype == MI355_F32) return launch_c<float, float>(a, c_dtype, grid, s);
+  if (a_dtype == MI355_BF16 && b_dtype == MI355_F32) return launch_c<uint16_t, float>(a, c_dtype, grid, s);
+  if (a_dtype == MI355_F32 && b_dtype == MI355_BF16) return launch_c<float, uint16_t>(a, c_dtype, grid, s);
+  if (a_dtype == MI355_BF16 && b_dtype == MI355_BF16) return launch_c<uint16_t, uint16_t>(a, c_dtype, grid, s);
+  return fail(MI355_EINVAL, "gemm: unknown dtype %d/%d", a_dtype, b_dtype);
+}
+
+dim3 gemm_grid_dense(int M, int N, int ksplit) {
+  return dim3((M + TM - 1) / TM, (N + TN - 1) / TN, ksplit > 1 ? ksplit : 1);
+}
+dim3 gemm_grid_rowseg(int64_t tile_capacity, int tile_m, int N) {
+  return dim3(static_cast<unsigned>(tile_capacity * (tile_m / TM)), (N + TN - 1) / TN, 1);
+}
+dim3 gemm_grid_kseg(int M, int N, int El) {
+  return dim3((M + TM - 1) / TM, (N + TN - 1) / TN, El);
+}
+
+int launch_splitk_reduce(const float* partial, void* out, int out_dtype, int64_t MN, int ksplit,
+                         hipStream_t s) {
+  if (MN == 0) return MI355_OK;
+  const unsigned blocks = static_cast<unsigned>((MN + 255) / 256);
+  if (out_dtype == MI355_F32)
+    hipLaunchKernelGGL(splitk_reduce_kernel<float>, dim3(blocks), dim3(256), 0, s, partial,
+                       static_cast<float*>(out), MN, ksplit);
+  else
+    hipLaunchKernelGGL(splitk_reduce_kernel<uint16_t>, dim3(blocks), dim3(256), 0, s, partial,
+                       static_cast<uint16_t*>(out), MN, ksplit);
+  return check_launch("splitk_reduce");
+}
+
+}  // namespace mi355

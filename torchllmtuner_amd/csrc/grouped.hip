@@ -1,0 +1,194 @@
+// Grouped SwiGLU experts: C entry points and the generic (any dtype, any shape)
+// path.  bf16 problems whose D and F are multiples of 64 go to the MFMA kernels of
+// grouped_bf16.hip; everything else (fp32, odd shapes) runs the strided fp32-MFMA
+// GEMM plus two small elementwise kernels.
+#include "common.h"
+#include "gemm_generic.h"
+
+namespace mi355 {
+
+constexpr int kTileM = 128;
+
+bool bf16_fast_path_ok(int64_t D, int64_t F);
+int bf16_grouped_fwd(const void* rows, const void* w1, const void* w3, const void* w2,
+                     const int32_t* seg_offsets, const int32_t* seg_counts,
+                     const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* num_tiles,
+                     int64_t tile_capacity, void* gate, void* up, void* h, void* y, int64_t D,
+                     int64_t F, hipStream_t s);
+int bf16_grouped_bwd(const void* dy, const void* rows, const void* w1, const void* w3,
+                     const void* w2, const void* gate, const void* up, const void* h,
+                     const int32_t* seg_offsets, const int32_t* seg_counts,
+                     const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* num_tiles,
+                     int64_t tile_capacity, void* dgate, void* dup, void* drows, void* dw1,
+                     void* dw3, void* dw2, int64_t El, int64_t D, int64_t F, hipStream_t s);
+
+namespace {
+
+template <typename T>
+__device__ __forceinline__ float rnd(float v);
+template <>
+__device__ __forceinline__ float rnd<float>(float v) { return v; }
+template <>
+__device__ __forceinline__ float rnd<uint16_t>(float v) { return round_bf16(v); }
+
+// h = silu(gate) * up over the first *total_rows rows, with the activation dtype's
+// rounding after the SiLU and after the product.
+template <typename T>
+__global__ void swiglu_fwd_kernel(const T* __restrict__ gate, const T* __restrict__ up,
+                                  T* __restrict__ h, const int32_t* __restrict__ total_rows, int F) {
+  const int64_t n = static_cast<int64_t>(*total_rows) * F;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const float g = load_as_f32(gate + i);
+    const float s = rnd<T>(g / (1.0f + expf(-g)));
+    store_from_f32(h + i, s * load_as_f32(up + i));
+  }
+}
+
+// in: dgate holds dh.  out: dgate = dh*up*silu'(gate), dup = dh*silu(gate).
+template <typename T>
+__global__ void swiglu_bwd_kernel(const T* __restrict__ gate, const T* __restrict__ up,
+                                  T* __restrict__ dgate, T* __restrict__ dup,
+                                  const int32_t* __restrict__ total_rows, int F) {
+  const int64_t n = static_cast<int64_t>(*total_rows) * F;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const float dh = load_as_f32(dgate + i);
+    const float g = load_as_f32(gate + i);
+    const float u = load_as_f32(up + i);
+    const float sig = 1.0f / (1.0f + expf(-g));
+    const float s = rnd<T>(g * sig);
+    const float ds = rnd<T>(dh * u);
+    store_from_f32(dup + i, dh * s);
+    store_from_f32(dgate + i, ds * (sig * (1.0f + g * (1.0f - sig))));
+  }
+}
+
+struct Seg {
+  const int32_t *seg_offsets, *seg_counts, *tile_expert, *tile_row0, *num_tiles;
+  int64_t tile_capacity;
+};
+
+// C(rows, N) = A(rows, K) . B[e]  over the tile-listed rows
+int rowseg(const Seg& sg, const void* A, int64_t lda, const void* B, int64_t b_rs, int64_t b_cs,
+           int64_t b_es, void* C, int64_t N, int64_t K, int dtype, int accumulate, hipStream_t s) {
+  GemmArgs g{};
+  g.A = A; g.B = B; g.C = C;
+  g.a_rs = lda; g.a_cs = 1; g.b_rs = b_rs; g.b_cs = b_cs; g.b_es = b_es;
+  g.ldc = N; g.M = 0; g.N = (int)N; g.K = (int)K;
+  g.mode = GEMM_ROWSEG; g.accumulate = accumulate; g.ksplit = 1; g.tile_m = kTileM;
+  g.seg_offsets = sg.seg_offsets; g.seg_counts = sg.seg_counts; g.tile_expert = sg.tile_expert;
+  g.tile_row0 = sg.tile_row0; g.num_tiles = sg.num_tiles;
+  return launch_gemm(g, dtype, dtype, dtype, gemm_grid_rowseg(sg.tile_capacity, kTileM, (int)N), s);
+}
+
+// C[e](M, N) = sum_{r in segment e} A[r][m] * B[r][n]
+int kseg(const Seg& sg, const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t El,
+         int dtype, hipStream_t s) {
+  GemmArgs g{};
+  g.A = A; g.B = B; g.C = C;
+  g.a_rs = 1; g.a_cs = M; g.b_rs = N; g.b_cs = 1; g.c_es = M * N;
+  g.ldc = N; g.M = (int)M; g.N = (int)N; g.K = 0;
+  g.mode = GEMM_KSEG; g.ksplit = 1;
+  g.seg_offsets = sg.seg_offsets; g.seg_counts = sg.seg_counts;
+  return launch_gemm(g, dtype, dtype, dtype, gemm_grid_kseg((int)M, (int)N, (int)El), s);
+}
+
+int check_common(const char* who, int dtype, int64_t El, int64_t D, int64_t F, int64_t row_capacity,
+                 int64_t tile_capacity) {
+  MI355_REQUIRE(dtype == MI355_F32 || dtype == MI355_BF16, "%s: unknown dtype %d", who, dtype);
+  MI355_REQUIRE(El >= 1 && D >= 1 && F >= 1, "%s: bad shape El=%lld D=%lld F=%lld", who, (long long)El,
+                (long long)D, (long long)F);
+  MI355_REQUIRE(D < (1ll << 24) && F < (1ll << 24) && D * F < (1ll << 31), "%s: D*F exceeds int32", who);
+  MI355_REQUIRE(row_capacity >= 0 && row_capacity < (1ll << 31) && tile_capacity >= 0 &&
+                    tile_capacity < (1ll << 24),
+                "%s: bad capacity", who);
+  return MI355_OK;
+}
+
+}  // namespace
+}  // namespace mi355
+
+using namespace mi355;
+
+extern "C" int64_t mi355_grouped_tile_m(int dtype) {
+  (void)dtype;
+  return kTileM;
+}
+
+extern "C" int mi355_grouped_swiglu_fwd(const void* rows, const void* w1, const void* w3,
+                                        const void* w2, int dtype, const int32_t* seg_offsets,
+                                        const int32_t* seg_counts, const int32_t* tile_expert,
+                                        const int32_t* tile_row0, const int32_t* num_tiles,
+                                        int64_t tile_capacity, void* gate, void* up, void* h, void* y,
+                                        int64_t El, int64_t D, int64_t F, int64_t row_capacity,
+                                        void* stream) {
+  if (int rc = check_common("grouped_swiglu_fwd", dtype, El, D, F, row_capacity, tile_capacity)) return rc;
+  if (row_capacity == 0 || tile_capacity == 0) return MI355_OK;
+  MI355_REQUIRE(rows && w1 && w3 && w2 && seg_offsets && seg_counts && tile_expert && tile_row0 &&
+                    num_tiles && gate && up && h && y,
+                "grouped_swiglu_fwd: null pointer");
+  hipStream_t s = as_stream(stream);
+  if (dtype == MI355_BF16 && bf16_fast_path_ok(D, F))
+    return bf16_grouped_fwd(rows, w1, w3, w2, seg_offsets, seg_counts, tile_expert, tile_row0,
+                            num_tiles, tile_capacity, gate, up, h, y, D, F, s);
+  const Seg sg{seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles, tile_capacity};
+  // gate/up: B(k=d, n=f) = w[e][f][d]
+  if (int rc = rowseg(sg, rows, D, w1, 1, D, F * D, gate, F, D, dtype, 0, s)) return rc;
+  if (int rc = rowseg(sg, rows, D, w3, 1, D, F * D, up, F, D, dtype, 0, s)) return rc;
+  const unsigned blocks = (unsigned)std::min<int64_t>((row_capacity * F + 255) / 256, 8192);
+  if (dtype == MI355_F32)
+    hipLaunchKernelGGL(swiglu_fwd_kernel<float>, dim3(blocks), dim3(256), 0, s, (const float*)gate,
+                       (const float*)up, (float*)h, seg_offsets + El, (int)F);
+  else
+    hipLaunchKernelGGL(swiglu_fwd_kernel<uint16_t>, dim3(blocks), dim3(256), 0, s,
+                       (const uint16_t*)gate, (const uint16_t*)up, (uint16_t*)h, seg_offsets + El, (int)F);
+  if (int rc = check_launch("swiglu_fwd")) return rc;
+  // down: B(k=f, n=d) = w2[e][d][f]
+  return rowseg(sg, h, F, w2, 1, F, D * F, y, D, F, dtype, 0, s);
+}
+
+extern "C" int mi355_grouped_swiglu_bwd(const void* dy, const void* rows, const void* w1,
+                                        const void* w3, const void* w2, const void* gate,
+                                        const void* up, const void* h, int dtype,
+                                        const int32_t* seg_offsets, const int32_t* seg_counts,
+                                        const int32_t* tile_expert, const int32_t* tile_row0,
+                                        const int32_t* num_tiles, int64_t tile_capacity, void* dgate,
+                                        void* dup, void* drows, void* dw1, void* dw3, void* dw2,
+                                        int64_t El, int64_t D, int64_t F, int64_t row_capacity,
+                                        void* stream) {
+  if (int rc = check_common("grouped_swiglu_bwd", dtype, El, D, F, row_capacity, tile_capacity)) return rc;
+  MI355_REQUIRE(seg_offsets && seg_counts && num_tiles, "grouped_swiglu_bwd: null plan pointer");
+  MI355_REQUIRE(row_capacity == 0 || (dy && rows && w1 && w3 && w2 && gate && up && h && dgate && dup &&
+                                      tile_expert && tile_row0),
+                "grouped_swiglu_bwd: null pointer");
+  hipStream_t s = as_stream(stream);
+  if (dtype == MI355_BF16 && bf16_fast_path_ok(D, F) && row_capacity > 0 && tile_capacity > 0)
+    return bf16_grouped_bwd(dy, rows, w1, w3, w2, gate, up, h, seg_offsets, seg_counts, tile_expert,
+                            tile_row0, num_tiles, tile_capacity, dgate, dup, drows, dw1, dw3, dw2, El,
+                            D, F, s);
+  const Seg sg{seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles, tile_capacity};
+  if (row_capacity > 0 && tile_capacity > 0) {
+    // dh = dy . w2[e]: B(k=d, n=f) = w2[e][d][f]   (lands in dgate, rewritten in place below)
+    if (int rc = rowseg(sg, dy, D, w2, F, 1, D * F, dgate, F, D, dtype, 0, s)) return rc;
+    const unsigned blocks = (unsigned)std::min<int64_t>((row_capacity * F + 255) / 256, 8192);
+    if (dtype == MI355_F32)
+      hipLaunchKernelGGL(swiglu_bwd_kernel<float>, dim3(blocks), dim3(256), 0, s, (const float*)gate,
+                         (const float*)up, (float*)dgate, (float*)dup, seg_offsets + El, (int)F);
+    else
+      hipLaunchKernelGGL(swiglu_bwd_kernel<uint16_t>, dim3(blocks), dim3(256), 0, s,
+                         (const uint16_t*)gate, (const uint16_t*)up, (uint16_t*)dgate, (uint16_t*)dup,
+                         seg_offsets + El, (int)F);
+    if (int rc = check_launch("swiglu_bwd")) return rc;
+    if (drows) {
+      // drows = dgate . w1[e] + dup . w3[e]: B(k=f, n=d) = w[e][f][d]
+      if (int rc = rowseg(sg, dgate, F, w1, D, 1, F * D, drows, D, F, dtype, 0, s)) return rc;
+      if (int rc = rowseg(sg, dup, F, w3, D, 1, F * D, drows, D, F, dtype, 1, s)) return rc;
+    }
+  }
+  // weight gradients also cover the no-rows case: every expert's gradient is written (zeros)
+  if (dw2) if (int rc = kseg(sg, dy, h, dw2, D, F, El, dtype, s)) return rc;
+  if (dw1) if (int rc = kseg(sg, dgate, rows, dw1, F, D, El, dtype, s)) return rc;
+  if (dw3) if (int rc = kseg(sg, dup, rows, dw3, F, D, El, dtype, s)) return rc;
+  return MI355_OK;
+}

@@ -1,0 +1,416 @@
+// Token permutation: the expert-major plan and the row movers.
+//
+// Plan = a stable counting sort of the N = T*K assignment slots by expert id.
+//   1. plan_rank    each wave walks 512 consecutive slots in 64-slot chunks; within
+//                   a chunk, slots of the same expert are ranked by a ballot loop
+//                   (one iteration per distinct expert in the chunk), running
+//                   per-wave expert counts live in LDS.  Emits the rank of every
+//                   slot inside its wave and the wave's histogram.
+//   2. plan_scan    one workgroup: per-expert exclusive scan of the wave histograms
+//                   (ascending wave = ascending slot, which is what makes the sort
+//                   stable), the padded segment offsets, and the MFMA tile list.
+//   3. plan_rows    row = segment offset + waves-before + rank-in-wave, written both
+//                   ways (row_of_slot, slot_of_row).
+// The row movers are pure bandwidth kernels: one wave per row, 16-byte lanes.
+#include "common.h"
+
+namespace mi355 {
+namespace {
+
+constexpr int kSlotsPerWave = 512;
+constexpr int kWavesPerBlock = 4;
+constexpr int kSlotsPerBlock = kSlotsPerWave * kWavesPerBlock;
+
+__global__ __launch_bounds__(256) void plan_rank_kernel(const int64_t* __restrict__ ids, int N,
+                                                        int E, int32_t* __restrict__ rank_in_wave,
+                                                        int32_t* __restrict__ wave_hist) {
+  extern __shared__ int32_t cnt[];  // [4][E]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  volatile int32_t* my = cnt + wave * E;
+  for (int e = lane; e < E; e += kWave) my[e] = 0;
+  __syncthreads();
+
+  const int gw = blockIdx.x * kWavesPerBlock + wave;
+  const int begin = gw * kSlotsPerWave;
+  const unsigned long long lt_mask = (1ull << lane) - 1ull;
+  for (int c = 0; c < kSlotsPerWave; c += kWave) {
+    const int slot = begin + c + lane;
+    const bool valid = slot < N;
+    int e = valid ? static_cast<int>(ids[slot]) : -1;
+    if (e < 0 || e >= E) e = valid ? 0 : -1;  // out-of-range ids are folded, never written OOB
+    unsigned long long todo = __ballot(valid);
+    int rank = 0;
+    while (todo) {
+      const int leader = __ffsll(static_cast<long long>(todo)) - 1;
+      const int e0 = __shfl(e, leader, kWave);
+      const unsigned long long same = __ballot(valid && e == e0);
+      const int base = my[e0];
+      if (e == e0) rank = base + __popcll(same & lt_mask);
+      __builtin_amdgcn_wave_barrier();
+      if (lane == leader) my[e0] = base + __popcll(same);
+      __builtin_amdgcn_wave_barrier();
+      todo &= ~same;
+    }
+    if (valid) rank_in_wave[slot] = rank;
+  }
+  __syncthreads();
+  for (int e = lane; e < E; e += kWave) wave_hist[static_cast<int64_t>(gw) * E + e] = my[e];
+}
+
+// One workgroup of 1024 lanes.  The per-expert scan over the wave histograms is
+// split into `parts` contiguous ranges of waves so its loads pipeline: pass 1 sums
+// each range, a short serial scan joins them, pass 2 writes the exclusive prefixes.
+__global__ __launch_bounds__(1024) void plan_scan_kernel(
+    const int32_t* __restrict__ wave_hist, int32_t* __restrict__ wave_prefix, int num_waves, int E,
+    int lo, int hi, int align, int tile_m, int32_t* __restrict__ counts_E,
+    int32_t* __restrict__ seg_offsets, int32_t* __restrict__ seg_counts,
+    int32_t* __restrict__ tile_expert, int32_t* __restrict__ tile_row0,
+    int32_t* __restrict__ num_tiles, int tile_capacity, int parts) {
+  extern __shared__ int32_t sh[];
+  const int El = hi - lo;
+  int32_t* part_sum = sh;                  // parts * E
+  int32_t* cnt_sh = part_sum + parts * E;  // E
+  int32_t* seg_off_sh = cnt_sh + E;        // El + 1
+  int32_t* tile_off_sh = seg_off_sh + El + 1;  // El + 1
+  const int tid = threadIdx.x;
+  const int per = (num_waves + parts - 1) / parts;
+
+  for (int idx = tid; idx < E * parts; idx += blockDim.x) {
+    const int e = idx % E, part = idx / E;
+    const int w0 = part * per, w1 = min(num_waves, w0 + per);
+    int sum = 0;
+    for (int w = w0; w < w1; ++w) sum += wave_hist[static_cast<int64_t>(w) * E + e];
+    part_sum[part * E + e] = sum;
+  }
+  __syncthreads();
+  for (int e = tid; e < E; e += blockDim.x) {
+    int run = 0;
+    for (int part = 0; part < parts; ++part) {
+      const int c = part_sum[part * E + e];
+      part_sum[part * E + e] = run;
+      run += c;
+    }
+    cnt_sh[e] = run;
+    counts_E[e] = run;
+    if (e >= lo && e < hi) seg_counts[e - lo] = run;
+  }
+  __syncthreads();
+  for (int idx = tid; idx < E * parts; idx += blockDim.x) {
+    const int e = idx % E, part = idx / E;
+    const int w0 = part * per, w1 = min(num_waves, w0 + per);
+    int run = part_sum[part * E + e];
+    for (int w = w0; w < w1; ++w) {
+      const int64_t i = static_cast<int64_t>(w) * E + e;
+      wave_prefix[i] = run;
+      run += wave_hist[i];
+    }
+  }
+  if (tid == 0) {
+    // El is at most a few hundred: a serial scan by one lane costs about a microsecond.
+    int off = 0, toff = 0;
+    for (int j = 0; j < El; ++j) {
+      const int c = cnt_sh[lo + j];
+      seg_off_sh[j] = off;
+      tile_off_sh[j] = toff;
+      off += c + ((align - (c % align)) % align);
+      toff += (c + tile_m - 1) / tile_m;
+    }
+    seg_off_sh[El] = off;
+    tile_off_sh[El] = toff;
+    *num_tiles = toff < tile_capacity ? toff : tile_capacity;
+  }
+  __syncthreads();
+  for (int j = tid; j <= El; j += blockDim.x) seg_offsets[j] = seg_off_sh[j];
+  for (int j = tid; j < El; j += blockDim.x) {
+    const int c = cnt_sh[lo + j];
+    const int nt = (c + tile_m - 1) / tile_m;
+    for (int i = 0; i < nt; ++i) {
+      const int idx = tile_off_sh[j] + i;
+      if (idx < tile_capacity) {
+        tile_expert[idx] = j;
+        tile_row0[idx] = seg_off_sh[j] + i * tile_m;
+      }
+    }
+  }
+}
+
+// Segment offsets and tile list for rows that are already expert-major with the
+// given per-expert row counts (the layout GroupedExperts.forward receives).
+__global__ __launch_bounds__(256) void segments_from_counts_kernel(
+    const int32_t* __restrict__ counts, int El, int tile_m, int row_capacity,
+    int32_t* __restrict__ seg_offsets, int32_t* __restrict__ seg_counts,
+    int32_t* __restrict__ tile_expert, int32_t* __restrict__ tile_row0,
+    int32_t* __restrict__ num_tiles, int tile_capacity) {
+  extern __shared__ int32_t sh[];
+  int32_t* seg_off_sh = sh;
+  int32_t* tile_off_sh = sh + El + 1;
+  int32_t* cnt_sh = sh + 2 * El + 2;
+  const int tid = threadIdx.x;
+  if (tid == 0) {
+    int off = 0, toff = 0;
+    for (int j = 0; j < El; ++j) {
+      // clamp so that no segment reaches past the rows that exist
+      const int c = min(max(counts[j], 0), row_capacity - off);
+      cnt_sh[j] = c;
+      seg_off_sh[j] = off;
+      tile_off_sh[j] = toff;
+      off += c;
+      toff += (c + tile_m - 1) / tile_m;
+    }
+    seg_off_sh[El] = off;
+    tile_off_sh[El] = toff;
+    *num_tiles = toff < tile_capacity ? toff : tile_capacity;
+  }
+  __syncthreads();
+  for (int j = tid; j <= El; j += blockDim.x) seg_offsets[j] = seg_off_sh[j];
+  for (int j = tid; j < El; j += blockDim.x) {
+    const int c = cnt_sh[j];
+    seg_counts[j] = c;
+    const int nt = (c + tile_m - 1) / tile_m;
+    for (int i = 0; i < nt; ++i) {
+      const int idx = tile_off_sh[j] + i;
+      if (idx < tile_capacity) {
+        tile_expert[idx] = j;
+        tile_row0[idx] = seg_off_sh[j] + i * tile_m;
+      }
+    }
+  }
+}
+
+__global__ void fill_i32_kernel(int32_t* p, int64_t n, int32_t v) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+__global__ __launch_bounds__(256) void plan_rows_kernel(
+    const int64_t* __restrict__ ids, const int32_t* __restrict__ rank_in_wave,
+    const int32_t* __restrict__ wave_prefix, const int32_t* __restrict__ seg_offsets, int N, int E,
+    int lo, int hi, int32_t* __restrict__ row_of_slot, int32_t* __restrict__ slot_of_row,
+    int row_capacity) {
+  const int slot = blockIdx.x * blockDim.x + threadIdx.x;
+  if (slot >= N) return;
+  int e = static_cast<int>(ids[slot]);
+  if (e < 0 || e >= E) e = 0;
+  int row = -1;
+  if (e >= lo && e < hi) {
+    const int gw = slot / kSlotsPerWave;
+    row = seg_offsets[e - lo] + wave_prefix[static_cast<int64_t>(gw) * E + e] + rank_in_wave[slot];
+    if (row >= 0 && row < row_capacity) slot_of_row[row] = slot; else row = -1;
+  }
+  row_of_slot[slot] = row;
+}
+
+// ---- row movers ---------------------------------------------------------------
+// One wave per row; VEC = 16-byte vectors when the row length allows, else scalars.
+template <typename T>
+__global__ __launch_bounds__(256) void permute_rows_fwd_kernel(
+    const T* __restrict__ x, const int32_t* __restrict__ slot_of_row,
+    const int32_t* __restrict__ total_rows, T* __restrict__ rows, int D, int K, int row_capacity) {
+  const int lane = threadIdx.x & 63;
+  const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= row_capacity || r >= *total_rows) return;
+  const int slot = slot_of_row[r];
+  T* dst = rows + static_cast<int64_t>(r) * D;
+  constexpr int V = 16 / sizeof(T);
+  if (D % V == 0) {
+    uint4* d4 = reinterpret_cast<uint4*>(dst);
+    const int nv = D / V;
+    if (slot < 0) {
+      for (int i = lane; i < nv; i += kWave) d4[i] = make_uint4(0, 0, 0, 0);
+    } else {
+      const uint4* s4 = reinterpret_cast<const uint4*>(x + static_cast<int64_t>(slot / K) * D);
+      for (int i = lane; i < nv; i += kWave) d4[i] = s4[i];
+    }
+  } else {
+    const T* src = x + static_cast<int64_t>(slot < 0 ? 0 : slot / K) * D;
+    for (int i = lane; i < D; i += kWave) dst[i] = slot < 0 ? T(0) : src[i];
+  }
+}
+
+template <typename T>
+__device__ __forceinline__ void acc_vec(float (&a)[16 / sizeof(T)], const uint4& v);
+template <>
+__device__ __forceinline__ void acc_vec<float>(float (&a)[4], const uint4& v) {
+  a[0] += __uint_as_float(v.x); a[1] += __uint_as_float(v.y);
+  a[2] += __uint_as_float(v.z); a[3] += __uint_as_float(v.w);
+}
+template <>
+__device__ __forceinline__ void acc_vec<uint16_t>(float (&a)[8], const uint4& v) {
+  a[0] += __uint_as_float(v.x << 16); a[1] += __uint_as_float(v.x & 0xffff0000u);
+  a[2] += __uint_as_float(v.y << 16); a[3] += __uint_as_float(v.y & 0xffff0000u);
+  a[4] += __uint_as_float(v.z << 16); a[5] += __uint_as_float(v.z & 0xffff0000u);
+  a[6] += __uint_as_float(v.w << 16); a[7] += __uint_as_float(v.w & 0xffff0000u);
+}
+template <typename T>
+__device__ __forceinline__ uint4 pack_vec(const float (&a)[16 / sizeof(T)]);
+template <>
+__device__ __forceinline__ uint4 pack_vec<float>(const float (&a)[4]) {
+  return make_uint4(__float_as_uint(a[0]), __float_as_uint(a[1]), __float_as_uint(a[2]),
+                    __float_as_uint(a[3]));
+}
+template <>
+__device__ __forceinline__ uint4 pack_vec<uint16_t>(const float (&a)[8]) {
+  return make_uint4(f32_to_bf16(a[0]) | (uint32_t)f32_to_bf16(a[1]) << 16,
+                    f32_to_bf16(a[2]) | (uint32_t)f32_to_bf16(a[3]) << 16,
+                    f32_to_bf16(a[4]) | (uint32_t)f32_to_bf16(a[5]) << 16,
+                    f32_to_bf16(a[6]) | (uint32_t)f32_to_bf16(a[7]) << 16);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void permute_rows_bwd_kernel(
+    const T* __restrict__ drows, const int32_t* __restrict__ row_of_slot, T* __restrict__ dx, int T_,
+    int D, int K) {
+  const int lane = threadIdx.x & 63;
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= T_) return;
+  constexpr int V = 16 / sizeof(T);
+  T* dst = dx + static_cast<int64_t>(t) * D;
+  const int my_row = lane < K ? row_of_slot[static_cast<int64_t>(t) * K + lane] : -1;  // K <= 64
+  if (D % V == 0) {
+    const int nv = D / V;
+    for (int i = lane; i < nv; i += kWave) {
+      float a[V];
+#pragma unroll
+      for (int q = 0; q < V; ++q) a[q] = 0.0f;
+      for (int k = 0; k < K; ++k) {
+        const int row = __shfl(my_row, k, kWave);
+        if (row < 0) continue;
+        acc_vec<T>(a, reinterpret_cast<const uint4*>(drows + static_cast<int64_t>(row) * D)[i]);
+      }
+      reinterpret_cast<uint4*>(dst)[i] = pack_vec<T>(a);
+    }
+  } else {
+    for (int i = lane; i < D; i += kWave) {
+      float a = 0.0f;
+      for (int k = 0; k < K; ++k) {
+        const int row = __shfl(my_row, k, kWave);
+        if (row >= 0) a += load_as_f32(drows + static_cast<int64_t>(row) * D + i);
+      }
+      store_from_f32(dst + i, a);
+    }
+  }
+}
+
+}  // namespace
+}  // namespace mi355
+
+using namespace mi355;
+
+static int64_t plan_num_waves(int64_t N) { return (N + kSlotsPerWave - 1) / kSlotsPerWave; }
+static int64_t plan_num_blocks(int64_t N) { return (N + kSlotsPerBlock - 1) / kSlotsPerBlock; }
+
+extern "C" int64_t mi355_permute_plan_workspace_bytes(int64_t T, int64_t K, int64_t E) {
+  const int64_t N = T * K;
+  // rank_in_wave[N] + wave_hist[blocks*4][E] + wave_prefix[blocks*4][E]
+  return (N + 2 * plan_num_blocks(N) * kWavesPerBlock * E + 64) * (int64_t)sizeof(int32_t);
+}
+
+extern "C" int mi355_permute_plan(const int64_t* ids, int64_t T, int64_t K, int64_t E,
+                                  int64_t lo, int64_t hi, int64_t align, int64_t tile_m,
+                                  int32_t* counts_E, int32_t* seg_offsets, int32_t* seg_counts,
+                                  int32_t* row_of_slot, int32_t* slot_of_row,
+                                  int64_t row_capacity, int32_t* tile_expert, int32_t* tile_row0,
+                                  int32_t* num_tiles, int64_t tile_capacity, void* workspace,
+                                  void* stream) {
+  const int64_t N = T * K;
+  MI355_REQUIRE(T >= 0 && K >= 1 && E >= 1 && N < (1ll << 30), "permute_plan: bad shape T=%lld K=%lld E=%lld",
+                (long long)T, (long long)K, (long long)E);
+  MI355_REQUIRE(E <= 4096, "permute_plan: E=%lld exceeds 4096", (long long)E);
+  MI355_REQUIRE(0 <= lo && lo < hi && hi <= E, "permute_plan: bad local range [%lld,%lld)", (long long)lo, (long long)hi);
+  MI355_REQUIRE(align >= 1 && tile_m >= 1, "permute_plan: align and tile_m must be positive");
+  MI355_REQUIRE(row_capacity >= 0 && row_capacity < (1ll << 31) && tile_capacity >= 0,
+                "permute_plan: bad capacity");
+  MI355_REQUIRE(counts_E && seg_offsets && seg_counts && num_tiles && workspace,
+                "permute_plan: null pointer");
+  MI355_REQUIRE(N == 0 || (ids && row_of_slot), "permute_plan: null pointer");
+  MI355_REQUIRE(row_capacity == 0 || slot_of_row, "permute_plan: null slot_of_row");
+  hipStream_t s = as_stream(stream);
+  int32_t* rank_in_wave = static_cast<int32_t*>(workspace);
+  int32_t* wave_hist = rank_in_wave + N;
+  const int nblocks = (int)plan_num_blocks(N);
+  const int nwaves = nblocks * kWavesPerBlock;
+  if (nblocks > 0) {
+    hipLaunchKernelGGL(plan_rank_kernel, dim3(nblocks), dim3(256), (size_t)kWavesPerBlock * E * 4, s,
+                       ids, (int)N, (int)E, rank_in_wave, wave_hist);
+    if (int rc = check_launch("plan_rank")) return rc;
+  }
+  if (row_capacity > 0) {
+    hipLaunchKernelGGL(fill_i32_kernel, dim3((unsigned)((row_capacity + 255) / 256)), dim3(256), 0, s,
+                       slot_of_row, row_capacity, -1);
+    if (int rc = check_launch("plan_fill")) return rc;
+  }
+  const int El = (int)(hi - lo);
+  int32_t* wave_prefix = wave_hist + (int64_t)nwaves * E;
+  int parts = (int)(1024 / E);
+  if (parts < 1) parts = 1;
+  if (parts > 16) parts = 16;
+  hipLaunchKernelGGL(plan_scan_kernel, dim3(1), dim3(1024),
+                     (size_t)((parts + 1) * E + 2 * El + 2) * 4, s, wave_hist, wave_prefix, nwaves,
+                     (int)E, (int)lo, (int)hi, (int)align, (int)tile_m, counts_E, seg_offsets,
+                     seg_counts, tile_expert, tile_row0, num_tiles, (int)tile_capacity, parts);
+  if (int rc = check_launch("plan_scan")) return rc;
+  if (N > 0) {
+    hipLaunchKernelGGL(plan_rows_kernel, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, s, ids,
+                       rank_in_wave, wave_prefix, seg_offsets, (int)N, (int)E, (int)lo, (int)hi,
+                       row_of_slot, slot_of_row, (int)row_capacity);
+    if (int rc = check_launch("plan_rows")) return rc;
+  }
+  return MI355_OK;
+}
+
+extern "C" int mi355_permute_rows_fwd(const void* x, int dtype, const int32_t* slot_of_row,
+                                      const int32_t* total_rows, void* rows, int64_t T, int64_t D,
+                                      int64_t K, int64_t row_capacity, void* stream) {
+  MI355_REQUIRE(D >= 1 && K >= 1 && T >= 0 && row_capacity >= 0 && row_capacity < (1ll << 31) &&
+                    D < (1ll << 31),
+                "permute_rows_fwd: bad shape");
+  if (row_capacity == 0) return MI355_OK;
+  MI355_REQUIRE(slot_of_row && total_rows && rows && (x || T == 0), "permute_rows_fwd: null pointer");
+  const dim3 grid((unsigned)((row_capacity + 3) / 4));
+  if (dtype == MI355_F32)
+    hipLaunchKernelGGL(permute_rows_fwd_kernel<float>, grid, dim3(256), 0, as_stream(stream),
+                       static_cast<const float*>(x), slot_of_row, total_rows,
+                       static_cast<float*>(rows), (int)D, (int)K, (int)row_capacity);
+  else if (dtype == MI355_BF16)
+    hipLaunchKernelGGL(permute_rows_fwd_kernel<uint16_t>, grid, dim3(256), 0, as_stream(stream),
+                       static_cast<const uint16_t*>(x), slot_of_row, total_rows,
+                       static_cast<uint16_t*>(rows), (int)D, (int)K, (int)row_capacity);
+  else
+    return fail(MI355_EINVAL, "permute_rows_fwd: unknown dtype %d", dtype);
+  return check_launch("permute_rows_fwd");
+}
+
+extern "C" int mi355_permute_rows_bwd(const void* drows, int dtype, const int32_t* row_of_slot,
+                                      void* dx, int64_t T, int64_t D, int64_t K, void* stream) {
+  MI355_REQUIRE(D >= 1 && K >= 1 && K <= 64 && T >= 0 && T < (1ll << 31) && D < (1ll << 31),
+                "permute_rows_bwd: bad shape (K must be <= 64)");
+  if (T == 0) return MI355_OK;
+  MI355_REQUIRE(row_of_slot && dx, "permute_rows_bwd: null pointer");
+  const dim3 grid((unsigned)((T + 3) / 4));
+  if (dtype == MI355_F32)
+    hipLaunchKernelGGL(permute_rows_bwd_kernel<float>, grid, dim3(256), 0, as_stream(stream),
+                       static_cast<const float*>(drows), row_of_slot, static_cast<float*>(dx),
+                       (int)T, (int)D, (int)K);
+  else if (dtype == MI355_BF16)
+    hipLaunchKernelGGL(permute_rows_bwd_kernel<uint16_t>, grid, dim3(256), 0, as_stream(stream),
+                       static_cast<const uint16_t*>(drows), row_of_slot,
+                       static_cast<uint16_t*>(dx), (int)T, (int)D, (int)K);
+  else
+    return fail(MI355_EINVAL, "permute_rows_bwd: unknown dtype %d", dtype);
+  return check_launch("permute_rows_bwd");
+}
+
+extern "C" int mi355_segments_from_counts(const int32_t* counts, int64_t El, int64_t tile_m,
+                                          int64_t row_capacity, int32_t* seg_offsets, int32_t* seg_counts,
+                                          int32_t* tile_expert, int32_t* tile_row0,
+                                          int32_t* num_tiles, int64_t tile_capacity, void* stream) {
+  MI355_REQUIRE(El >= 1 && El <= 8192 && tile_m >= 1 && tile_capacity >= 0 && row_capacity >= 0 &&
+                    row_capacity < (1ll << 31),
+                "segments_from_counts: bad shape El=%lld", (long long)El);
+  MI355_REQUIRE(counts && seg_offsets && seg_counts && num_tiles, "segments_from_counts: null pointer");
+  MI355_REQUIRE(tile_capacity == 0 || (tile_expert && tile_row0), "segments_from_counts: null tile list");
+  hipLaunchKernelGGL(segments_from_counts_kernel, dim3(1), dim3(256), (size_t)(3 * El + 2) * 4,
+                     as_stream(stream), counts, (int)El, (int)tile_m, (int)row_capacity, seg_offsets, seg_counts,
+                     tile_expert, tile_row0, num_tiles, (int)tile_capacity);
+  return check_launch("segments_from_counts");
+}

@@ -1,0 +1,402 @@
+// Router: fp32 gate projection and the fused score / top-k / gather / norm pass.
+//
+// Selection kernel: one 64-lane wavefront owns one token.  Lane l keeps experts
+// l, l+64, l+128, ... in registers (coalesced logit loads), the softmax max / sum
+// and every arg-max are wave-level shuffle reductions, and the K winners are
+// written by lanes 0..K-1.  No LDS, no atomics; HBM traffic is the (T,E) logits
+// once plus the (T,K) outputs.
+#include "common.h"
+#include "gemm_generic.h"
+
+namespace mi355 {
+namespace {
+
+constexpr int kMaxVPL = 8;  // experts per lane -> E <= 512
+
+__device__ __forceinline__ float softplus_f32(float x) {
+  return x > 20.0f ? x : log1pf(expf(x));  // torch's threshold=20, beta=1
+}
+
+// (value, index) arg-max across the wave; ties go to the lower index.
+__device__ __forceinline__ void wave_argmax(float& v, int& idx) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(v, o, kWave);
+    const int oi = __shfl_xor(idx, o, kWave);
+    if (ov > v || (ov == v && oi < idx)) { v = ov; idx = oi; }
+  }
+}
+
+template <int VPL>
+__device__ __forceinline__ float pick(const float (&a)[VPL], int j) {
+  float r = a[0];
+#pragma unroll
+  for (int q = 1; q < VPL; ++q) r = (j == q) ? a[q] : r;
+  return r;
+}
+
+template <int VPL>
+__device__ __forceinline__ void compute_scores(const float* __restrict__ row, int E, int lane,
+                                               int score_func, float (&s)[VPL]) {
+  float x[VPL];
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) {
+    const int e = lane + j * kWave;
+    x[j] = e < E ? row[e] : -INFINITY;
+  }
+  if (score_func == MI355_SCORE_SOFTMAX) {
+    float m = x[0];
+#pragma unroll
+    for (int j = 1; j < VPL; ++j) m = fmaxf(m, x[j]);
+    m = wave_max(m);
+    float sum = 0.0f;
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+      s[j] = (lane + j * kWave < E) ? expf(x[j] - m) : 0.0f;
+      sum += s[j];
+    }
+    sum = wave_sum(sum);
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) s[j] = s[j] / sum;
+  } else if (score_func == MI355_SCORE_SIGMOID) {
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) s[j] = 1.0f / (1.0f + expf(-x[j]));
+  } else {
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) s[j] = sqrtf(softplus_f32(x[j]));
+  }
+}
+
+template <int VPL>
+__global__ __launch_bounds__(256) void select_fwd_kernel(
+    const float* __restrict__ logits, const float* __restrict__ expert_bias,
+    float* __restrict__ weights, int64_t* __restrict__ ids, float* __restrict__ scores_out,
+    int T, int E, int K, int score_func, int route_norm, float route_scale, int num_groups,
+    int num_limited, int mode) {
+  const int lane = threadIdx.x & 63;
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= T) return;
+
+  float s[VPL];
+  compute_scores<VPL>(logits + static_cast<int64_t>(t) * E, E, lane, score_func, s);
+  if (scores_out) {
+#pragma unroll
+    for (int j = 0; j < VPL; ++j)
+      if (lane + j * kWave < E) scores_out[static_cast<int64_t>(t) * E + lane + j * kWave] = s[j];
+  }
+
+  float my_w = 0.0f;
+  int my_id = 0;
+
+  if (mode == MI355_SELECT_TOPK) {
+    float c[VPL];
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+      const int e = lane + j * kWave;
+      c[j] = e < E ? (expert_bias ? s[j] + expert_bias[e] : s[j]) : -INFINITY;
+    }
+    unsigned taken = 0;
+#pragma unroll
+    for (int j = 0; j < VPL; ++j)
+      if (lane + j * kWave >= E) taken |= 1u << j;  // never selectable
+
+    if (num_groups > 0) {
+      // group score = sum of the group's two best choice scores; keep the best
+      // num_limited groups (ties to the lower group), mask the rest to -inf.
+      const int P = E / num_groups;
+      float gscore = -INFINITY;  // lane g (< num_groups) keeps group g's score
+      for (int g = 0; g < num_groups; ++g) {
+        float top2 = 0.0f;
+        unsigned used = 0;
+        for (int r = 0; r < 2; ++r) {
+          float bv = -INFINITY;
+          int bi = 0x7fffffff;
+#pragma unroll
+          for (int j = 0; j < VPL; ++j) {
+            const int e = lane + j * kWave;
+            const bool in = e < E && e / P == g && !((used >> j) & 1u);
+            if (in && (c[j] > bv || bi == 0x7fffffff)) { bv = c[j]; bi = e; }
+          }
+          wave_argmax(bv, bi);
+          top2 += bv;
+          if ((bi & 63) == lane) used |= 1u << (bi >> 6);
+        }
+        if (lane == g) gscore = top2;
+      }
+      unsigned long long keep = 0;  // bit g set = group kept
+      float gs = gscore;
+      for (int r = 0; r < num_limited; ++r) {
+        float bv = gs;
+        int bi = lane < num_groups ? lane : 0x7fffffff;
+        if (lane >= num_groups) bv = -INFINITY;
+        // lanes already chosen drop out
+        if ((keep >> lane) & 1ull) { bv = -INFINITY; bi = 0x7fffffff; }
+        wave_argmax(bv, bi);
+        keep |= 1ull << bi;
+      }
+#pragma unroll
+      for (int j = 0; j < VPL; ++j) {
+        const int e = lane + j * kWave;
+        if (e < E && !((keep >> (e / P)) & 1ull)) c[j] = -INFINITY;
+      }
+    }
+
+    for (int k = 0; k < K; ++k) {
+      float bv = -INFINITY;
+      int bi = 0x7fffffff;
+#pragma unroll
+      for (int j = 0; j < VPL; ++j) {
+        if ((taken >> j) & 1u) continue;
+        if (bi == 0x7fffffff || c[j] > bv) { bv = c[j]; bi = lane + j * kWave; }
+      }
+      wave_argmax(bv, bi);
+      const int owner = bi & 63, slot = bi >> 6;
+      float sv = 0.0f;
+      if (lane == owner) {
+        taken |= 1u << slot;
+        sv = pick<VPL>(s, slot);
+      }
+      sv = __shfl(sv, owner, kWave);
+      if (lane == k) { my_w = sv; my_id = bi; }
+    }
+  } else {
+    // fixed: (t + k) % E ; balanced: (t*K + k) % E ; lane k owns slot k (K <= 64)
+    const int64_t base = mode == MI355_SELECT_FIXED ? static_cast<int64_t>(t) + lane
+                                                    : static_cast<int64_t>(t) * K + lane;
+    my_id = static_cast<int>(base % E);
+    // gather the unbiased score of each slot's expert from its owner lane
+    for (int k = 0; k < K; ++k) {
+      const int want = __shfl(my_id, k, kWave);
+      const float got = __shfl(pick<VPL>(s, want >> 6), want & 63, kWave);
+      if (lane == k) my_w = got;
+    }
+  }
+
+  if (mode == MI355_SELECT_FIXED) {
+    my_w = 1.0f / static_cast<float>(K);
+  } else {
+    if (route_norm) {
+      const float sum = wave_sum(lane < K ? my_w : 0.0f);
+      my_w = my_w / (sum + 1e-20f);
+    }
+    my_w = my_w * route_scale;
+  }
+  if (lane < K) {
+    weights[static_cast<int64_t>(t) * K + lane] = my_w;
+    ids[static_cast<int64_t>(t) * K + lane] = my_id;
+  }
+}
+
+template <int VPL>
+__global__ __launch_bounds__(256) void select_bwd_kernel(
+    const float* __restrict__ logits, const int64_t* __restrict__ ids,
+    const float* __restrict__ dweights, const float* __restrict__ dscores,
+    float* __restrict__ dlogits, int T, int E, int K, int score_func, int route_norm,
+    float route_scale, int mode) {
+  extern __shared__ float lds[];  // per wave: sc[E], ds[E]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int t_raw = blockIdx.x * 4 + wave;
+  const bool active = t_raw < T;
+  const int t = active ? t_raw : T - 1;  // inactive waves shadow the last token, store nothing
+  float* sc = lds + static_cast<size_t>(wave) * 2 * E;
+  float* ds = sc + E;
+
+  const float* row = logits + static_cast<int64_t>(t) * E;
+  float s[VPL];
+  compute_scores<VPL>(row, E, lane, score_func, s);
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) {
+    const int e = lane + j * kWave;
+    if (e < E) {
+      sc[e] = s[j];
+      ds[e] = dscores ? dscores[static_cast<int64_t>(t) * E + e] : 0.0f;
+    }
+  }
+  __syncthreads();
+
+  if (mode != MI355_SELECT_FIXED && dweights) {
+    // lanes 0..K-1 own one selected expert each (K <= 64)
+    int id = lane < K ? static_cast<int>(ids[static_cast<int64_t>(t) * K + lane]) : 0;
+    id = min(max(id, 0), E - 1);
+    const float sk = lane < K ? sc[id] : 0.0f;
+    const float dw = lane < K ? dweights[static_cast<int64_t>(t) * K + lane] : 0.0f;
+    float g;
+    if (route_norm) {
+      const float denom = wave_sum(sk) + 1e-20f;
+      const float dot = wave_sum(dw * sk);
+      g = route_scale * (dw / denom - dot / (denom * denom));
+    } else {
+      g = route_scale * dw;
+    }
+    // scatter-add into the dense score gradient, serially so a repeated id adds up
+    for (int k = 0; k < K; ++k) {
+      const int idk = __shfl(id, k, kWave);
+      const float gk = __shfl(g, k, kWave);
+      if (lane == 0) ds[idk] += gk;
+    }
+  }
+  __syncthreads();
+
+  float d[VPL];
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) {
+    const int e = lane + j * kWave;
+    d[j] = e < E ? ds[e] : 0.0f;
+  }
+  if (score_func == MI355_SCORE_SOFTMAX) {
+    float dot = 0.0f;
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) dot += (lane + j * kWave < E) ? s[j] * d[j] : 0.0f;
+    dot = wave_sum(dot);
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) d[j] = s[j] * (d[j] - dot);
+  } else if (score_func == MI355_SCORE_SIGMOID) {
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) d[j] = d[j] * s[j] * (1.0f - s[j]);
+  } else {
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+      const int e = lane + j * kWave;
+      const float x = e < E ? row[e] : 0.0f;
+      const float sig = 1.0f / (1.0f + expf(-x));
+      const float dsp = x > 20.0f ? 1.0f : sig;  // d softplus / dx
+      d[j] = s[j] > 0.0f ? d[j] * dsp / (2.0f * s[j]) : 0.0f;
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) {
+    const int e = lane + j * kWave;
+    if (e < E && active) dlogits[static_cast<int64_t>(t) * E + e] = d[j];
+  }
+}
+
+int check_router_args(int64_t T, int64_t E, int64_t K) {
+  MI355_REQUIRE(T >= 0 && T < (1ll << 31), "router: T=%lld out of range", (long long)T);
+  MI355_REQUIRE(E >= 1 && E <= kMaxVPL * kWave, "router: E=%lld must be in [1,%d]", (long long)E,
+                kMaxVPL * kWave);
+  MI355_REQUIRE(K >= 1 && K <= E, "router: K=%lld must be in [1,E]", (long long)K);
+  return MI355_OK;
+}
+
+}  // namespace
+}  // namespace mi355
+
+using namespace mi355;
+
+extern "C" int mi355_router_gate_fwd(const void* x, int x_dtype, const void* w, int w_dtype,
+                                     const float* logit_bias, float* logits, int64_t T, int64_t D,
+                                     int64_t E, void* stream) {
+  MI355_REQUIRE(T >= 0 && D >= 1 && E >= 1, "router_gate_fwd: bad shape T=%lld D=%lld E=%lld",
+                (long long)T, (long long)D, (long long)E);
+  MI355_REQUIRE(T < (1ll << 31) && D < (1ll << 31), "router_gate_fwd: shape exceeds int32");
+  if (T == 0) return MI355_OK;
+  MI355_REQUIRE(x && w && logits, "router_gate_fwd: null pointer");
+  GemmArgs g{};
+  g.A = x; g.B = w; g.C = logits; g.bias = logit_bias;
+  g.a_rs = D; g.a_cs = 1;
+  g.b_rs = 1; g.b_cs = D;  // B(k=d, n=e) = w[e][d]
+  g.ldc = E; g.M = (int)T; g.N = (int)E; g.K = (int)D;
+  g.mode = GEMM_DENSE; g.ksplit = 1;
+  return launch_gemm(g, x_dtype, w_dtype, MI355_F32, gemm_grid_dense(g.M, g.N, 1), as_stream(stream));
+}
+
+static int gate_bwd_ksplit(int64_t T, int64_t D, int64_t E) {
+  const int64_t tiles = ((E + 63) / 64) * ((D + 63) / 64);
+  int64_t split = (1024 + tiles - 1) / tiles;
+  const int64_t max_split = (T + 255) / 256;
+  if (split > max_split) split = max_split;
+  if (split < 1) split = 1;
+  if (split > 64) split = 64;
+  return (int)split;
+}
+
+extern "C" int64_t mi355_router_gate_bwd_workspace_bytes(int64_t T, int64_t D, int64_t E) {
+  const int s = gate_bwd_ksplit(T, D, E);
+  return s > 1 ? (int64_t)s * E * D * 4 : 0;
+}
+
+extern "C" int mi355_router_gate_bwd(const float* dlogits, const void* x, int x_dtype,
+                                     const void* w, int w_dtype, void* dx, void* dw,
+                                     void* workspace, int64_t T, int64_t D, int64_t E,
+                                     void* stream) {
+  MI355_REQUIRE(T >= 0 && D >= 1 && E >= 1 && T < (1ll << 31) && D < (1ll << 31),
+                "router_gate_bwd: bad shape");
+  hipStream_t s = as_stream(stream);
+  if (dx && T > 0) {
+    GemmArgs g{};
+    g.A = dlogits; g.B = w; g.C = dx;
+    g.a_rs = E; g.a_cs = 1;
+    g.b_rs = D; g.b_cs = 1;  // B(k=e, n=d) = w[e][d]
+    g.ldc = D; g.M = (int)T; g.N = (int)D; g.K = (int)E;
+    g.mode = GEMM_DENSE; g.ksplit = 1;
+    int rc = launch_gemm(g, MI355_F32, w_dtype, x_dtype, gemm_grid_dense(g.M, g.N, 1), s);
+    if (rc) return rc;
+  }
+  if (dw) {
+    const int split = gate_bwd_ksplit(T, D, E);
+    MI355_REQUIRE(split == 1 || workspace, "router_gate_bwd: workspace required");
+    GemmArgs g{};
+    g.A = dlogits; g.B = x;
+    g.a_rs = 1; g.a_cs = E;  // A(m=e, k=t) = dlogits[t][e]
+    g.b_rs = D; g.b_cs = 1;  // B(k=t, n=d) = x[t][d]
+    g.ldc = D; g.M = (int)E; g.N = (int)D; g.K = (int)T;
+    g.mode = GEMM_DENSE; g.ksplit = split;
+    g.C = split > 1 ? workspace : dw;
+    int rc = launch_gemm(g, MI355_F32, x_dtype, w_dtype, gemm_grid_dense(g.M, g.N, split), s);
+    if (rc) return rc;
+    if (split > 1)
+      return launch_splitk_reduce(static_cast<const float*>(workspace), dw, w_dtype, E * D, split, s);
+  }
+  return MI355_OK;
+}
+
+#define DISPATCH_VPL(E, ...)                           \
+  do {                                                 \
+    const int vpl_ = (int)(((E) + 63) / 64);           \
+    if (vpl_ <= 1) { constexpr int VPL = 1; __VA_ARGS__; } \
+    else if (vpl_ <= 2) { constexpr int VPL = 2; __VA_ARGS__; } \
+    else if (vpl_ <= 4) { constexpr int VPL = 4; __VA_ARGS__; } \
+    else { constexpr int VPL = 8; __VA_ARGS__; }       \
+  } while (0)
+
+extern "C" int mi355_router_select_fwd(const float* logits, const float* expert_bias,
+                                       float* weights, int64_t* ids, float* scores_TE, int64_t T,
+                                       int64_t E, int64_t K, int score_func, int route_norm,
+                                       float route_scale, int num_groups, int num_limited,
+                                       int select_mode, void* stream) {
+  if (int rc = check_router_args(T, E, K)) return rc;
+  MI355_REQUIRE(score_func >= 0 && score_func <= 2, "router_select_fwd: unknown score_func %d", score_func);
+  MI355_REQUIRE(select_mode >= 0 && select_mode <= 2, "router_select_fwd: unknown select_mode %d", select_mode);
+  MI355_REQUIRE(K <= 64, "router_select_fwd: top_k > 64 unsupported");
+  if (num_groups > 0) {
+    MI355_REQUIRE(num_groups <= 64 && E % num_groups == 0 && E / num_groups >= 2 &&
+                      num_limited >= 1 && num_limited <= num_groups &&
+                      K <= (int64_t)num_limited * (E / num_groups),
+                  "router_select_fwd: bad group config G=%d L=%d", num_groups, num_limited);
+  }
+  if (T == 0) return MI355_OK;
+  MI355_REQUIRE(logits && weights && ids, "router_select_fwd: null pointer");
+  const dim3 grid((unsigned)((T + 3) / 4));
+  DISPATCH_VPL(E, hipLaunchKernelGGL(select_fwd_kernel<VPL>, grid, dim3(256), 0, as_stream(stream),
+                                     logits, expert_bias, weights, ids, scores_TE, (int)T, (int)E,
+                                     (int)K, score_func, route_norm, route_scale, num_groups,
+                                     num_limited, select_mode));
+  return check_launch("router_select_fwd");
+}
+
+extern "C" int mi355_router_select_bwd(const float* logits, const int64_t* ids,
+                                       const float* dweights, const float* dscores_TE,
+                                       float* dlogits, int64_t T, int64_t E, int64_t K,
+                                       int score_func, int route_norm, float route_scale,
+                                       int select_mode, void* stream) {
+  if (int rc = check_router_args(T, E, K)) return rc;
+  MI355_REQUIRE(K <= 64, "router_select_bwd: top_k > 64 unsupported");
+  if (T == 0) return MI355_OK;
+  MI355_REQUIRE(logits && ids && dlogits, "router_select_bwd: null pointer");
+  const dim3 grid((unsigned)((T + 3) / 4));
+  const size_t lds = (size_t)4 * 2 * E * sizeof(float);
+  DISPATCH_VPL(E, hipLaunchKernelGGL(select_bwd_kernel<VPL>, grid, dim3(256), lds, as_stream(stream),
+                                     logits, ids, dweights, dscores_TE, dlogits, (int)T, (int)E,
+                                     (int)K, score_func, route_norm, route_scale, select_mode));
+  return check_launch("router_select_bwd");
+}

@@ -1,0 +1,182 @@
+"""Expert weights and the routed-expert module, on the grouped SwiGLU kernels.
+
+Constructor surface, parameter names and validation of
+llmtuner/models/common/moe/experts.py:73-343 (``GroupedExperts``,
+``RoutedExperts``, ``DispatchObservation``, ``ExpertErrorCapture``).  The three
+stacked parameters keep their names and layouts -- ``w1_EFD`` and ``w3_EFD`` of
+shape ``(E, F, D)``, ``w2_EDF`` of shape ``(E, D, F)`` -- so a reference state
+dict loads key for key.
+
+``RoutedExperts.forward`` keeps the reference signature; ``forward_planned`` is the
+same computation for a caller that already holds the permutation plan (the MoE
+block does), and never synchronises the host with the device.
+"""
+
+from __future__ import annotations
+
+from contextlib import AbstractContextManager, nullcontext
+from dataclasses import dataclass
+from typing import Protocol
+
+import torch
+import torch.nn as nn
+
+from .. import functional as Fn
+from .. import ops
+from .activation import SwiGLU
+
+__all__ = [
+    "DenseSwiGLU",
+    "DispatchObservation",
+    "ExpertErrorCapture",
+    "GroupedExperts",
+    "RoutedExperts",
+]
+
+
+class DispatchObserver(Protocol):
+    def measure(self, device: torch.device) -> AbstractContextManager[None]: ...
+
+
+@dataclass(eq=False, slots=True)
+class DispatchObservation:
+    """Optional observation boundary entered by the expert dispatch forward."""
+
+    observer: DispatchObserver | None = None
+
+    def measure(self, device: torch.device) -> AbstractContextManager[None]:
+        return nullcontext() if self.observer is None else self.observer.measure(device)
+
+
+@dataclass
+class ExpertErrorCapture:
+    """Carries a local compute error past module hooks; check ``error`` before use."""
+
+    error: BaseException | None = None
+
+
+class GroupedExperts(nn.Module):
+    """All experts' weights as three ``(E, O, I)`` tensors."""
+
+    def __init__(
+        self,
+        dim: int,
+        hidden_dim: int,
+        num_experts: int,
+        *,
+        activation_fn: nn.Module | None = None,
+        use_grouped_mm: bool | None = None,
+    ) -> None:
+        super().__init__()
+        for name, value in (("dim", dim), ("hidden_dim", hidden_dim), ("num_experts", num_experts)):
+            if not isinstance(value, int) or isinstance(value, bool) or value < 1:
+                raise ValueError(f"{name} must be positive integer, got {value!r}")
+        if use_grouped_mm is not None and not isinstance(use_grouped_mm, bool):
+            raise TypeError("use_grouped_mm must be bool or None")
+        if activation_fn is not None and not isinstance(activation_fn, SwiGLU):
+            raise NotImplementedError(
+                "the grouped expert kernels fuse SwiGLU; other activations are not implemented"
+            )
+        self.num_experts = num_experts
+        self.hidden_dim = hidden_dim
+        self.dim = dim
+        # Kept for interface parity; the device path always runs the grouped kernels.
+        self.use_grouped_mm = True if use_grouped_mm is None else use_grouped_mm
+        self.activation_fn = activation_fn if activation_fn is not None else SwiGLU()
+        self.w1_EFD = nn.Parameter(torch.empty(num_experts, hidden_dim, dim))
+        self.w3_EFD = nn.Parameter(torch.empty(num_experts, hidden_dim, dim))
+        self.w2_EDF = nn.Parameter(torch.empty(num_experts, dim, hidden_dim))
+
+    def forward(self, x_RD, num_tokens_per_expert_E, *, error_capture: ExpertErrorCapture | None = None):
+        if error_capture is None:
+            return self._compute(x_RD, num_tokens_per_expert_E)
+        error_capture.error = None
+        try:
+            return self._compute(x_RD, num_tokens_per_expert_E)
+        except BaseException as error:  # noqa: BLE001 - deferred to the caller by contract
+            error_capture.error = error
+            return x_RD.detach()
+
+    def _weights_as(self, dtype):
+        cast = lambda w: w if w.dtype == dtype else w.to(dtype)
+        return cast(self.w1_EFD), cast(self.w3_EFD), cast(self.w2_EDF)
+
+    def _compute(self, x_RD, num_tokens_per_expert_E):
+        if x_RD.ndim != 2 or x_RD.shape[1] != self.dim:
+            raise ValueError(
+                f"Expert inputs must have shape (routed_tokens, {self.dim}), got {tuple(x_RD.shape)}"
+            )
+        if x_RD.shape[0] > torch.iinfo(torch.int32).max:
+            raise ValueError("Routed token count exceeds int32 grouped GEMM offsets")
+        if tuple(num_tokens_per_expert_E.shape) != (self.num_experts,):
+            raise ValueError(
+                f"Expert token counts must have shape ({self.num_experts},), "
+                f"got {tuple(num_tokens_per_expert_E.shape)}"
+            )
+        if num_tokens_per_expert_E.dtype not in (
+            torch.uint8, torch.int8, torch.int16, torch.int32, torch.int64,
+        ):
+            raise TypeError("Expert token counts must use an integer dtype")
+        # Counts are clamped on the device (negatives to zero, segments to the rows
+        # that exist), so malformed counts cannot make a kernel read out of bounds.
+        plan = ops.segments_from_counts(num_tokens_per_expert_E, x_RD.shape[0])
+        return self.compute_planned(x_RD, plan)
+
+    def compute_planned(self, x_RD, plan: ops.PermutePlan):
+        w1, w3, w2 = self._weights_as(x_RD.dtype)
+        return Fn.grouped_swiglu(x_RD, w1, w3, w2, plan)
+
+
+class RoutedExperts(nn.Module):
+    """The dispatch/combine pair wrapped around the grouped expert weights."""
+
+    def __init__(self, grouped_experts: GroupedExperts, dispatcher) -> None:
+        super().__init__()
+        self.inner_experts = grouped_experts
+        self.token_dispatcher = dispatcher
+        self.dispatch_observation = DispatchObservation() if type(self) is RoutedExperts else None
+
+    def forward(self, x_TD, topk_scores_TK, topk_expert_ids_TK, num_local_tokens_per_expert_E):
+        """Dispatch tokens to experts, run them, and combine the results."""
+        del num_local_tokens_per_expert_E  # the plan recounts on the device
+        self.token_dispatcher._check_routing(x_TD, topk_scores_TK, topk_expert_ids_TK)
+        plan = self.token_dispatcher.plan(topk_expert_ids_TK)
+        return self.forward_planned(x_TD, topk_scores_TK, plan)
+
+    def forward_planned(self, x_TD, topk_scores_TK, plan: ops.PermutePlan):
+        with (
+            self.dispatch_observation.measure(x_TD.device)
+            if self.dispatch_observation is not None
+            else nullcontext()
+        ):
+            rows = Fn.permute_rows(x_TD, plan)
+        y = self.inner_experts.compute_planned(rows, plan)
+        out = Fn.combine(y, topk_scores_TK, plan, not self.token_dispatcher.accumulate_in_fp32)
+        return out.to(x_TD.dtype)
+
+
+class DenseSwiGLU(nn.Module):
+    """A dense SwiGLU MLP (the shared expert) on the same grouped kernels, E = 1.
+
+    Parameter names follow the HF MLP the reference reuses as the shared expert
+    (llmtuner/parallel/expert_parallel/block_conversion.py:278-291):
+    ``gate_proj.weight (F, D)``, ``up_proj.weight (F, D)``, ``down_proj.weight (D, F)``.
+    """
+
+    def __init__(self, dim: int, hidden_dim: int) -> None:
+        super().__init__()
+        self.gate_proj = nn.Linear(dim, hidden_dim, bias=False)
+        self.up_proj = nn.Linear(dim, hidden_dim, bias=False)
+        self.down_proj = nn.Linear(hidden_dim, dim, bias=False)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        lead = x.shape[:-1]
+        x2 = x.reshape(-1, x.shape[-1])
+        counts = torch.full((1,), x2.shape[0], dtype=torch.int32, device=x2.device)
+        plan = ops.segments_from_counts(counts, x2.shape[0])
+        dt = x2.dtype
+        cast = lambda w: (w if w.dtype == dt else w.to(dt)).unsqueeze(0)
+        y = Fn.grouped_swiglu(
+            x2, cast(self.gate_proj.weight), cast(self.up_proj.weight), cast(self.down_proj.weight), plan
+        )
+        return y.reshape(*lead, y.shape[-1])

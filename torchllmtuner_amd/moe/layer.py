@@ -1,0 +1,159 @@
+"""The MoE block: route, dispatch, expert compute, combine, (shared experts), sum.
+
+Drop-in for llmtuner/models/common/moe/layer.py:88-309 (``MoE``): same
+constructor, same module tree and state-dict keys (``router.gate.weight``,
+``routed_experts.inner_experts.{w1_EFD,w3_EFD,w2_EDF}``, persistent fp32 buffer
+``expert_bias_E``, non-persistent fp32 buffer ``tokens_per_expert_E``,
+``shared_experts.*``), same ``forward(x, *, padding_mask=None)`` contract
+including ``(..., T, D)`` inputs, staged padding masks, training-only counters
+committed after both expert paths succeed, and ``returns_router_logits``.
+"""
+
+from __future__ import annotations
+
+import math
+from collections.abc import Iterator
+from contextvars import ContextVar
+from numbers import Real
+
+import torch
+import torch.nn as nn
+
+from .experts import RoutedExperts
+from .routing import TokenChoiceTopKRouter
+
+__all__ = ["MoE", "in_checkpoint_recompute"]
+
+# Set by an activation-checkpointing wrapper while it replays a forward; counter
+# updates are skipped there (llmtuner/models/common/aux_loss.py:47-68).
+in_checkpoint_recompute: ContextVar[bool] = ContextVar("in_checkpoint_recompute", default=False)
+
+
+class MoE(nn.Module):
+    def __init__(
+        self,
+        num_experts: int,
+        routed_experts: RoutedExperts,
+        router: TokenChoiceTopKRouter,
+        *,
+        load_balance_coeff: float | None = 1e-3,
+        shared_experts: nn.Module | None = None,
+    ) -> None:
+        super().__init__()
+        if not isinstance(num_experts, int) or isinstance(num_experts, bool) or num_experts < 1:
+            raise ValueError("num_experts must be a positive integer")
+        if num_experts != router.num_experts:
+            raise ValueError(
+                f"MoE num_experts ({num_experts}) must match router.num_experts ({router.num_experts})"
+            )
+        dispatcher = routed_experts.token_dispatcher
+        if dispatcher is None:
+            raise ValueError("MoE routed experts require a token dispatcher")
+        if dispatcher.num_experts != num_experts:
+            raise ValueError(
+                "MoE dispatcher.num_experts must match router.num_experts; "
+                f"got {dispatcher.num_experts} and {num_experts}"
+            )
+        if dispatcher.top_k != router.top_k:
+            raise ValueError(
+                f"MoE dispatcher.top_k must match router.top_k; got {dispatcher.top_k} and {router.top_k}"
+            )
+        if load_balance_coeff is not None and (
+            not isinstance(load_balance_coeff, Real)
+            or isinstance(load_balance_coeff, bool)
+            or not math.isfinite(load_balance_coeff)
+            or load_balance_coeff <= 0.0
+        ):
+            raise ValueError(f"load_balance_coeff must be finite and positive, got {load_balance_coeff}")
+        self.routed_experts = routed_experts
+        self.router = router
+        self.shared_experts = shared_experts
+        self.load_balance_coeff = load_balance_coeff
+        if load_balance_coeff is not None:
+            self.register_buffer(
+                "expert_bias_E", torch.zeros(num_experts, dtype=torch.float32), persistent=True
+            )
+        else:
+            self.expert_bias_E = None
+        self.register_buffer(
+            "tokens_per_expert_E", torch.zeros(num_experts, dtype=torch.float32), persistent=False
+        )
+        self._pending_padding_mask: torch.Tensor | None = None
+        self.returns_router_logits = False
+
+    # The two statistics buffers stay fp32 when the block is cast to bf16
+    # (llmtuner/parallel/expert_parallel/block_conversion.py:61-79).
+    def _apply(self, fn, *args, **kwargs):
+        keep = {
+            name: getattr(self, name)
+            for name in ("expert_bias_E", "tokens_per_expert_E")
+            if isinstance(getattr(self, name, None), torch.Tensor)
+        }
+        super()._apply(fn, *args, **kwargs)
+        for name, old in keep.items():
+            new = getattr(self, name)
+            if new.dtype != torch.float32:
+                self._buffers[name] = old.to(device=new.device, dtype=torch.float32)
+        return self
+
+    def expert_parallel_parameters(self) -> Iterator[nn.Parameter]:
+        yield from self.routed_experts.inner_experts.parameters()
+
+    @torch.no_grad()
+    def update_expert_bias(self) -> None:
+        """Sign-based, mean-centred bias nudge from the accumulated counts (layer.py:204-228)."""
+        if self.expert_bias_E is None or self.load_balance_coeff is None:
+            return
+        counts_E = self.tokens_per_expert_E
+        delta_E = self.load_balance_coeff * torch.sign(counts_E.mean() - counts_E)
+        self.expert_bias_E.add_(delta_E - delta_E.mean())
+        self.tokens_per_expert_E.zero_()
+
+    def set_padding_mask(self, padding_mask: torch.Tensor | None) -> None:
+        self._pending_padding_mask = padding_mask
+
+    def forward(self, x: torch.Tensor, *, padding_mask: torch.Tensor | None = None):
+        if padding_mask is None:
+            padding_mask = self._pending_padding_mask
+        restore_shape = x.dim() > 2
+        tokens = x.reshape(-1, x.shape[-1]) if restore_shape else x
+        if restore_shape and padding_mask is not None:
+            padding_mask = padding_mask.reshape(-1)
+        if padding_mask is not None:
+            if padding_mask.dtype != torch.bool:
+                raise ValueError(f"padding_mask_T must have dtype bool, got {padding_mask.dtype}.")
+            if padding_mask.shape != tokens.shape[:-1]:
+                raise ValueError(
+                    "padding_mask_T must have shape matching the routing-map token axis, "
+                    f"got {tuple(padding_mask.shape)} for {tokens.shape[0]} tokens."
+                )
+
+        router = self.router
+        if router.training and router.aux_loss is not None:
+            # the aux-loss hook needs the full score map and the routing map
+            topk_scores_TK, topk_expert_ids_TK, _ = router(
+                tokens, self.expert_bias_E, padding_mask_T=padding_mask
+            )
+        else:
+            topk_scores_TK, topk_expert_ids_TK = router.route(tokens, self.expert_bias_E)
+
+        plan = self.routed_experts.token_dispatcher.plan(topk_expert_ids_TK)
+        out_TD = self.routed_experts.forward_planned(tokens, topk_scores_TK, plan)
+
+        if self.shared_experts is not None:
+            out_TD = out_TD + self.shared_experts(tokens)
+        # Commit this block's observations only after both expert paths succeeded.
+        if self.training and not in_checkpoint_recompute.get():
+            with torch.no_grad():
+                if padding_mask is None:
+                    valid_counts_E = plan.counts_E.to(torch.float32)
+                else:
+                    keep = (~padding_mask).to(torch.float32).repeat_interleave(plan.top_k)
+                    valid_counts_E = torch.zeros_like(self.tokens_per_expert_E).scatter_add_(
+                        0, topk_expert_ids_TK.reshape(-1), keep
+                    )
+                self.tokens_per_expert_E.add_(valid_counts_E)
+
+        if restore_shape:
+            out_TD = out_TD.reshape(*x.shape[:-1], out_TD.shape[-1])
+        return (out_TD, None) if self.returns_router_logits else out_TD

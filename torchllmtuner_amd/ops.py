@@ -1,0 +1,343 @@
+"""Tensor-level wrappers over the C ABI: allocate outputs, pass pointers, check codes.
+
+PyTorch is used here for device memory and the current stream only.  Every function
+requires device tensors and raises if given CPU tensors -- the kernels are the only
+implementation.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+from . import _lib
+
+_DT = {torch.float32: 0, torch.bfloat16: 1}
+SCORE_FUNCS = {"sigmoid": 0, "softmax": 1, "sqrtsoftplus": 2}
+SELECT_TOPK, SELECT_FIXED, SELECT_BALANCED = 0, 1, 2
+
+
+def _dt(t: torch.Tensor) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise TypeError(f"MI355 MoE kernels support float32 and bfloat16, got {t.dtype}") from None
+
+
+def _dev(*tensors: torch.Tensor | None) -> torch.device:
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if t.device.type != "cuda":
+            raise RuntimeError(
+                "MI355 MoE kernels need tensors on a HIP device (got "
+                f"{t.device}); there is no CPU implementation"
+            )
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise RuntimeError(f"tensors on different devices: {dev} and {t.device}")
+    return dev
+
+
+def _p(t: torch.Tensor | None):
+    return None if t is None else t.data_ptr()
+
+
+def _stream(dev: torch.device):
+    return torch.cuda.current_stream(dev).cuda_stream
+
+
+def _c(t: torch.Tensor) -> torch.Tensor:
+    return t if t.is_contiguous() else t.contiguous()
+
+
+def tile_m(dtype: torch.dtype = torch.bfloat16) -> int:
+    return int(_lib.load().mi355_grouped_tile_m(_DT[dtype]))
+
+
+# ------------------------------------------------------------------ router
+def router_gate_fwd(x_TD, w_ED, logit_bias_E=None):
+    dev = _dev(x_TD, w_ED, logit_bias_E)
+    x_TD, w_ED = _c(x_TD), _c(w_ED)
+    T, D = x_TD.shape
+    E = w_ED.shape[0]
+    if w_ED.shape[1] != D:
+        raise ValueError(f"gate weight {tuple(w_ED.shape)} does not match input dim {D}")
+    bias = None if logit_bias_E is None else _c(logit_bias_E.float())
+    out = torch.empty(T, E, dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_router_gate_fwd(
+            _p(x_TD), _dt(x_TD), _p(w_ED), _dt(w_ED), _p(bias), _p(out), T, D, E, _stream(dev)
+        )
+    _lib.check(rc, "router_gate_fwd")
+    return out
+
+
+def router_gate_bwd(dlogits_TE, x_TD, w_ED, need_dx=True, need_dw=True):
+    dev = _dev(dlogits_TE, x_TD, w_ED)
+    dlogits_TE, x_TD, w_ED = _c(dlogits_TE.float()), _c(x_TD), _c(w_ED)
+    T, D = x_TD.shape
+    E = w_ED.shape[0]
+    lib = _lib.load()
+    dx = torch.empty_like(x_TD) if need_dx else None
+    dw = torch.empty_like(w_ED) if need_dw else None
+    ws = None
+    if need_dw:
+        nbytes = lib.mi355_router_gate_bwd_workspace_bytes(T, D, E)
+        if nbytes:
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        rc = lib.mi355_router_gate_bwd(
+            _p(dlogits_TE), _p(x_TD), _dt(x_TD), _p(w_ED), _dt(w_ED), _p(dx), _p(dw), _p(ws),
+            T, D, E, _stream(dev),
+        )
+    _lib.check(rc, "router_gate_bwd")
+    return dx, dw
+
+
+def router_select_fwd(logits_TE, expert_bias_E, top_k, score_func, route_norm, route_scale,
+                      num_groups=0, num_limited=0, mode=SELECT_TOPK, want_scores=False):
+    dev = _dev(logits_TE, expert_bias_E)
+    if logits_TE.dtype != torch.float32:
+        raise TypeError("router logits must be float32")
+    logits_TE = _c(logits_TE)
+    T, E = logits_TE.shape
+    bias = None if expert_bias_E is None else _c(expert_bias_E.float())
+    weights = torch.empty(T, top_k, dtype=torch.float32, device=dev)
+    ids = torch.empty(T, top_k, dtype=torch.int64, device=dev)
+    scores = torch.empty(T, E, dtype=torch.float32, device=dev) if want_scores else None
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_router_select_fwd(
+            _p(logits_TE), _p(bias), _p(weights), _p(ids), _p(scores), T, E, top_k,
+            SCORE_FUNCS[score_func], int(route_norm), float(route_scale), int(num_groups or 0),
+            int(num_limited or 0), mode, _stream(dev),
+        )
+    _lib.check(rc, "router_select_fwd")
+    return weights, ids, scores
+
+
+def router_select_bwd(logits_TE, ids_TK, dweights_TK, dscores_TE, score_func, route_norm,
+                      route_scale, mode=SELECT_TOPK):
+    dev = _dev(logits_TE, ids_TK, dweights_TK, dscores_TE)
+    logits_TE, ids_TK = _c(logits_TE), _c(ids_TK)
+    T, E = logits_TE.shape
+    K = ids_TK.shape[1]
+    dweights_TK = None if dweights_TK is None else _c(dweights_TK.float())
+    dscores_TE = None if dscores_TE is None else _c(dscores_TE.float())
+    out = torch.empty_like(logits_TE)
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_router_select_bwd(
+            _p(logits_TE), _p(ids_TK), _p(dweights_TK), _p(dscores_TE), _p(out), T, E, K,
+            SCORE_FUNCS[score_func], int(route_norm), float(route_scale), mode, _stream(dev),
+        )
+    _lib.check(rc, "router_select_bwd")
+    return out
+
+
+# ------------------------------------------------------------------ plan
+@dataclass
+class PermutePlan:
+    """Device-resident description of the expert-major row layout (all int32)."""
+
+    num_tokens: int
+    top_k: int
+    num_experts: int
+    local_lo: int
+    local_hi: int
+    align: int
+    tile_m: int
+    row_capacity: int
+    tile_capacity: int
+    counts_E: torch.Tensor | None
+    seg_offsets: torch.Tensor
+    seg_counts: torch.Tensor
+    row_of_slot: torch.Tensor | None
+    slot_of_row: torch.Tensor | None
+    tile_expert: torch.Tensor
+    tile_row0: torch.Tensor
+    num_tiles: torch.Tensor
+
+    @property
+    def num_local_experts(self) -> int:
+        return self.local_hi - self.local_lo
+
+    @property
+    def total_rows(self) -> torch.Tensor:
+        """0-d device view of the number of rows in use (padding included)."""
+        return self.seg_offsets[self.num_local_experts]
+
+
+def permute_plan(ids_TK, num_experts, local_lo=0, local_hi=None, align=1) -> PermutePlan:
+    dev = _dev(ids_TK)
+    if ids_TK.dtype != torch.int64:
+        ids_TK = ids_TK.to(torch.int64)
+    ids_TK = _c(ids_TK)
+    T, K = ids_TK.shape
+    E = int(num_experts)
+    hi = E if local_hi is None else int(local_hi)
+    lo = int(local_lo)
+    El = hi - lo
+    N = T * K
+    tm = tile_m()
+    row_cap = N + (El * (align - 1) if align > 1 else 0)
+    tile_cap = N // tm + El + 1
+    lib = _lib.load()
+    i32 = dict(dtype=torch.int32, device=dev)
+    # one allocation for the small arrays, one for the per-slot / per-row ones
+    small = torch.empty(E + (El + 1) + El + 2 * tile_cap + 1, **i32)
+    o = 0
+    counts_E = small[o:o + E]; o += E
+    seg_offsets = small[o:o + El + 1]; o += El + 1
+    seg_counts = small[o:o + El]; o += El
+    tile_expert = small[o:o + tile_cap]; o += tile_cap
+    tile_row0 = small[o:o + tile_cap]; o += tile_cap
+    num_tiles = small[o:o + 1]
+    row_of_slot = torch.empty(N, **i32)
+    slot_of_row = torch.empty(row_cap, **i32)
+    ws = torch.empty(lib.mi355_permute_plan_workspace_bytes(T, K, E), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        rc = lib.mi355_permute_plan(
+            _p(ids_TK), T, K, E, lo, hi, align, tm, _p(counts_E), _p(seg_offsets), _p(seg_counts),
+            _p(row_of_slot), _p(slot_of_row), row_cap, _p(tile_expert), _p(tile_row0),
+            _p(num_tiles), tile_cap, _p(ws), _stream(dev),
+        )
+    _lib.check(rc, "permute_plan")
+    return PermutePlan(T, K, E, lo, hi, align, tm, row_cap, tile_cap, counts_E, seg_offsets,
+                       seg_counts, row_of_slot, slot_of_row, tile_expert, tile_row0, num_tiles)
+
+
+def segments_from_counts(counts_e, total_rows: int) -> PermutePlan:
+    """Plan for rows that are already expert-major with ``counts_e`` rows each."""
+    dev = _dev(counts_e)
+    counts = _c(counts_e.to(torch.int32))
+    El = counts.shape[0]
+    tm = tile_m()
+    tile_cap = total_rows // tm + El + 1
+    i32 = dict(dtype=torch.int32, device=dev)
+    small = torch.empty((El + 1) + El + 2 * tile_cap + 1, **i32)
+    o = 0
+    seg_offsets = small[o:o + El + 1]; o += El + 1
+    seg_counts = small[o:o + El]; o += El
+    tile_expert = small[o:o + tile_cap]; o += tile_cap
+    tile_row0 = small[o:o + tile_cap]; o += tile_cap
+    num_tiles = small[o:o + 1]
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_segments_from_counts(
+            _p(counts), El, tm, total_rows, _p(seg_offsets), _p(seg_counts), _p(tile_expert), _p(tile_row0),
+            _p(num_tiles), tile_cap, _stream(dev),
+        )
+    _lib.check(rc, "segments_from_counts")
+    return PermutePlan(0, 1, El, 0, El, 1, tm, total_rows, tile_cap, None, seg_offsets, seg_counts,
+                       None, None, tile_expert, tile_row0, num_tiles)
+
+
+# ------------------------------------------------------------------ row movers
+def permute_rows_fwd(x_TD, plan: PermutePlan):
+    dev = _dev(x_TD, plan.slot_of_row)
+    x_TD = _c(x_TD)
+    T, D = x_TD.shape
+    rows = torch.empty(plan.row_capacity, D, dtype=x_TD.dtype, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_permute_rows_fwd(
+            _p(x_TD), _dt(x_TD), _p(plan.slot_of_row), _p(plan.total_rows), _p(rows), T, D,
+            plan.top_k, plan.row_capacity, _stream(dev),
+        )
+    _lib.check(rc, "permute_rows_fwd")
+    return rows
+
+
+def permute_rows_bwd(drows_RD, plan: PermutePlan):
+    dev = _dev(drows_RD, plan.row_of_slot)
+    drows_RD = _c(drows_RD)
+    D = drows_RD.shape[1]
+    dx = torch.empty(plan.num_tokens, D, dtype=drows_RD.dtype, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_permute_rows_bwd(
+            _p(drows_RD), _dt(drows_RD), _p(plan.row_of_slot), _p(dx), plan.num_tokens, D,
+            plan.top_k, _stream(dev),
+        )
+    _lib.check(rc, "permute_rows_bwd")
+    return dx
+
+
+def combine_fwd(y_RD, weights_TK, plan: PermutePlan, round_terms=True, out_dtype=None):
+    dev = _dev(y_RD, weights_TK, plan.row_of_slot)
+    y_RD, weights_TK = _c(y_RD), _c(weights_TK.float())
+    D = y_RD.shape[1]
+    out = torch.empty(plan.num_tokens, D, dtype=y_RD.dtype, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_combine_fwd(
+            _p(y_RD), _dt(y_RD), _p(weights_TK), _p(plan.row_of_slot), _p(out), plan.num_tokens, D,
+            plan.top_k, int(round_terms), _stream(dev),
+        )
+    _lib.check(rc, "combine_fwd")
+    return out
+
+
+def combine_bwd(dout_TD, y_RD, weights_TK, plan: PermutePlan, zero_padding=True):
+    dev = _dev(dout_TD, y_RD, weights_TK)
+    dout_TD, y_RD, weights_TK = _c(dout_TD), _c(y_RD), _c(weights_TK.float())
+    if dout_TD.dtype != y_RD.dtype:
+        dout_TD = dout_TD.to(y_RD.dtype)
+    D = y_RD.shape[1]
+    dy = torch.empty_like(y_RD)
+    dw = torch.empty(plan.num_tokens, plan.top_k, dtype=torch.float32, device=dev)
+    pad = plan.slot_of_row if (zero_padding and plan.align > 1) else None
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_combine_bwd(
+            _p(dout_TD), _p(y_RD), _dt(y_RD), _p(weights_TK), _p(plan.row_of_slot), _p(pad),
+            _p(plan.total_rows), _p(dy), _p(dw), plan.num_tokens, D, plan.top_k,
+            y_RD.shape[0], _stream(dev),
+        )
+    _lib.check(rc, "combine_bwd")
+    return dy, dw
+
+
+# ------------------------------------------------------------------ experts
+def grouped_swiglu_fwd(rows_RD, w1_EFD, w3_EFD, w2_EDF, plan: PermutePlan):
+    dev = _dev(rows_RD, w1_EFD, w3_EFD, w2_EDF)
+    rows_RD, w1_EFD, w3_EFD, w2_EDF = _c(rows_RD), _c(w1_EFD), _c(w3_EFD), _c(w2_EDF)
+    R, D = rows_RD.shape
+    El, F, D2 = w1_EFD.shape
+    if D2 != D or w3_EFD.shape != w1_EFD.shape or w2_EDF.shape != (El, D, F):
+        raise ValueError("expert weight shapes do not match (E,F,D)/(E,F,D)/(E,D,F)")
+    if not (w1_EFD.dtype == w3_EFD.dtype == w2_EDF.dtype == rows_RD.dtype):
+        raise TypeError("expert weights and rows must share one dtype")
+    if El != plan.num_local_experts:
+        raise ValueError(f"plan covers {plan.num_local_experts} experts, weights hold {El}")
+    mk = lambda n: torch.empty(R, n, dtype=rows_RD.dtype, device=dev)
+    gate, up, h, y = mk(F), mk(F), mk(F), mk(D)
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_grouped_swiglu_fwd(
+            _p(rows_RD), _p(w1_EFD), _p(w3_EFD), _p(w2_EDF), _dt(rows_RD), _p(plan.seg_offsets),
+            _p(plan.seg_counts), _p(plan.tile_expert), _p(plan.tile_row0), _p(plan.num_tiles),
+            plan.tile_capacity, _p(gate), _p(up), _p(h), _p(y), El, D, F, R, _stream(dev),
+        )
+    _lib.check(rc, "grouped_swiglu_fwd")
+    return y, gate, up, h
+
+
+def grouped_swiglu_bwd(dy_RD, rows_RD, w1_EFD, w3_EFD, w2_EDF, gate, up, h, plan: PermutePlan,
+                       need_drows=True, need_dw=True):
+    dev = _dev(dy_RD, rows_RD)
+    dy_RD = _c(dy_RD)
+    w1_EFD, w3_EFD, w2_EDF = _c(w1_EFD), _c(w3_EFD), _c(w2_EDF)
+    R, D = rows_RD.shape
+    El, F, _ = w1_EFD.shape
+    dgate, dup = torch.empty_like(gate), torch.empty_like(up)
+    drows = torch.empty_like(rows_RD) if need_drows else None
+    dw1 = torch.empty_like(w1_EFD) if need_dw else None
+    dw3 = torch.empty_like(w3_EFD) if need_dw else None
+    dw2 = torch.empty_like(w2_EDF) if need_dw else None
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_grouped_swiglu_bwd(
+            _p(dy_RD), _p(rows_RD), _p(w1_EFD), _p(w3_EFD), _p(w2_EDF), _p(gate), _p(up), _p(h),
+            _dt(rows_RD), _p(plan.seg_offsets), _p(plan.seg_counts), _p(plan.tile_expert),
+            _p(plan.tile_row0), _p(plan.num_tiles), plan.tile_capacity, _p(dgate), _p(dup),
+            _p(drows), _p(dw1), _p(dw3), _p(dw2), El, D, F, R, _stream(dev),
+        )
+    _lib.check(rc, "grouped_swiglu_bwd")
+    return drows, dw1, dw3, dw2
