@@ -88,4 +88,6 @@ def build_block(p: R.MoEParams, spec: R.RouterSpec, D, F, dtype, device, *, disp
             shared.down_proj.weight.copy_(p.shared_down_DF)
         if p.expert_bias_E is not None:
             block.expert_bias_E.copy_(p.expert_bias_E)
+    if p.router_logit_bias_E is not None:  # carried as router.gate.bias (linear.py:181-182)
+        block.router.gate.bias = torch.nn.Parameter(p.router_logit_bias_E.clone(), requires_grad=False)
     return block.to(device)

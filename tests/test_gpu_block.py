@@ -26,7 +26,7 @@ def _run_pair(p, spec, x, gout, dtype, D, F, **kw):
     leaves = {k: getattr(p, k).clone().requires_grad_() for k in
               ("router_w_ED", "w1_EFD", "w3_EFD", "w2_EDF", "shared_gate_FD", "shared_up_FD", "shared_down_DF")
               if getattr(p, k) is not None}
-    pr = R.MoEParams(expert_bias_E=p.expert_bias_E, **leaves)
+    pr = R.MoEParams(expert_bias_E=p.expert_bias_E, router_logit_bias_E=p.router_logit_bias_E, **leaves)
     xr = x.clone().requires_grad_()
     ref, aux = R.moe_forward(xr, pr, spec, **oracle_kw)
     ref.backward(gout)
@@ -80,8 +80,7 @@ def test_qwen3_shape_bf16_forward_backward(dispatcher, T):
     x = torch.randn(T, D, generator=torch.Generator().manual_seed(0)).bfloat16()
     gout = torch.randn(T, D, generator=torch.Generator().manual_seed(1)).bfloat16()
     kw = dict(dispatcher=dispatcher, pad_multiple=128) if dispatcher == "padded" else {}
-    leaves_bias = p.router_logit_bias_E
-    got, want, aux, block = _run_pair_with_logit_bias(p, spec, x, gout, D, F, leaves_bias, **kw)
+    got, want, aux, block = _run_pair(p, spec, x, gout, torch.bfloat16, D, F, **kw)
     # routing: compare on tokens that are not near ties of the oracle's own logits
     ok = stable_tokens(aux["logits"], spec)
     assert ok.float().mean() > 0.97
@@ -94,30 +93,6 @@ def test_qwen3_shape_bf16_forward_backward(dispatcher, T):
     for k in want:
         err = rel_l2(got[k], want[k])
         assert err < 2e-2, f"{k}: rel-L2 {err}"
-
-
-def _run_pair_with_logit_bias(p, spec, x, gout, D, F, logit_bias, **kw):
-    if logit_bias is None:
-        return _run_pair(p, spec, x, gout, torch.bfloat16, D, F, **kw)
-    # the device block carries the logit bias as router.gate.bias
-    import torch.nn as nn
-
-    from tests import helpers
-
-    orig = helpers.build_block
-
-    def patched(*a, **k):
-        block = orig(*a, **k)
-        block.router.gate.bias = nn.Parameter(logit_bias.to(DEV), requires_grad=False)
-        return block
-
-    helpers.build_block = patched
-    globals()["build_block"] = patched
-    try:
-        return _run_pair(p, spec, x, gout, torch.bfloat16, D, F, **kw)
-    finally:
-        helpers.build_block = orig
-        globals()["build_block"] = orig
 
 
 def test_deepseek_shape_local_share_with_shared_expert():

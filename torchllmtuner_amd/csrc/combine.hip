@@ -76,15 +76,19 @@ __global__ __launch_bounds__(256) void combine_fwd_kernel(
 
   constexpr int V = Vec<T>::N;
   T* dst = out + static_cast<int64_t>(t) * D;
+  // Loops are uniform across the wave (shuffles need every lane).
   if (D % V == 0) {
     const int nv = D / V;
-    for (int i = lane; i < nv; i += kWave) {
+    for (int base = 0; base < nv; base += kWave) {
+      const int i = base + lane;
+      const bool on = i < nv;
       float a[V];
 #pragma unroll
       for (int q = 0; q < V; ++q) a[q] = 0.0f;
       for (int p = 0; p < nvalid; ++p) {
         const int r = __shfl(o_row, p, kWave);
         const float ww = __shfl(o_w, p, kWave);
+        if (!on) continue;
         float f[V];
         Vec<T>::unpack(reinterpret_cast<const uint4*>(y + static_cast<int64_t>(r) * D)[i], f);
 #pragma unroll
@@ -93,18 +97,21 @@ __global__ __launch_bounds__(256) void combine_fwd_kernel(
           a[q] += round_terms ? round_to<T>(term) : term;
         }
       }
-      reinterpret_cast<uint4*>(dst)[i] = Vec<T>::pack(a);
+      if (on) reinterpret_cast<uint4*>(dst)[i] = Vec<T>::pack(a);
     }
   } else {
-    for (int i = lane; i < D; i += kWave) {
+    for (int base = 0; base < D; base += kWave) {
+      const int i = base + lane;
+      const bool on = i < D;
       float a = 0.0f;
       for (int p = 0; p < nvalid; ++p) {
         const int r = __shfl(o_row, p, kWave);
         const float ww = __shfl(o_w, p, kWave);
+        if (!on) continue;
         const float term = load_as_f32(y + static_cast<int64_t>(r) * D + i) * ww;
         a += round_terms ? round_to<T>(term) : term;
       }
-      store_from_f32(dst + i, a);
+      if (on) store_from_f32(dst + i, a);
     }
   }
 }

@@ -266,27 +266,33 @@ __global__ __launch_bounds__(256) void permute_rows_bwd_kernel(
   constexpr int V = 16 / sizeof(T);
   T* dst = dx + static_cast<int64_t>(t) * D;
   const int my_row = lane < K ? row_of_slot[static_cast<int64_t>(t) * K + lane] : -1;  // K <= 64
+  // Loops are uniform across the wave (shuffles need every lane); lanes past the
+  // end of the row just skip their loads and stores.
   if (D % V == 0) {
     const int nv = D / V;
-    for (int i = lane; i < nv; i += kWave) {
+    for (int base = 0; base < nv; base += kWave) {
+      const int i = base + lane;
+      const bool on = i < nv;
       float a[V];
 #pragma unroll
       for (int q = 0; q < V; ++q) a[q] = 0.0f;
       for (int k = 0; k < K; ++k) {
         const int row = __shfl(my_row, k, kWave);
-        if (row < 0) continue;
+        if (row < 0 || !on) continue;
         acc_vec<T>(a, reinterpret_cast<const uint4*>(drows + static_cast<int64_t>(row) * D)[i]);
       }
-      reinterpret_cast<uint4*>(dst)[i] = pack_vec<T>(a);
+      if (on) reinterpret_cast<uint4*>(dst)[i] = pack_vec<T>(a);
     }
   } else {
-    for (int i = lane; i < D; i += kWave) {
+    for (int base = 0; base < D; base += kWave) {
+      const int i = base + lane;
+      const bool on = i < D;
       float a = 0.0f;
       for (int k = 0; k < K; ++k) {
         const int row = __shfl(my_row, k, kWave);
-        if (row >= 0) a += load_as_f32(drows + static_cast<int64_t>(row) * D + i);
+        if (row >= 0 && on) a += load_as_f32(drows + static_cast<int64_t>(row) * D + i);
       }
-      store_from_f32(dst + i, a);
+      if (on) store_from_f32(dst + i, a);
     }
   }
 }
