@@ -253,6 +253,27 @@ int mi355_grouped_swiglu_bwd(const void* dy, const void* rows, const void* w1,
                              void* dw3, void* dw2, int64_t El, int64_t D, int64_t F,
                              int64_t row_capacity, void* stream);
 
+/*
+ * One of the seven bf16 MFMA kernels behind the two calls above, by itself, on the
+ * same buffers: for profilers and for callers that schedule the stages themselves.
+ * No counterpart in the reference.  bf16 only, D and F multiples of 64.
+ */
+#define MI355_STAGE_GATEUP 1 /* gate, up, h   <- rows, w1, w3 */
+#define MI355_STAGE_DOWN 2   /* y             <- h, w2        */
+#define MI355_STAGE_DH 4     /* dgate, dup    <- dy, w2, gate, up */
+#define MI355_STAGE_DX 8     /* drows         <- dgate, dup, w1, w3 */
+#define MI355_STAGE_DW2 16   /* dw2           <- dy, h        */
+#define MI355_STAGE_DW1 32   /* dw1           <- dgate, rows  */
+#define MI355_STAGE_DW3 64   /* dw3           <- dup, rows    */
+int mi355_grouped_swiglu_stage(int stage, const void* dy, const void* rows, const void* w1,
+                               const void* w3, const void* w2, void* gate, void* up,
+                               void* h, void* y, const int32_t* seg_offsets,
+                               const int32_t* seg_counts, const int32_t* tile_expert,
+                               const int32_t* tile_row0, const int32_t* num_tiles,
+                               int64_t tile_capacity, void* dgate, void* dup, void* drows,
+                               void* dw1, void* dw3, void* dw2, int64_t El, int64_t D,
+                               int64_t F, int64_t row_capacity, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -38,6 +38,10 @@ SIGNATURES = {
     "mi355_combine_bwd": (I, [P, P, I, P, P, P, P, P, P, L, L, L, L, P]),
     "mi355_grouped_tile_m": (L, [I]),
     "mi355_grouped_swiglu_fwd": (I, [P, P, P, P, I, P, P, P, P, P, L, P, P, P, P, L, L, L, L, P]),
+    "mi355_grouped_swiglu_stage": (
+        I,
+        [I, P, P, P, P, P, P, P, P, P, P, P, P, P, P, L, P, P, P, P, P, P, L, L, L, L, P],
+    ),
     "mi355_grouped_swiglu_bwd": (
         I,
         [P, P, P, P, P, P, P, P, I, P, P, P, P, P, L, P, P, P, P, P, P, L, L, L, L, P],

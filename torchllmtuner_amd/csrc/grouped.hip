@@ -14,13 +14,14 @@ int bf16_grouped_fwd(const void* rows, const void* w1, const void* w3, const voi
                      const int32_t* seg_offsets, const int32_t* seg_counts,
                      const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* num_tiles,
                      int64_t tile_capacity, void* gate, void* up, void* h, void* y, int64_t D,
-                     int64_t F, hipStream_t s);
+                     int64_t F, int stages, hipStream_t s);
 int bf16_grouped_bwd(const void* dy, const void* rows, const void* w1, const void* w3,
                      const void* w2, const void* gate, const void* up, const void* h,
                      const int32_t* seg_offsets, const int32_t* seg_counts,
                      const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* num_tiles,
                      int64_t tile_capacity, void* dgate, void* dup, void* drows, void* dw1,
-                     void* dw3, void* dw2, int64_t El, int64_t D, int64_t F, hipStream_t s);
+                     void* dw3, void* dw2, int64_t El, int64_t D, int64_t F, int stages,
+                     hipStream_t s);
 
 namespace {
 
@@ -131,7 +132,7 @@ extern "C" int mi355_grouped_swiglu_fwd(const void* rows, const void* w1, const 
   hipStream_t s = as_stream(stream);
   if (dtype == MI355_BF16 && bf16_fast_path_ok(D, F))
     return bf16_grouped_fwd(rows, w1, w3, w2, seg_offsets, seg_counts, tile_expert, tile_row0,
-                            num_tiles, tile_capacity, gate, up, h, y, D, F, s);
+                            num_tiles, tile_capacity, gate, up, h, y, D, F, 3, s);
   const Seg sg{seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles, tile_capacity};
   // gate/up: B(k=d, n=f) = w[e][f][d]
   if (int rc = rowseg(sg, rows, D, w1, 1, D, F * D, gate, F, D, dtype, 0, s)) return rc;
@@ -166,7 +167,7 @@ extern "C" int mi355_grouped_swiglu_bwd(const void* dy, const void* rows, const 
   if (dtype == MI355_BF16 && bf16_fast_path_ok(D, F) && row_capacity > 0 && tile_capacity > 0)
     return bf16_grouped_bwd(dy, rows, w1, w3, w2, gate, up, h, seg_offsets, seg_counts, tile_expert,
                             tile_row0, num_tiles, tile_capacity, dgate, dup, drows, dw1, dw3, dw2, El,
-                            D, F, s);
+                            D, F, 0x7c, s);
   const Seg sg{seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles, tile_capacity};
   if (row_capacity > 0 && tile_capacity > 0) {
     // dh = dy . w2[e]: B(k=d, n=f) = w2[e][d][f]   (lands in dgate, rewritten in place below)
@@ -191,4 +192,25 @@ extern "C" int mi355_grouped_swiglu_bwd(const void* dy, const void* rows, const 
   if (dw1) if (int rc = kseg(sg, dgate, rows, dw1, F, D, El, dtype, s)) return rc;
   if (dw3) if (int rc = kseg(sg, dup, rows, dw3, F, D, El, dtype, s)) return rc;
   return MI355_OK;
+}
+
+extern "C" int mi355_grouped_swiglu_stage(int stage, const void* dy, const void* rows, const void* w1,
+                                          const void* w3, const void* w2, void* gate, void* up,
+                                          void* h, void* y, const int32_t* seg_offsets,
+                                          const int32_t* seg_counts, const int32_t* tile_expert,
+                                          const int32_t* tile_row0, const int32_t* num_tiles,
+                                          int64_t tile_capacity, void* dgate, void* dup, void* drows,
+                                          void* dw1, void* dw3, void* dw2, int64_t El, int64_t D,
+                                          int64_t F, int64_t row_capacity, void* stream) {
+  if (int rc = check_common("grouped_swiglu_stage", MI355_BF16, El, D, F, row_capacity, tile_capacity)) return rc;
+  MI355_REQUIRE(bf16_fast_path_ok(D, F), "grouped_swiglu_stage: needs bf16 with D and F multiples of 64");
+  MI355_REQUIRE(stage > 0 && stage < 128 && (stage & (stage - 1)) == 0, "grouped_swiglu_stage: one stage bit expected");
+  if (row_capacity == 0 || tile_capacity == 0) return MI355_OK;
+  hipStream_t s = as_stream(stream);
+  if (stage <= 2)
+    return bf16_grouped_fwd(rows, w1, w3, w2, seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles,
+                            tile_capacity, gate, up, h, y, D, F, stage, s);
+  return bf16_grouped_bwd(dy, rows, w1, w3, w2, gate, up, h, seg_offsets, seg_counts, tile_expert,
+                          tile_row0, num_tiles, tile_capacity, dgate, dup, drows, dw1, dw3, dw2, El, D, F,
+                          stage, s);
 }

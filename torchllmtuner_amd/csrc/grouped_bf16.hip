@@ -403,6 +403,8 @@ __global__ __launch_bounds__(256, 2) void wgrad_kernel(WgradArgs p) {
 }  // namespace
 
 // ---- host side (called from grouped.hip) ---------------------------------------------
+// `stages` is a mask of MI355_STAGE_* bits: which of the seven GEMM kernels to launch.
+enum { STAGE_GATEUP = 1, STAGE_DOWN = 2, STAGE_DH = 4, STAGE_DX = 8, STAGE_DW2 = 16, STAGE_DW1 = 32, STAGE_DW3 = 64 };
 bool bf16_fast_path_ok(int64_t D, int64_t F) { return D % 64 == 0 && F % 64 == 0 && D >= 64 && F >= 64; }
 
 static unsigned round8(int64_t v) { return static_cast<unsigned>((v + 7) / 8 * 8); }
@@ -411,15 +413,18 @@ int bf16_grouped_fwd(const void* rows, const void* w1, const void* w3, const voi
                      const int32_t* seg_offsets, const int32_t* seg_counts,
                      const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* num_tiles,
                      int64_t tile_capacity, void* gate, void* up, void* h, void* y, int64_t D,
-                     int64_t F, hipStream_t s) {
+                     int64_t F, int stages, hipStream_t s) {
   RowArgs a{};
   a.seg_offsets = seg_offsets; a.seg_counts = seg_counts; a.tile_expert = tile_expert;
   a.tile_row0 = tile_row0; a.num_tiles = num_tiles; a.D = (int)D; a.F = (int)F;
   a.a0 = (const uint16_t*)rows; a.b0 = (const uint16_t*)w1; a.b1 = (const uint16_t*)w3;
   a.o0 = (uint16_t*)gate; a.o1 = (uint16_t*)up; a.o2 = (uint16_t*)h;
   a.n_tiles = (int)((F + BN / 2 - 1) / (BN / 2));
-  hipLaunchKernelGGL(row_tiled_kernel<RM_GATEUP>, dim3(round8(tile_capacity * a.n_tiles)), dim3(256), 0, s, a);
-  if (int rc = check_launch("grouped gate/up")) return rc;
+  if (stages & STAGE_GATEUP) {
+    hipLaunchKernelGGL(row_tiled_kernel<RM_GATEUP>, dim3(round8(tile_capacity * a.n_tiles)), dim3(256), 0, s, a);
+    if (int rc = check_launch("grouped gate/up")) return rc;
+  }
+  if (!(stages & STAGE_DOWN)) return MI355_OK;
   RowArgs b{};
   b.seg_offsets = seg_offsets; b.seg_counts = seg_counts; b.tile_expert = tile_expert;
   b.tile_row0 = tile_row0; b.num_tiles = num_tiles; b.D = (int)D; b.F = (int)F;
@@ -434,7 +439,8 @@ int bf16_grouped_bwd(const void* dy, const void* rows, const void* w1, const voi
                      const int32_t* seg_offsets, const int32_t* seg_counts,
                      const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* num_tiles,
                      int64_t tile_capacity, void* dgate, void* dup, void* drows, void* dw1,
-                     void* dw3, void* dw2, int64_t El, int64_t D, int64_t F, hipStream_t s) {
+                     void* dw3, void* dw2, int64_t El, int64_t D, int64_t F, int stages,
+                     hipStream_t s) {
   RowArgs a{};
   a.seg_offsets = seg_offsets; a.seg_counts = seg_counts; a.tile_expert = tile_expert;
   a.tile_row0 = tile_row0; a.num_tiles = num_tiles; a.D = (int)D; a.F = (int)F;
@@ -442,9 +448,11 @@ int bf16_grouped_bwd(const void* dy, const void* rows, const void* w1, const voi
   a.gate = (const uint16_t*)gate; a.up = (const uint16_t*)up;
   a.o0 = (uint16_t*)dgate; a.o1 = (uint16_t*)dup;
   a.n_tiles = (int)((F + BN - 1) / BN);
-  hipLaunchKernelGGL(row_tiled_kernel<RM_DH>, dim3(round8(tile_capacity * a.n_tiles)), dim3(256), 0, s, a);
-  if (int rc = check_launch("grouped dh")) return rc;
-  if (drows) {
+  if (stages & STAGE_DH) {
+    hipLaunchKernelGGL(row_tiled_kernel<RM_DH>, dim3(round8(tile_capacity * a.n_tiles)), dim3(256), 0, s, a);
+    if (int rc = check_launch("grouped dh")) return rc;
+  }
+  if (drows && (stages & STAGE_DX)) {
     RowArgs b{};
     b.seg_offsets = seg_offsets; b.seg_counts = seg_counts; b.tile_expert = tile_expert;
     b.tile_row0 = tile_row0; b.num_tiles = num_tiles; b.D = (int)D; b.F = (int)F;
@@ -463,9 +471,9 @@ int bf16_grouped_bwd(const void* dy, const void* rows, const void* w1, const voi
     hipLaunchKernelGGL(wgrad_kernel, dim3(round8(w.total)), dim3(256), 0, s, w);
     return check_launch(what);
   };
-  if (dw2) if (int rc = wgrad(dy, h, dw2, D, F, "grouped dw2")) return rc;
-  if (dw1) if (int rc = wgrad(dgate, rows, dw1, F, D, "grouped dw1")) return rc;
-  if (dw3) if (int rc = wgrad(dup, rows, dw3, F, D, "grouped dw3")) return rc;
+  if (dw2 && (stages & STAGE_DW2)) if (int rc = wgrad(dy, h, dw2, D, F, "grouped dw2")) return rc;
+  if (dw1 && (stages & STAGE_DW1)) if (int rc = wgrad(dgate, rows, dw1, F, D, "grouped dw1")) return rc;
+  if (dw3 && (stages & STAGE_DW3)) if (int rc = wgrad(dup, rows, dw3, F, D, "grouped dw3")) return rc;
   return MI355_OK;
 }
 

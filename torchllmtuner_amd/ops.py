@@ -341,3 +341,27 @@ def grouped_swiglu_bwd(dy_RD, rows_RD, w1_EFD, w3_EFD, w2_EDF, gate, up, h, plan
         )
     _lib.check(rc, "grouped_swiglu_bwd")
     return drows, dw1, dw3, dw2
+
+
+STAGES = {"gate_up": 1, "down": 2, "dh": 4, "drows": 8, "dw2": 16, "dw1": 32, "dw3": 64}
+
+
+def grouped_swiglu_stage(stage: str, buf: dict, plan: PermutePlan):
+    """Launch exactly one of the seven bf16 MFMA kernels on pre-allocated buffers.
+
+    ``buf`` maps the C argument names (dy, rows, w1, w3, w2, gate, up, h, y, dgate,
+    dup, drows, dw1, dw3, dw2) to device tensors.
+    """
+    rows = buf["rows"]
+    dev = _dev(rows)
+    R, D = rows.shape
+    El, F, _ = buf["w1"].shape
+    g = lambda k: _p(buf.get(k))
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_grouped_swiglu_stage(
+            STAGES[stage], g("dy"), g("rows"), g("w1"), g("w3"), g("w2"), g("gate"), g("up"), g("h"),
+            g("y"), _p(plan.seg_offsets), _p(plan.seg_counts), _p(plan.tile_expert),
+            _p(plan.tile_row0), _p(plan.num_tiles), plan.tile_capacity, g("dgate"), g("dup"),
+            g("drows"), g("dw1"), g("dw3"), g("dw2"), El, D, F, R, _stream(dev),
+        )
+    _lib.check(rc, f"grouped_swiglu_stage[{stage}]")
