@@ -1,0 +1,111 @@
+"""CPU-side checks of the C-ABI library and the host layer (no GPU, no compute calls)."""
+
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "mi355_moe.h")
+
+
+def _declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mi355_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_loads_and_exports_every_declared_symbol():
+    from torchllmtuner_amd import _lib
+
+    lib = _lib.load()
+    names = _declared_functions()
+    assert len(names) >= 18
+    raw = ctypes.CDLL(_lib.LIB_PATH)
+    for name in names:
+        assert hasattr(raw, name), f"{name} is declared in mi355_moe.h but not exported"
+        assert name in _lib.SIGNATURES, f"{name} has no ctypes prototype"
+    assert set(_lib.SIGNATURES) == set(names)
+    assert lib.mi355_moe_abi_version() == 1
+    assert lib.mi355_grouped_tile_m(1) == 128
+
+
+def test_argument_validation_reports_errors_without_a_gpu():
+    from torchllmtuner_amd import _lib
+
+    lib = _lib.load()
+    # E = 0 is rejected before any launch
+    rc = lib.mi355_router_select_fwd(None, None, None, None, None, 4, 0, 1, 0, 0, 1.0, 0, 0, 0, None)
+    assert rc == -1
+    assert b"E=0" in lib.mi355_moe_last_error()
+    rc = lib.mi355_permute_plan(None, 4, 2, 8, 5, 3, 1, 128, None, None, None, None, None, 8, None, None,
+                                None, 2, None, None)
+    assert rc == -1 and b"local range" in lib.mi355_moe_last_error()
+    with pytest.raises(ValueError, match="local range"):
+        _lib.check(rc, "permute_plan")
+
+
+def test_ops_refuse_cpu_tensors():
+    from torchllmtuner_amd import ops
+
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        ops.router_gate_fwd(torch.zeros(2, 4), torch.zeros(3, 4))
+    with pytest.raises(TypeError, match="float32 and bfloat16"):
+        ops._dt(torch.zeros(1, dtype=torch.float64))
+
+
+def test_module_surface_matches_the_reference_block():
+    """Constructor validation, parameter names and buffers of the block
+    (llmtuner/models/common/moe/layer.py:109-193, routing.py:64-144, experts.py:87-120)."""
+    from torchllmtuner_amd import moe
+
+    with pytest.raises(ValueError, match="num_limited_groups must be set"):
+        moe.TokenChoiceTopKRouter(8, 16, 2, num_expert_groups=2)
+    with pytest.raises(ValueError, match="must be divisible by num_expert_groups"):
+        moe.TokenChoiceTopKRouter(8, 16, 2, num_expert_groups=3, num_limited_groups=1)
+    with pytest.raises(ValueError, match="cannot exceed num_expert_groups"):
+        moe.TokenChoiceTopKRouter(8, 16, 2, num_expert_groups=2, num_limited_groups=5)
+    with pytest.raises(ValueError, match="must be >= 2"):
+        moe.TokenChoiceTopKRouter(8, 16, 2, num_expert_groups=8, num_limited_groups=1)
+    with pytest.raises(ValueError, match="top_k must be in"):
+        moe.TokenChoiceTopKRouter(4, 16, 5)
+    with pytest.raises(ValueError, match="Unknown score function"):
+        moe.TokenChoiceTopKRouter(4, 16, 1, score_func="relu")
+    for field in ("dim", "hidden_dim", "num_experts"):
+        opts = {"dim": 4, "hidden_dim": 8, "num_experts": 2}
+        opts[field] = True
+        with pytest.raises(ValueError, match=field + " must be positive integer"):
+            moe.GroupedExperts(**opts)
+    with pytest.raises(TypeError, match="use_grouped_mm must be bool or None"):
+        moe.GroupedExperts(4, 8, 2, use_grouped_mm=1)
+    with pytest.raises(ValueError, match="pad_multiple"):
+        moe.PaddedTokenDispatcher(4, 2, pad_multiple=0)
+
+    router = moe.TokenChoiceTopKRouter(8, 16, 2, score_func="softmax", route_norm=True)
+    experts = moe.RoutedExperts(moe.GroupedExperts(16, 32, 8), moe.LocalTokenDispatcher(8, 2))
+    with pytest.raises(ValueError, match="must match router.num_experts"):
+        moe.MoE(4, experts, router)
+    with pytest.raises(ValueError, match="load_balance_coeff must be finite and positive"):
+        moe.MoE(8, experts, router, load_balance_coeff=0.0)
+    block = moe.MoE(8, experts, router, shared_experts=moe.DenseSwiGLU(16, 32))
+    assert list(block.state_dict()) == [
+        "expert_bias_E",
+        "routed_experts.inner_experts.w1_EFD",
+        "routed_experts.inner_experts.w3_EFD",
+        "routed_experts.inner_experts.w2_EDF",
+        "router.gate.weight",
+        "shared_experts.gate_proj.weight",
+        "shared_experts.up_proj.weight",
+        "shared_experts.down_proj.weight",
+    ]
+    ie = block.routed_experts.inner_experts
+    assert ie.w1_EFD.shape == (8, 32, 16) and ie.w3_EFD.shape == (8, 32, 16) and ie.w2_EDF.shape == (8, 16, 32)
+    assert router.gate.bias is None and router.gate.weight.shape == (8, 16)
+    # statistics buffers stay fp32 under a bf16 cast; the counter is not persistent
+    block = block.to(torch.bfloat16)
+    assert block.expert_bias_E.dtype == torch.float32 and block.tokens_per_expert_E.dtype == torch.float32
+    assert "tokens_per_expert_E" not in block.state_dict()
+    assert moe.MoE(8, experts, router, load_balance_coeff=None).expert_bias_E is None
+    assert list(block.expert_parallel_parameters()) == list(ie.parameters())

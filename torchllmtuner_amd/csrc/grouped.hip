@@ -2,6 +2,8 @@
 // path.  bf16 problems whose D and F are multiples of 64 go to the MFMA kernels of
 // grouped_bf16.hip; everything else (fp32, odd shapes) runs the strided fp32-MFMA
 // GEMM plus two small elementwise kernels.
+#include <cstdlib>
+
 #include "common.h"
 #include "gemm_generic.h"
 
@@ -131,8 +133,9 @@ extern "C" int mi355_grouped_swiglu_fwd(const void* rows, const void* w1, const 
                 "grouped_swiglu_fwd: null pointer");
   hipStream_t s = as_stream(stream);
   if (dtype == MI355_BF16 && bf16_fast_path_ok(D, F))
-    return bf16_grouped_fwd(rows, w1, w3, w2, seg_offsets, seg_counts, tile_expert, tile_row0,
-                            num_tiles, tile_capacity, gate, up, h, y, D, F, 3, s);
+    return bf16_grouped_fwd(rows, w1, w3, w2, seg_offsets, seg_counts,
+                                                             tile_expert, tile_row0, num_tiles,
+                                                             tile_capacity, gate, up, h, y, D, F, 3, s);
   const Seg sg{seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles, tile_capacity};
   // gate/up: B(k=d, n=f) = w[e][f][d]
   if (int rc = rowseg(sg, rows, D, w1, 1, D, F * D, gate, F, D, dtype, 0, s)) return rc;
@@ -165,9 +168,9 @@ extern "C" int mi355_grouped_swiglu_bwd(const void* dy, const void* rows, const 
                 "grouped_swiglu_bwd: null pointer");
   hipStream_t s = as_stream(stream);
   if (dtype == MI355_BF16 && bf16_fast_path_ok(D, F) && row_capacity > 0 && tile_capacity > 0)
-    return bf16_grouped_bwd(dy, rows, w1, w3, w2, gate, up, h, seg_offsets, seg_counts, tile_expert,
-                            tile_row0, num_tiles, tile_capacity, dgate, dup, drows, dw1, dw3, dw2, El,
-                            D, F, 0x7c, s);
+    return bf16_grouped_bwd(
+        dy, rows, w1, w3, w2, gate, up, h, seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles,
+        tile_capacity, dgate, dup, drows, dw1, dw3, dw2, El, D, F, 0x7c, s);
   const Seg sg{seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles, tile_capacity};
   if (row_capacity > 0 && tile_capacity > 0) {
     // dh = dy . w2[e]: B(k=d, n=f) = w2[e][d][f]   (lands in dgate, rewritten in place below)
@@ -208,9 +211,10 @@ extern "C" int mi355_grouped_swiglu_stage(int stage, const void* dy, const void*
   if (row_capacity == 0 || tile_capacity == 0) return MI355_OK;
   hipStream_t s = as_stream(stream);
   if (stage <= 2)
-    return bf16_grouped_fwd(rows, w1, w3, w2, seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles,
-                            tile_capacity, gate, up, h, y, D, F, stage, s);
-  return bf16_grouped_bwd(dy, rows, w1, w3, w2, gate, up, h, seg_offsets, seg_counts, tile_expert,
-                          tile_row0, num_tiles, tile_capacity, dgate, dup, drows, dw1, dw3, dw2, El, D, F,
-                          stage, s);
+    return bf16_grouped_fwd(rows, w1, w3, w2, seg_offsets, seg_counts,
+                                                             tile_expert, tile_row0, num_tiles,
+                                                             tile_capacity, gate, up, h, y, D, F, stage, s);
+  return bf16_grouped_bwd(
+      dy, rows, w1, w3, w2, gate, up, h, seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles,
+      tile_capacity, dgate, dup, drows, dw1, dw3, dw2, El, D, F, stage, s);
 }

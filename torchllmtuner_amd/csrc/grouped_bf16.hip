@@ -1,27 +1,49 @@
 // Grouped SwiGLU expert GEMMs in bf16 on the gfx950 matrix cores.
 //
-// All kernels use v_mfma_f32_32x32x16_bf16: per lane 8 bf16 of A (row lane%32,
-// k = 8*(lane/32)..+7) and 8 bf16 of B (column lane%32, same k), 16 fp32 of C
-// (column lane%32, rows 8*(i/4) + 4*(lane/32) + i%4).
-//
-// Operands reach LDS in one of two layouts, chosen by which axis is contiguous in
-// HBM:
-//   KC  contraction axis contiguous ([row][k], 64 k per row): 16-byte chunks are
-//       XOR-swizzled by row so the 32 rows a fragment read touches hit distinct
-//       banks; a fragment is one ds_read_b128.
-//   KS  contraction axis strided ([k][col], col contiguous): stored as is with a
-//       padded pitch; a fragment is two ds_read_b64_tr_b16, the LDS transpose read
-//       that hands each lane 4 consecutive k of its own column.
-// That covers every product of the block without materialising a transpose:
+// Products (no transpose is ever materialised):
 //   gate/up  rows . w1^T, rows . w3^T   A KC, B KC   fused SiLU*up epilogue
 //   down     h . w2^T                   A KC, B KC
 //   dh       dy . w2                    A KC, B KS   fused SwiGLU backward epilogue
 //   drows    dgate . w1 + dup . w3      A KC, B KS   (one accumulator, K = 2F)
 //   dw*      a_e^T . b_e                A KS, B KS   K = the expert's rows
 //
-// Row-tiled kernels take their work from the permutation plan's tile list (128
-// rows of one expert each) and remap block ids so that each XCD walks a contiguous
-// run of tiles: the blocks sharing an expert's weights share an L2.
+// Shape of the kernels.  Measured on MI355X these GEMMs are bound by the number of
+// cache-line requests a CU's vector L1 keeps in flight (about 50 x 128 B at ~600 clk
+// average L2 latency = 13 B/clk/CU), not by the matrix cores: what matters is bytes
+// requested per flop.  Hence 128x512 output tiles for the row-tiled products and
+// 256x256 for the weight gradients, eight waves per workgroup (two per SIMD), one
+// workgroup per CU with the 160 KiB of LDS holding two stages of the operand tiles.
+// Row tiles come from the permutation plan's tile list (128 rows of one expert each)
+// and block ids are remapped so that each XCD walks a contiguous run of tiles: the
+// blocks that share an expert's weights share an L2.
+//
+// Row-tiled main loop: a ping-pong schedule.  Waves 4..7 run one phase behind waves
+// 0..3 (wave w and w+4 share a SIMD); a phase is either "memory" (park 2-3 chunks of
+// the next tile in the other LDS stage, fetch the same chunks of the tile after it,
+// read this step's fragments) or "MFMA" (8 matrix instructions), separated by
+// s_barrier with only the wave's own LDS traffic waited for, so global loads stay in
+// flight across barriers.  The pipeline tail is peeled at compile time: every load
+// of the steady-state loop is unconditional, which lets the compiler count
+// outstanding loads exactly instead of draining the queue once per K step.
+//
+// MFMA: v_mfma_f32_32x32x16_bf16.  Per lane 8 bf16 of each operand (row lane%32,
+// k = 8*(lane/32)..+7), 16 fp32 of the result (column lane%32, rows
+// 8*(i/4) + 4*(lane/32) + i%4).  The weight tile is passed as the FIRST operand
+// and the activation tile as the second, so a lane ends up with four CONSECUTIVE
+// output columns of one output row: epilogues pack them and go through LDS to
+// write 16-byte, fully coalesced rows.
+//
+// LDS layouts (no padding, XOR swizzles; 16-byte chunks):
+//   KC  contraction axis contiguous in HBM: [row][64 k], chunk c of row r stored at
+//       c ^ ((r >> 1) & 7); a fragment is one ds_read_b128 (measured conflict-free;
+//       the key r & 7 costs a 2-way conflict).
+//   KS  contraction axis strided in HBM: [k][cols], chunk c of row k stored at
+//       c ^ ((k & 3) << 1); a fragment is two ds_read_b64_tr_b16 (LDS transpose
+//       reads: lane i of a 16-lane group supplies the address of row i/4, 8-byte
+//       piece i%4, and receives column i of the four rows).
+#include <cstdlib>
+#include <type_traits>
+
 #include "common.h"
 
 namespace mi355 {
@@ -32,28 +54,33 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
-constexpr int BM = 128, BN = 256, BK = 64;
-constexpr int KS_PAD = 32;  // elements; keeps rows 16-byte aligned and shifts banks
+constexpr int BK = 64;
+constexpr int NT = 512;  // threads per workgroup
 
 #define LDS_PTR(p) ((__attribute__((address_space(3))) s16x4*)(p))
 
+// ---- fragment reads -----------------------------------------------------------------
 __device__ __forceinline__ bf16x8 frag_kc(const uint16_t* tile, int row, int kk, int lane) {
   const int r = row + (lane & 31);
   const int c = kk * 2 + (lane >> 5);
-  return *reinterpret_cast<const bf16x8*>(tile + r * BK + ((c ^ (r & 7)) << 3));
+  return *reinterpret_cast<const bf16x8*>(tile + r * BK + ((c ^ ((r >> 1) & 7)) << 3));
 }
 
-__device__ __forceinline__ bf16x8 frag_ks(const uint16_t* tile, int col, int kk, int lane, int pitch) {
+template <int COLS>
+__device__ __forceinline__ bf16x8 frag_ks(const uint16_t* tile, int col, int kk, int lane) {
   const int g = lane >> 4, i = lane & 15;
-  const uint16_t* p = tile + (kk * 16 + 8 * (g >> 1) + (i >> 2)) * pitch + col + 16 * (g & 1) + 4 * (i & 3);
+  const int k = kk * 16 + 8 * (g >> 1) + (i >> 2);  // k & 3 == i >> 2 for both reads
+  const int c = col + 16 * (g & 1) + 4 * (i & 3);
+  const int off = (((c >> 3) ^ ((k & 3) << 1)) << 3) + (c & 7);
+  const uint16_t* p = tile + k * COLS + off;
   const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(p));
-  const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(p + 4 * pitch));
+  const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(p + 4 * COLS));
   const s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
   return __builtin_bit_cast(bf16x8, v);
 }
 
-// block id -> work id such that XCD x (= bid % 8) walks ids [x*chunk, (x+1)*chunk)
 __device__ __forceinline__ int xcd_remap(int bid, int total) {
   const int chunk = (total + 7) >> 3;
   const int within = bid >> 3;
@@ -61,29 +88,37 @@ __device__ __forceinline__ int xcd_remap(int bid, int total) {
   return (within < chunk && pid < total) ? pid : -1;
 }
 
-// One 32x32 accumulator tile of the dh GEMM -> dgate / dup (bf16 rounding after dh,
-// after silu(gate) and after dh*up, like the elementwise ops it replaces).
-__device__ __forceinline__ void dh_epilogue_tile(const f32x16& v, const uint16_t* __restrict__ gate,
-                                                 const uint16_t* __restrict__ up,
-                                                 uint16_t* __restrict__ dgate,
-                                                 uint16_t* __restrict__ dup, int row0, int m_base,
-                                                 int valid, int f, int F) {
-#pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const int m = m_base + (i >> 2) * 8 + (i & 3);
-    if (m < valid && f < F) {
-      const int64_t o = static_cast<int64_t>(row0 + m) * F + f;
-      const float dh = round_bf16(v[i]);
-      const float g = bf16_to_f32(gate[o]);
-      const float u = bf16_to_f32(up[o]);
-      const float sig = 1.0f / (1.0f + __expf(-g));
-      const float s = round_bf16(g * sig);
-      const float ds = round_bf16(dh * u);
-      dup[o] = f32_to_bf16(dh * s);
-      dgate[o] = f32_to_bf16(ds * (sig * (1.0f + g * (1.0f - sig))));
-    }
-  }
+// Barrier between the memory phase and the MFMA phase of the ping-pong schedule: wait
+// for this wave's own LDS operations only (global loads stay in flight), then s_barrier.
+__device__ __forceinline__ void phase_barrier() {
+  __builtin_amdgcn_sched_barrier(0);
+  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
 }
+
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+  return static_cast<uint32_t>(f32_to_bf16(a)) | (static_cast<uint32_t>(f32_to_bf16(b)) << 16);
+}
+
+// ---- epilogue staging -----------------------------------------------------------------
+// A wave parks its 64 x W sub-tile (bf16) in its private LDS region, [64][W + 8], then
+// streams it out as 16-byte row pieces.  acc was produced with the weight fragment as
+// the first MFMA operand: lane = output row (lane & 31), registers = output columns.
+template <int W>
+struct WaveStage {
+  static constexpr int PITCH = W + 8;
+  static constexpr int ELEMS = 64 * PITCH;
+  // element (row m of 64, col n of W) for register i of the accumulator tile (mi, nj-th 32 columns)
+  __device__ static __forceinline__ void put4(uint16_t* st, int mi, int col0, int lane, int q,
+                                              float v0, float v1, float v2, float v3) {
+    const int m = mi * 32 + (lane & 31);
+    const int n = col0 + q * 8 + (lane >> 5) * 4;
+    u32x2 pk = {pack2(v0, v1), pack2(v2, v3)};
+    *reinterpret_cast<u32x2*>(st + m * PITCH + n) = pk;
+  }
+};
+
 
 enum RowMode { RM_GATEUP = 0, RM_DOWN = 1, RM_DH = 2, RM_DX = 3 };
 
@@ -103,103 +138,93 @@ struct RowArgs {
   const int32_t* tile_row0;
   const int32_t* num_tiles;
   int D, F;
-  int n_tiles;  // column tiles per row tile
+  int n_tiles;
 };
 
-template <int MODE>
-__global__ __launch_bounds__(256, 2) void row_tiled_kernel(RowArgs p) {
-  constexpr bool B_KS = (MODE == RM_DH || MODE == RM_DX);
-  constexpr int B_PITCH = BN + KS_PAD;
-  constexpr int B_ELEMS = B_KS ? BK * B_PITCH : BN * BK;
-  __shared__ __attribute__((aligned(16))) uint16_t As[BM * BK];
-  __shared__ __attribute__((aligned(16))) uint16_t Bs[B_ELEMS];
+// Row-tiled kernel: 128 rows of one expert x 512 output columns, 8 waves as 2 (rows) x 4
+// (columns), each wave 64 x 128.  GATEUP's 512 columns are 256 gate + 256 up columns of
+// the same f range, so a wave holds gate and up of the same 64 f.
+constexpr int RBM = 128, RBN = 512;
+constexpr int R_STAGE = (RBM + RBN) * BK;  // elements per LDS stage (80 KiB)
 
-  const int total = *p.num_tiles * p.n_tiles;
+template <int MODE>
+__global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
+  constexpr bool B_KS = (MODE == RM_DH || MODE == RM_DX);
+  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+
+  const int num_tiles = *p.num_tiles;
+  const int total = num_tiles * p.n_tiles;
   const int pid = xcd_remap(blockIdx.x, total);
   if (pid < 0) return;
   const int tile = pid / p.n_tiles, nt = pid % p.n_tiles;
   const int e = p.tile_expert[tile];
   const int row0 = p.tile_row0[tile];
-  const int valid = min(BM, p.seg_offsets[e] + p.seg_counts[e] - row0);
+  const int valid = min(RBM, p.seg_offsets[e] + p.seg_counts[e] - row0);
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = (wave >> 1) * 64, wn = wave & 1;
+  const int wm = (wave >> 2) * 64, wn = wave & 3;
   const int D = p.D, F = p.F;
 
-  // contraction length, leading dims, output width
   const int Kdim = (MODE == RM_GATEUP || MODE == RM_DH) ? D : (MODE == RM_DOWN ? F : 2 * F);
   const int lda = (MODE == RM_GATEUP || MODE == RM_DH) ? D : F;
-  const int Ncols = (MODE == RM_GATEUP || MODE == RM_DH) ? F : D;  // width of the output matrix
-  const int n0 = nt * (MODE == RM_GATEUP ? BN / 2 : BN);
+  const int Ncols = (MODE == RM_GATEUP || MODE == RM_DH) ? F : D;  // output width
+  const int n0 = nt * (MODE == RM_GATEUP ? RBN / 2 : RBN);
   const int64_t wsz = static_cast<int64_t>(D) * F;
   const uint16_t* B0 = p.b0 + e * wsz;
   const uint16_t* B1 = (MODE == RM_GATEUP || MODE == RM_DX) ? p.b1 + e * wsz : B0;
   const int64_t b1_off = B1 - B0;  // both weight stacks live in one flat address space
 
-  // ---- global -> register staging -------------------------------------------
-  // Thread `tid` moves 16-byte chunks q = tid + 256*i.  For KC tiles (8 chunks per
-  // row) that is row (tid>>3) + 32*i, chunk tid&7; for KS tiles (32 chunks per k)
-  // it is k = (tid>>5) + 8*i, chunk tid&31.  Only the clamped row offsets need
-  // per-i storage; everything else is affine in i.
-  u32x4 ra[4], rb[8];
+  // ---- global -> register staging: 16-byte chunks q = tid + 512*i ---------------------
+  // KC tiles (8 chunks per row): row (tid>>3) + 64*i, chunk tid&7.
+  // KS tile (64 chunks per k row of 512 columns): k = (tid>>6) + 8*i, chunk tid&63.
+  u32x4 ra[2], rb[8];
   const int kc_row = tid >> 3, kc_chunk = tid & 7;
-  const int kc_lds = kc_row * BK + ((kc_chunk ^ (kc_row & 7)) << 3);  // + i*32*BK
+  const int kc_lds = kc_row * BK + ((kc_chunk ^ ((kc_row >> 1) & 7)) << 3);  // + i*64*BK (64 % 16 == 0)
   const uint16_t* a_base0 = p.a0 + static_cast<int64_t>(row0) * lda + kc_chunk * 8;
   const uint16_t* a_base1 = (MODE == RM_DX) ? p.a1 + static_cast<int64_t>(row0) * lda + kc_chunk * 8 : a_base0;
-  int a_off[4];
+  int a_off[2];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) a_off[i] = min(kc_row + 32 * i, valid - 1) * lda;
+  for (int i = 0; i < 2; ++i) a_off[i] = min(kc_row + 64 * i, valid - 1) * lda;
 
   const uint16_t* b_base = B0;
   int b_off[8];
-  int b_lds0, b_lds_step;
+  int b_lds[8];
   if constexpr (!B_KS) {
     b_base += kc_chunk * 8;
-    b_lds0 = kc_lds;
-    b_lds_step = 32 * BK;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const int r = kc_row + 32 * i;
+      const int r = kc_row + 64 * i;
       if constexpr (MODE == RM_GATEUP)
-        b_off[i] = min(n0 + (r & 127), F - 1) * D;  // rows 0..127 from w1, 128..255 from w3
+        b_off[i] = min(n0 + (r & 255), F - 1) * D;  // rows 0..255 from w1, 256..511 from w3
       else
         b_off[i] = min(n0 + r, D - 1) * F;  // DOWN: w2[e] is (D,F); a tile row is an output column d
+      b_lds[i] = kc_lds + i * 64 * BK;
     }
   } else {
     // DH: B(k=d, n=f) = w2[e][d][f], ld F.  DX: B(k=f, n=d) = w1/w3[e][f][d], ld D.
-    const int ks_k = tid >> 5, ks_chunk = tid & 31;
-    b_base += static_cast<int64_t>(ks_k) * Ncols + min(n0 + ks_chunk * 8, Ncols - 8);
-    b_lds0 = ks_k * B_PITCH + ks_chunk * 8;
-    b_lds_step = 8 * B_PITCH;
+    const int ks_k = tid >> 6, ks_chunk = tid & 63;
+    b_base += min(n0 + ks_chunk * 8, Ncols - 8);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) b_off[i] = 8 * i * Ncols;
+    for (int i = 0; i < 8; ++i) {
+      const int k = ks_k + 8 * i;
+      b_off[i] = k * Ncols;
+      b_lds[i] = k * RBN + ((ks_chunk ^ ((k & 3) << 1)) << 3);
+    }
   }
 
-#define LOAD_REGS(K0)                                                                          \
-  do {                                                                                         \
-    const int k0_ = (K0);                                                                      \
-    if constexpr (MODE == RM_DX) {                                                             \
-      const bool second = k0_ >= F;                                                            \
-      const int kk0 = second ? k0_ - F : k0_;                                                  \
-      const uint16_t* ab = (second ? a_base1 : a_base0) + kk0;                                 \
-      const uint16_t* bb = b_base + (second ? b1_off : 0) + static_cast<int64_t>(kk0) * Ncols; \
-      _Pragma("unroll") for (int i = 0; i < 4; ++i)                                            \
-          ra[i] = *reinterpret_cast<const u32x4*>(ab + a_off[i]);                              \
-      _Pragma("unroll") for (int i = 0; i < 8; ++i)                                            \
-          rb[i] = *reinterpret_cast<const u32x4*>(bb + b_off[i]);                              \
-    } else {                                                                                   \
-      const uint16_t* ab = a_base0 + k0_;                                                      \
-      const uint16_t* bb = B_KS ? b_base + static_cast<int64_t>(k0_) * Ncols : b_base + k0_;   \
-      _Pragma("unroll") for (int i = 0; i < 4; ++i)                                            \
-          ra[i] = *reinterpret_cast<const u32x4*>(ab + a_off[i]);                              \
-      _Pragma("unroll") for (int i = 0; i < 8; ++i) {                                          \
-        if constexpr (MODE == RM_GATEUP)                                                       \
-          rb[i] = *reinterpret_cast<const u32x4*>(bb + (i >= 4 ? b1_off : 0) + b_off[i]);      \
-        else                                                                                   \
-          rb[i] = *reinterpret_cast<const u32x4*>(bb + b_off[i]);                              \
-      }                                                                                        \
-    }                                                                                          \
-  } while (0)
+  // pointers for the K step being fetched
+  auto a_ptr = [&](int k0) -> const uint16_t* {
+    if constexpr (MODE == RM_DX) return (k0 >= F ? a_base1 + (k0 - F) : a_base0 + k0);
+    return a_base0 + k0;
+  };
+  auto b_ptr = [&](int k0) -> const uint16_t* {
+    if constexpr (MODE == RM_DX) {
+      const int kk0 = k0 >= F ? k0 - F : k0;
+      return b_base + (k0 >= F ? b1_off : 0) + static_cast<int64_t>(kk0) * Ncols;
+    }
+    if constexpr (B_KS) return b_base + static_cast<int64_t>(k0) * Ncols;
+    return b_base + k0;
+  };
 
   f32x16 acc[2][4];
 #pragma unroll
@@ -209,84 +234,204 @@ __global__ __launch_bounds__(256, 2) void row_tiled_kernel(RowArgs p) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[mi][nj][i] = 0.0f;
 
-  // LDS row/column of this wave's four 32-wide column tiles
   int bcol[4];
 #pragma unroll
   for (int nj = 0; nj < 4; ++nj) {
     if constexpr (MODE == RM_GATEUP)
-      bcol[nj] = (nj < 2 ? 0 : 128) + wn * 64 + (nj & 1) * 32;
+      bcol[nj] = (nj < 2 ? 0 : RBN / 2) + wn * 64 + (nj & 1) * 32;
     else
       bcol[nj] = wn * 128 + nj * 32;
   }
 
-  LOAD_REGS(0);
-  for (int k0 = 0; k0 < Kdim; k0 += BK) {
+  const int ksteps = Kdim / BK;
+  auto kofs = [&](int ks) { return ks * BK; };
+  // prologue: tile 0 -> LDS stage 0, tile 1 -> registers
+  {
+    const uint16_t* ab = a_ptr(kofs(0));
+    const uint16_t* bb = b_ptr(kofs(0));
 #pragma unroll
-    for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(As + kc_lds + i * 32 * BK) = ra[i];
+    for (int i = 0; i < 2; ++i) ra[i] = *reinterpret_cast<const u32x4*>(ab + a_off[i]);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(Bs + b_lds0 + i * b_lds_step) = rb[i];
-    __syncthreads();
-    if (k0 + BK < Kdim) LOAD_REGS(k0 + BK);
+    for (int i = 0; i < 8; ++i) {
+      const int64_t x = (MODE == RM_GATEUP && i >= 4) ? b1_off : 0;
+      rb[i] = *reinterpret_cast<const u32x4*>(bb + x + b_off[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) *reinterpret_cast<u32x4*>(smem + kc_lds + i * 64 * BK) = ra[i];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(smem + RBM * BK + b_lds[i]) = rb[i];
+    if (ksteps > 1) {
+      const uint16_t* ab1 = a_ptr(kofs(1));
+      const uint16_t* bb1 = b_ptr(kofs(1));
+#pragma unroll
+      for (int i = 0; i < 2; ++i) ra[i] = *reinterpret_cast<const u32x4*>(ab1 + a_off[i]);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int64_t x = (MODE == RM_GATEUP && i >= 4) ? b1_off : 0;
+        rb[i] = *reinterpret_cast<const u32x4*>(bb1 + x + b_off[i]);
+      }
+    }
+  }
+  __syncthreads();
+
+  // One K step.  HAS_NEXT: the registers hold tile ks+1 and are parked in the other LDS
+  // stage.  HAS_NEXT2: tile ks+2 is fetched into the registers.  Both are compile-time
+  // so that every load of the steady-state loop is unconditional: the compiler can then
+  // count outstanding loads exactly and wait only for the three oldest before each park,
+  // instead of draining the queue (vmcnt(0)) once per K step.
+  auto kstep = [&](int ks, auto has_next_t, auto has_next2_t) {
+    constexpr bool has_next = decltype(has_next_t)::value;
+    constexpr bool has_next2 = decltype(has_next2_t)::value;
+    const uint16_t* As = smem + (ks & 1) * R_STAGE;
+    const uint16_t* Bs = As + RBM * BK;
+    uint16_t* An = smem + ((ks + 1) & 1) * R_STAGE;
+    uint16_t* Bn = An + RBM * BK;
+    const uint16_t* ab2 = has_next2 ? a_ptr(kofs(ks + 2)) : nullptr;
+    const uint16_t* bb2 = has_next2 ? b_ptr(kofs(ks + 2)) : nullptr;
 #pragma unroll
     for (int kk = 0; kk < BK / 16; ++kk) {
+      // a quarter of the staging traffic rides along with each quarter of the MFMAs:
+      // park the held chunks of tile ks+1 in the other LDS stage, then refill the
+      // same registers with the same chunks of tile ks+2.
+      if constexpr (has_next) {
+        if (kk < 2) *reinterpret_cast<u32x4*>(An + kc_lds + kk * 64 * BK) = ra[kk];
+        *reinterpret_cast<u32x4*>(Bn + b_lds[2 * kk]) = rb[2 * kk];
+        *reinterpret_cast<u32x4*>(Bn + b_lds[2 * kk + 1]) = rb[2 * kk + 1];
+      }
+      if constexpr (has_next2) {
+        if (kk < 2) ra[kk] = *reinterpret_cast<const u32x4*>(ab2 + a_off[kk]);
+        const int64_t x = (MODE == RM_GATEUP && kk >= 2) ? b1_off : 0;
+        rb[2 * kk] = *reinterpret_cast<const u32x4*>(bb2 + x + b_off[2 * kk]);
+        rb[2 * kk + 1] = *reinterpret_cast<const u32x4*>(bb2 + x + b_off[2 * kk + 1]);
+      }
       bf16x8 af[2], bf[4];
 #pragma unroll
       for (int mi = 0; mi < 2; ++mi) af[mi] = frag_kc(As, wm + mi * 32, kk, lane);
 #pragma unroll
       for (int nj = 0; nj < 4; ++nj) {
         if constexpr (B_KS)
-          bf[nj] = frag_ks(Bs, bcol[nj], kk, lane, B_PITCH);
+          bf[nj] = frag_ks<RBN>(Bs, bcol[nj], kk, lane);
         else
           bf[nj] = frag_kc(Bs, bcol[nj], kk, lane);
       }
+      // end of the memory phase: this wave's LDS traffic has landed; swap roles with the
+      // sibling group, which has just finished issuing its MFMAs
+      phase_barrier();
 #pragma unroll
       for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
         for (int nj = 0; nj < 4; ++nj)
-          acc[mi][nj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[mi], bf[nj], acc[mi][nj], 0, 0, 0);
+          acc[mi][nj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[nj], af[mi], acc[mi][nj], 0, 0, 0);
+      phase_barrier();
     }
-    __syncthreads();
-  }
+  };
+  using T_ = std::true_type;
+  using F_ = std::false_type;
+  // Ping-pong: waves 4..7 run one phase behind waves 0..3 (wave w and w+4 share a SIMD),
+  // so each SIMD always has one wave in its MFMA phase while the other parks, fetches
+  // and reads fragments.  Every wave executes the same number of barriers.
+  if (wave >= 4) phase_barrier();
+  int ks = 0;
+  for (; ks + 2 < ksteps; ++ks) kstep(ks, T_{}, T_{});
+  if (ks + 1 < ksteps) { kstep(ks, T_{}, F_{}); ++ks; }
+  if (ks < ksteps) kstep(ks, F_{}, F_{});
+  if (wave < 4) phase_barrier();
+  __syncthreads();
 
-  // ---- epilogue -----------------------------------------------------------------
-#undef LOAD_REGS
-  const int ln = lane & 31, lh = lane >> 5;
-  if constexpr (MODE == RM_DH) {
-    // SwiGLU backward on the accumulators: dgate = dh*up*silu'(gate), dup = dh*silu(gate)
-#define DH_TILE(MI, NJ) \
-  dh_epilogue_tile(acc[MI][NJ], p.gate, p.up, p.o0, p.o1, row0, wm + MI * 32 + lh * 4, valid, \
-                   n0 + wn * 128 + NJ * 32 + ln, F)
-    DH_TILE(0, 0); DH_TILE(0, 1); DH_TILE(0, 2); DH_TILE(0, 3);
-    DH_TILE(1, 0); DH_TILE(1, 1); DH_TILE(1, 2); DH_TILE(1, 3);
-#undef DH_TILE
-    return;
-  }
+  // ---- epilogue: through the wave's private LDS region, 16-byte coalesced rows ---------
+  // acc[mi][nj][i]: output row = wm + mi*32 + (lane&31); output column within the nj-th
+  // 32-column group = (i>>2)*8 + (lane>>5)*4 + (i&3).
+  uint16_t* st = smem + wave * (64 * 136);  // 8 waves x 17 KiB < 160 KiB; the barrier ending the K loop freed the tiles
+  if constexpr (MODE == RM_GATEUP) {
+    // per 32-row half: three 32 x 64 tiles gate | up | h at columns 0, 64, 128 of a
+    // [32][192+8] region (12.5 KiB per wave)
+    using S = WaveStage<192>;
+    uint16_t* sg = smem + wave * (32 * S::PITCH);
+    const int f0 = n0 + wn * 64;
 #pragma unroll
-  for (int mi = 0; mi < 2; ++mi) {
+    for (int mi = 0; mi < 2; ++mi) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int m = wm + mi * 32 + (i >> 2) * 8 + lh * 4 + (i & 3);
-      const bool row_ok = m < valid;
-      const int64_t r = row0 + m;
-      if constexpr (MODE == RM_GATEUP) {
+      for (int j = 0; j < 2; ++j)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          const int f = n0 + wn * 64 + j * 32 + ln;
-          if (row_ok && f < F) {
-            const uint16_t gb = f32_to_bf16(acc[mi][j][i]);
-            const uint16_t ub = f32_to_bf16(acc[mi][j + 2][i]);
-            const float g = bf16_to_f32(gb);
-            const float s = round_bf16(g / (1.0f + __expf(-g)));
-            p.o0[r * F + f] = gb;
-            p.o1[r * F + f] = ub;
-            p.o2[r * F + f] = f32_to_bf16(s * bf16_to_f32(ub));
+        for (int q = 0; q < 4; ++q) {
+          float g[4], u[4], h[4];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            g[r] = round_bf16(acc[mi][j][q * 4 + r]);
+            u[r] = round_bf16(acc[mi][j + 2][q * 4 + r]);
+            const float s = round_bf16(g[r] / (1.0f + __expf(-g[r])));
+            h[r] = s * u[r];
           }
+          S::put4(sg, 0, j * 32, lane, q, g[0], g[1], g[2], g[3]);
+          S::put4(sg, 0, 64 + j * 32, lane, q, u[0], u[1], u[2], u[3]);
+          S::put4(sg, 0, 128 + j * 32, lane, q, h[0], h[1], h[2], h[3]);
         }
-      } else {
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the wave's own LDS writes have landed
+      __builtin_amdgcn_wave_barrier();
+      // 32 rows x 3 tiles x 8 chunks = 768 chunks, 12 per lane
+#pragma unroll 4
+      for (int it = 0; it < 12; ++it) {
+        const int idx = it * 64 + lane;
+        const int m = idx / 24, rem = idx % 24, t = rem >> 3, c = rem & 7;
+        const int f = f0 + c * 8;
+        const int mr = wm + mi * 32 + m;
+        if (mr < valid && f < F) {
+          const u32x4 v = *reinterpret_cast<const u32x4*>(sg + m * S::PITCH + t * 64 + c * 8);
+          uint16_t* dst = (t == 0 ? p.o0 : (t == 1 ? p.o1 : p.o2)) + static_cast<int64_t>(row0 + mr) * F + f;
+          *reinterpret_cast<u32x4*>(dst) = v;
+        }
+      }
+      __builtin_amdgcn_s_waitcnt(0xc07f);
+      __builtin_amdgcn_wave_barrier();
+    }
+  } else {
+    using S = WaveStage<128>;
 #pragma unroll
-        for (int nj = 0; nj < 4; ++nj) {
-          const int d = n0 + wn * 128 + nj * 32 + ln;
-          if (row_ok && d < D) p.o0[r * D + d] = f32_to_bf16(acc[mi][nj][i]);
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+      for (int nj = 0; nj < 4; ++nj)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          S::put4(st, mi, nj * 32, lane, q, acc[mi][nj][q * 4], acc[mi][nj][q * 4 + 1],
+                  acc[mi][nj][q * 4 + 2], acc[mi][nj][q * 4 + 3]);
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __builtin_amdgcn_wave_barrier();
+    const int c0 = n0 + wn * 128;
+    // 64 rows x 16 chunks = 1024 chunks, 16 per lane; a row's 256 bytes go out contiguously
+#pragma unroll 4
+    for (int it = 0; it < 16; ++it) {
+      const int idx = it * 64 + lane;
+      const int m = idx >> 4, c = idx & 15;
+      const int n = c0 + c * 8;
+      if (wm + m < valid && n < Ncols) {
+        const u32x4 v = *reinterpret_cast<const u32x4*>(st + m * S::PITCH + c * 8);
+        const int64_t o = static_cast<int64_t>(row0 + wm + m) * Ncols + n;
+        if constexpr (MODE == RM_DH) {
+          // SwiGLU backward on 8 consecutive f: dgate = dh*up*silu'(gate), dup = dh*silu(gate)
+          const u32x4 gv = *reinterpret_cast<const u32x4*>(p.gate + o);
+          const u32x4 uv = *reinterpret_cast<const u32x4*>(p.up + o);
+          u32x4 dg, du;
+#pragma unroll
+          for (int w = 0; w < 4; ++w) {
+            float r_dg[2], r_du[2];
+#pragma unroll
+            for (int hlf = 0; hlf < 2; ++hlf) {
+              const float dh = __uint_as_float(hlf ? (v[w] & 0xffff0000u) : (v[w] << 16));
+              const float g = __uint_as_float(hlf ? (gv[w] & 0xffff0000u) : (gv[w] << 16));
+              const float u = __uint_as_float(hlf ? (uv[w] & 0xffff0000u) : (uv[w] << 16));
+              const float sig = 1.0f / (1.0f + __expf(-g));
+              const float s = round_bf16(g * sig);
+              const float ds = round_bf16(dh * u);
+              r_du[hlf] = dh * s;
+              r_dg[hlf] = ds * (sig * (1.0f + g * (1.0f - sig)));
+            }
+            dg[w] = pack2(r_dg[0], r_dg[1]);
+            du[w] = pack2(r_du[0], r_du[1]);
+          }
+          *reinterpret_cast<u32x4*>(p.o0 + o) = dg;
+          *reinterpret_cast<u32x4*>(p.o1 + o) = du;
+        } else {
+          *reinterpret_cast<u32x4*>(p.o0 + o) = v;
         }
       }
     }
@@ -294,6 +439,10 @@ __global__ __launch_bounds__(256, 2) void row_tiled_kernel(RowArgs p) {
 }
 
 // ---- weight gradients: C[e](M,N) = sum_{r in segment e} A[r][m] * B[r][n] ----------
+// 256 x 256 output tile, 8 waves as 4 (m) x 2 (n), each wave 64 x 128; both operands KS.
+constexpr int WBM = 256, WBN = 256;
+constexpr int W_STAGE = (WBM + WBN) * BK;  // 64 KiB
+
 struct WgradArgs {
   const uint16_t* a;  // (rows, M) row-major
   const uint16_t* b;  // (rows, N) row-major
@@ -305,52 +454,33 @@ struct WgradArgs {
   int total;  // El * m_tiles * n_tiles
 };
 
-__global__ __launch_bounds__(256, 2) void wgrad_kernel(WgradArgs p) {
-  constexpr int A_PITCH = BM + KS_PAD, B_PITCH = BN + KS_PAD;
-  __shared__ __attribute__((aligned(16))) uint16_t As[BK * A_PITCH];
-  __shared__ __attribute__((aligned(16))) uint16_t Bs[BK * B_PITCH];
-
-  const int per_e = p.m_tiles * p.n_tiles;
+__global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
   const int pid = xcd_remap(blockIdx.x, p.total);
   if (pid < 0) return;
+  const int per_e = p.m_tiles * p.n_tiles;
   const int e = pid / per_e;
   const int rem = pid % per_e;
   const int mt = rem / p.n_tiles, nt = rem % p.n_tiles;
-  const int m0 = mt * BM, n0 = nt * BN;
+  const int m0 = mt * WBM, n0 = nt * WBN;
   const int M = p.M, N = p.N;
   const int seg0 = p.seg_offsets[e], cnt = p.seg_counts[e];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = (wave >> 1) * 64, wn = (wave & 1) * 128;
 
-  u32x4 ra[4], rb[8];
-  int a_k[4], a_c[4], b_k[8], b_c[8];
-  const uint16_t* a_ptr[4];
-  const uint16_t* b_ptr[8];
+  // KS tiles of 256 columns = 32 chunks per k row: k = (tid>>5) + 16*i, chunk tid&31
+  u32x4 ra[4], rb[4];
+  const int ks_k = tid >> 5, ks_chunk = tid & 31;
+  const uint16_t* a_base = p.a + static_cast<int64_t>(seg0) * M + min(m0 + ks_chunk * 8, M - 8);
+  const uint16_t* b_base = p.b + static_cast<int64_t>(seg0) * N + min(n0 + ks_chunk * 8, N - 8);
+  int lds_off[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int q = tid + 256 * i;
-    a_k[i] = q >> 4;
-    a_c[i] = q & 15;
-    a_ptr[i] = p.a + static_cast<int64_t>(seg0 + a_k[i]) * M + min(m0 + a_c[i] * 8, M - 8);
+    const int k = ks_k + 16 * i;
+    lds_off[i] = k * 256 + ((ks_chunk ^ ((k & 3) << 1)) << 3);
   }
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int q = tid + 256 * i;
-    b_k[i] = q >> 5;
-    b_c[i] = q & 31;
-    b_ptr[i] = p.b + static_cast<int64_t>(seg0 + b_k[i]) * N + min(n0 + b_c[i] * 8, N - 8);
-  }
-  auto load_regs = [&](int k0) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      ra[i] = (k0 + a_k[i] < cnt) ? *reinterpret_cast<const u32x4*>(a_ptr[i] + static_cast<int64_t>(k0) * M)
-                                  : u32x4{0, 0, 0, 0};
-#pragma unroll
-    for (int i = 0; i < 8; ++i)
-      rb[i] = (k0 + b_k[i] < cnt) ? *reinterpret_cast<const u32x4*>(b_ptr[i] + static_cast<int64_t>(k0) * N)
-                                  : u32x4{0, 0, 0, 0};
-  };
+  const u32x4 zero = {0, 0, 0, 0};
 
   f32x16 acc[2][4];
 #pragma unroll
@@ -360,115 +490,179 @@ __global__ __launch_bounds__(256, 2) void wgrad_kernel(WgradArgs p) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[mi][nj][i] = 0.0f;
 
-  if (cnt > 0) load_regs(0);
-  for (int k0 = 0; k0 < cnt; k0 += BK) {
+  const int ksteps = (cnt + BK - 1) / BK;
+  if (ksteps > 0) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(As + a_k[i] * A_PITCH + a_c[i] * 8) = ra[i];
+    for (int i = 0; i < 4; ++i) {
+      const int k = ks_k + 16 * i;
+      ra[i] = k < cnt ? *reinterpret_cast<const u32x4*>(a_base + static_cast<int64_t>(k) * M) : zero;
+      rb[i] = k < cnt ? *reinterpret_cast<const u32x4*>(b_base + static_cast<int64_t>(k) * N) : zero;
+    }
 #pragma unroll
-    for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(Bs + b_k[i] * B_PITCH + b_c[i] * 8) = rb[i];
-    __syncthreads();
-    if (k0 + BK < cnt) load_regs(k0 + BK);
+    for (int i = 0; i < 4; ++i) {
+      *reinterpret_cast<u32x4*>(smem + lds_off[i]) = ra[i];
+      *reinterpret_cast<u32x4*>(smem + WBM * BK + lds_off[i]) = rb[i];
+    }
+    if (ksteps > 1) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int k = BK + ks_k + 16 * i;
+        ra[i] = k < cnt ? *reinterpret_cast<const u32x4*>(a_base + static_cast<int64_t>(k) * M) : zero;
+        rb[i] = k < cnt ? *reinterpret_cast<const u32x4*>(b_base + static_cast<int64_t>(k) * N) : zero;
+      }
+    }
+  }
+  __syncthreads();
+
+  // The K extent here is one expert's rows (a handful of 64-row steps), so the loop is
+  // kept simple: one barrier per step, next tile parked and the one after fetched while
+  // the MFMAs of the current tile issue.
+  for (int ks = 0; ks < ksteps; ++ks) {
+    const uint16_t* As = smem + (ks & 1) * W_STAGE;
+    const uint16_t* Bs = As + WBM * BK;
+    uint16_t* An = smem + ((ks + 1) & 1) * W_STAGE;
+    uint16_t* Bn = An + WBM * BK;
+    const bool has_next = ks + 1 < ksteps;
+    const bool has_next2 = ks + 2 < ksteps;
+    const int kbase2 = (ks + 2) * BK;
 #pragma unroll
     for (int kk = 0; kk < BK / 16; ++kk) {
+      if (has_next) {
+        *reinterpret_cast<u32x4*>(An + lds_off[kk]) = ra[kk];
+        *reinterpret_cast<u32x4*>(Bn + lds_off[kk]) = rb[kk];
+      }
+      if (has_next2) {
+        const int k = kbase2 + ks_k + 16 * kk;
+        ra[kk] = k < cnt ? *reinterpret_cast<const u32x4*>(a_base + static_cast<int64_t>(k) * M) : zero;
+        rb[kk] = k < cnt ? *reinterpret_cast<const u32x4*>(b_base + static_cast<int64_t>(k) * N) : zero;
+      }
       bf16x8 af[2], bf[4];
 #pragma unroll
-      for (int mi = 0; mi < 2; ++mi) af[mi] = frag_ks(As, wm + mi * 32, kk, lane, A_PITCH);
+      for (int mi = 0; mi < 2; ++mi) af[mi] = frag_ks<256>(As, wm + mi * 32, kk, lane);
 #pragma unroll
-      for (int nj = 0; nj < 4; ++nj) bf[nj] = frag_ks(Bs, wn + nj * 32, kk, lane, B_PITCH);
+      for (int nj = 0; nj < 4; ++nj) bf[nj] = frag_ks<256>(Bs, wn + nj * 32, kk, lane);
 #pragma unroll
       for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
         for (int nj = 0; nj < 4; ++nj)
-          acc[mi][nj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[mi], bf[nj], acc[mi][nj], 0, 0, 0);
+          acc[mi][nj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[nj], af[mi], acc[mi][nj], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
     __syncthreads();
   }
 
-  uint16_t* C = p.c + static_cast<int64_t>(e) * M * N;
-  const int ln = lane & 31, lh = lane >> 5;
+  using S = WaveStage<128>;
+  uint16_t* st = smem + wave * S::ELEMS;
 #pragma unroll
   for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int m = m0 + wm + mi * 32 + (i >> 2) * 8 + lh * 4 + (i & 3);
-      if (m >= M) continue;
+    for (int nj = 0; nj < 4; ++nj)
 #pragma unroll
-      for (int nj = 0; nj < 4; ++nj) {
-        const int n = n0 + wn + nj * 32 + ln;
-        if (n < N) C[static_cast<int64_t>(m) * N + n] = f32_to_bf16(acc[mi][nj][i]);
-      }
-    }
+      for (int q = 0; q < 4; ++q)
+        S::put4(st, mi, nj * 32, lane, q, acc[mi][nj][q * 4], acc[mi][nj][q * 4 + 1],
+                acc[mi][nj][q * 4 + 2], acc[mi][nj][q * 4 + 3]);
+  __builtin_amdgcn_s_waitcnt(0xc07f);
+  __builtin_amdgcn_wave_barrier();
+  uint16_t* C = p.c + static_cast<int64_t>(e) * M * N;
+#pragma unroll 4
+  for (int it = 0; it < 16; ++it) {
+    const int idx = it * 64 + lane;
+    const int m = m0 + wm + (idx >> 4), n = n0 + wn + (idx & 15) * 8;
+    if (m < M && n < N)
+      *reinterpret_cast<u32x4*>(C + static_cast<int64_t>(m) * N + n) =
+          *reinterpret_cast<const u32x4*>(st + (idx >> 4) * S::PITCH + (idx & 15) * 8);
+  }
+}
+
+template <typename K>
+int set_lds(K kernel, int bytes) {
+  const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  return e == hipSuccess ? MI355_OK : fail(MI355_ELAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
 }
 
 }  // namespace
 
-// ---- host side (called from grouped.hip) ---------------------------------------------
-// `stages` is a mask of MI355_STAGE_* bits: which of the seven GEMM kernels to launch.
-enum { STAGE_GATEUP = 1, STAGE_DOWN = 2, STAGE_DH = 4, STAGE_DX = 8, STAGE_DW2 = 16, STAGE_DW1 = 32, STAGE_DW3 = 64 };
+// The MFMA path needs whole 64-wide K steps and 16-byte aligned rows.
 bool bf16_fast_path_ok(int64_t D, int64_t F) { return D % 64 == 0 && F % 64 == 0 && D >= 64 && F >= 64; }
+
+enum { STAGE_GATEUP = 1, STAGE_DOWN = 2, STAGE_DH = 4, STAGE_DX = 8, STAGE_DW2 = 16, STAGE_DW1 = 32, STAGE_DW3 = 64 };
 
 static unsigned round8(int64_t v) { return static_cast<unsigned>((v + 7) / 8 * 8); }
 
+constexpr int R_LDS_BYTES = 2 * R_STAGE * 2;  // 163840
+constexpr int W_LDS_BYTES = 8 * 64 * 136 * 2;  // 139264: the 8 epilogue regions (> 2 stages = 131072)
+
+template <int MODE>
+static int launch_row(RowArgs& a, int64_t tile_capacity, hipStream_t s, const char* what) {
+  static bool configured = false;  // per process; the attribute is per function
+  if (!configured) {
+    if (int rc = set_lds(row_tiled_kernel<MODE>, R_LDS_BYTES)) return rc;
+    configured = true;
+  }
+  hipLaunchKernelGGL(row_tiled_kernel<MODE>, dim3(round8(tile_capacity * a.n_tiles)), dim3(NT), R_LDS_BYTES, s, a);
+  return check_launch(what);
+}
+
 int bf16_grouped_fwd(const void* rows, const void* w1, const void* w3, const void* w2,
-                     const int32_t* seg_offsets, const int32_t* seg_counts,
-                     const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* num_tiles,
-                     int64_t tile_capacity, void* gate, void* up, void* h, void* y, int64_t D,
-                     int64_t F, int stages, hipStream_t s) {
+                       const int32_t* seg_offsets, const int32_t* seg_counts,
+                       const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* num_tiles,
+                       int64_t tile_capacity, void* gate, void* up, void* h, void* y, int64_t D,
+                       int64_t F, int stages, hipStream_t s) {
   RowArgs a{};
   a.seg_offsets = seg_offsets; a.seg_counts = seg_counts; a.tile_expert = tile_expert;
   a.tile_row0 = tile_row0; a.num_tiles = num_tiles; a.D = (int)D; a.F = (int)F;
-  a.a0 = (const uint16_t*)rows; a.b0 = (const uint16_t*)w1; a.b1 = (const uint16_t*)w3;
-  a.o0 = (uint16_t*)gate; a.o1 = (uint16_t*)up; a.o2 = (uint16_t*)h;
-  a.n_tiles = (int)((F + BN / 2 - 1) / (BN / 2));
   if (stages & STAGE_GATEUP) {
-    hipLaunchKernelGGL(row_tiled_kernel<RM_GATEUP>, dim3(round8(tile_capacity * a.n_tiles)), dim3(256), 0, s, a);
-    if (int rc = check_launch("grouped gate/up")) return rc;
+    a.a0 = (const uint16_t*)rows; a.b0 = (const uint16_t*)w1; a.b1 = (const uint16_t*)w3;
+    a.o0 = (uint16_t*)gate; a.o1 = (uint16_t*)up; a.o2 = (uint16_t*)h;
+    a.n_tiles = (int)((F + RBN / 2 - 1) / (RBN / 2));
+    if (int rc = launch_row<RM_GATEUP>(a, tile_capacity, s, "grouped gate/up")) return rc;
   }
-  if (!(stages & STAGE_DOWN)) return MI355_OK;
-  RowArgs b{};
-  b.seg_offsets = seg_offsets; b.seg_counts = seg_counts; b.tile_expert = tile_expert;
-  b.tile_row0 = tile_row0; b.num_tiles = num_tiles; b.D = (int)D; b.F = (int)F;
-  b.a0 = (const uint16_t*)h; b.b0 = (const uint16_t*)w2; b.o0 = (uint16_t*)y;
-  b.n_tiles = (int)((D + BN - 1) / BN);
-  hipLaunchKernelGGL(row_tiled_kernel<RM_DOWN>, dim3(round8(tile_capacity * b.n_tiles)), dim3(256), 0, s, b);
-  return check_launch("grouped down");
+  if (stages & STAGE_DOWN) {
+    RowArgs b = a;
+    b.a0 = (const uint16_t*)h; b.b0 = (const uint16_t*)w2; b.o0 = (uint16_t*)y;
+    b.n_tiles = (int)((D + RBN - 1) / RBN);
+    if (int rc = launch_row<RM_DOWN>(b, tile_capacity, s, "grouped down")) return rc;
+  }
+  return MI355_OK;
 }
 
 int bf16_grouped_bwd(const void* dy, const void* rows, const void* w1, const void* w3,
-                     const void* w2, const void* gate, const void* up, const void* h,
-                     const int32_t* seg_offsets, const int32_t* seg_counts,
-                     const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* num_tiles,
-                     int64_t tile_capacity, void* dgate, void* dup, void* drows, void* dw1,
-                     void* dw3, void* dw2, int64_t El, int64_t D, int64_t F, int stages,
-                     hipStream_t s) {
+                       const void* w2, const void* gate, const void* up, const void* h,
+                       const int32_t* seg_offsets, const int32_t* seg_counts,
+                       const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* num_tiles,
+                       int64_t tile_capacity, void* dgate, void* dup, void* drows, void* dw1,
+                       void* dw3, void* dw2, int64_t El, int64_t D, int64_t F, int stages,
+                       hipStream_t s) {
   RowArgs a{};
   a.seg_offsets = seg_offsets; a.seg_counts = seg_counts; a.tile_expert = tile_expert;
   a.tile_row0 = tile_row0; a.num_tiles = num_tiles; a.D = (int)D; a.F = (int)F;
-  a.a0 = (const uint16_t*)dy; a.b0 = (const uint16_t*)w2;
-  a.gate = (const uint16_t*)gate; a.up = (const uint16_t*)up;
-  a.o0 = (uint16_t*)dgate; a.o1 = (uint16_t*)dup;
-  a.n_tiles = (int)((F + BN - 1) / BN);
   if (stages & STAGE_DH) {
-    hipLaunchKernelGGL(row_tiled_kernel<RM_DH>, dim3(round8(tile_capacity * a.n_tiles)), dim3(256), 0, s, a);
-    if (int rc = check_launch("grouped dh")) return rc;
+    a.a0 = (const uint16_t*)dy; a.b0 = (const uint16_t*)w2;
+    a.gate = (const uint16_t*)gate; a.up = (const uint16_t*)up;
+    a.o0 = (uint16_t*)dgate; a.o1 = (uint16_t*)dup;
+    a.n_tiles = (int)((F + RBN - 1) / RBN);
+    if (int rc = launch_row<RM_DH>(a, tile_capacity, s, "grouped dh")) return rc;
   }
   if (drows && (stages & STAGE_DX)) {
-    RowArgs b{};
-    b.seg_offsets = seg_offsets; b.seg_counts = seg_counts; b.tile_expert = tile_expert;
-    b.tile_row0 = tile_row0; b.num_tiles = num_tiles; b.D = (int)D; b.F = (int)F;
+    RowArgs b = a;
     b.a0 = (const uint16_t*)dgate; b.a1 = (const uint16_t*)dup;
     b.b0 = (const uint16_t*)w1; b.b1 = (const uint16_t*)w3; b.o0 = (uint16_t*)drows;
-    b.n_tiles = (int)((D + BN - 1) / BN);
-    hipLaunchKernelGGL(row_tiled_kernel<RM_DX>, dim3(round8(tile_capacity * b.n_tiles)), dim3(256), 0, s, b);
-    if (int rc = check_launch("grouped drows")) return rc;
+    b.n_tiles = (int)((D + RBN - 1) / RBN);
+    if (int rc = launch_row<RM_DX>(b, tile_capacity, s, "grouped drows")) return rc;
+  }
+  static bool wconfigured = false;
+  if (!wconfigured) {
+    if (int rc = set_lds(wgrad_kernel, W_LDS_BYTES)) return rc;
+    wconfigured = true;
   }
   auto wgrad = [&](const void* A, const void* B, void* C, int64_t M, int64_t N, const char* what) {
     WgradArgs w{};
     w.a = (const uint16_t*)A; w.b = (const uint16_t*)B; w.c = (uint16_t*)C;
     w.seg_offsets = seg_offsets; w.seg_counts = seg_counts; w.M = (int)M; w.N = (int)N;
-    w.m_tiles = (int)((M + BM - 1) / BM); w.n_tiles = (int)((N + BN - 1) / BN);
+    w.m_tiles = (int)((M + WBM - 1) / WBM); w.n_tiles = (int)((N + WBN - 1) / WBN);
     w.total = (int)(El * w.m_tiles * w.n_tiles);
-    hipLaunchKernelGGL(wgrad_kernel, dim3(round8(w.total)), dim3(256), 0, s, w);
+    hipLaunchKernelGGL(wgrad_kernel, dim3(round8(w.total)), dim3(NT), W_LDS_BYTES, s, w);
     return check_launch(what);
   };
   if (dw2 && (stages & STAGE_DW2)) if (int rc = wgrad(dy, h, dw2, D, F, "grouped dw2")) return rc;
@@ -478,3 +672,4 @@ int bf16_grouped_bwd(const void* dy, const void* rows, const void* w1, const voi
 }
 
 }  // namespace mi355
+
