@@ -296,6 +296,7 @@ def test_grouped_experts_bf16_generic_shapes(ops, counts, D, Fd):
 @pytest.mark.parametrize("counts,D,Fd", [
     ((128, 128), 64, 64), ((5, 6, 4, 7), 128, 64), ((200, 0, 129, 1, 300), 256, 192),
     ((0, 0, 0), 64, 128), ((513, 77), 512, 320), ((1000,), 256, 768),
+    ((200, 0, 129), 384, 768), ((131, 260), 768, 384),
 ])
 def test_grouped_experts_bf16_mfma(ops, counts, D, Fd):
     print(f"experts bf16 mfma {counts} D={D} F={Fd}", flush=True)

@@ -147,8 +147,11 @@ struct RowArgs {
 constexpr int RBM = 128, RBN = 512;
 constexpr int R_STAGE = (RBM + RBN) * BK;  // elements per LDS stage (80 KiB)
 
-template <int MODE>
+template <int MODE, int NJ>
 __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
+  constexpr int BNT = 128 * NJ;            // output columns of the tile (4 waves x NJ x 32)
+  constexpr int NB = BNT / 64;             // 16-byte B chunks staged per thread and K step
+  constexpr int STAGE = (RBM + BNT) * BK;  // elements per LDS stage
   constexpr bool B_KS = (MODE == RM_DH || MODE == RM_DX);
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
 
@@ -168,7 +171,7 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
   const int Kdim = (MODE == RM_GATEUP || MODE == RM_DH) ? D : (MODE == RM_DOWN ? F : 2 * F);
   const int lda = (MODE == RM_GATEUP || MODE == RM_DH) ? D : F;
   const int Ncols = (MODE == RM_GATEUP || MODE == RM_DH) ? F : D;  // output width
-  const int n0 = nt * (MODE == RM_GATEUP ? RBN / 2 : RBN);
+  const int n0 = nt * (MODE == RM_GATEUP ? BNT / 2 : BNT);
   const int64_t wsz = static_cast<int64_t>(D) * F;
   const uint16_t* B0 = p.b0 + e * wsz;
   const uint16_t* B1 = (MODE == RM_GATEUP || MODE == RM_DX) ? p.b1 + e * wsz : B0;
@@ -176,8 +179,8 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
 
   // ---- global -> register staging: 16-byte chunks q = tid + 512*i ---------------------
   // KC tiles (8 chunks per row): row (tid>>3) + 64*i, chunk tid&7.
-  // KS tile (64 chunks per k row of 512 columns): k = (tid>>6) + 8*i, chunk tid&63.
-  u32x4 ra[2], rb[8];
+  // KS tile (BNT/8 chunks per k row): chunk q -> k = q / (BNT/8), chunk q % (BNT/8).
+  u32x4 ra[2], rb[NB];
   const int kc_row = tid >> 3, kc_chunk = tid & 7;
   const int kc_lds = kc_row * BK + ((kc_chunk ^ ((kc_row >> 1) & 7)) << 3);  // + i*64*BK (64 % 16 == 0)
   const uint16_t* a_base0 = p.a0 + static_cast<int64_t>(row0) * lda + kc_chunk * 8;
@@ -187,28 +190,29 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
   for (int i = 0; i < 2; ++i) a_off[i] = min(kc_row + 64 * i, valid - 1) * lda;
 
   const uint16_t* b_base = B0;
-  int b_off[8];
-  int b_lds[8];
+  int b_off[NB];
+  int b_lds[NB];
   if constexpr (!B_KS) {
     b_base += kc_chunk * 8;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < NB; ++i) {
       const int r = kc_row + 64 * i;
       if constexpr (MODE == RM_GATEUP)
-        b_off[i] = min(n0 + (r & 255), F - 1) * D;  // rows 0..255 from w1, 256..511 from w3
+        b_off[i] = min(n0 + (r % (BNT / 2)), F - 1) * D;  // first half of the rows from w1, second from w3
       else
         b_off[i] = min(n0 + r, D - 1) * F;  // DOWN: w2[e] is (D,F); a tile row is an output column d
       b_lds[i] = kc_lds + i * 64 * BK;
     }
   } else {
     // DH: B(k=d, n=f) = w2[e][d][f], ld F.  DX: B(k=f, n=d) = w1/w3[e][f][d], ld D.
-    const int ks_k = tid >> 6, ks_chunk = tid & 63;
-    b_base += min(n0 + ks_chunk * 8, Ncols - 8);
+    // (b_off carries both the k row and the clamped column of each chunk)
+    constexpr int CPR = BNT / 8;  // chunks per k row
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int k = ks_k + 8 * i;
-      b_off[i] = k * Ncols;
-      b_lds[i] = k * RBN + ((ks_chunk ^ ((k & 3) << 1)) << 3);
+    for (int i = 0; i < NB; ++i) {
+      const int q = tid + NT * i;
+      const int k = q / CPR, cc = q % CPR;
+      b_off[i] = k * Ncols + min(n0 + cc * 8, Ncols - 8);
+      b_lds[i] = k * BNT + ((cc ^ ((k & 3) << 1)) << 3);
     }
   }
 
@@ -226,21 +230,21 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
     return b_base + k0;
   };
 
-  f32x16 acc[2][4];
+  f32x16 acc[2][NJ];
 #pragma unroll
   for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
-    for (int nj = 0; nj < 4; ++nj)
+    for (int nj = 0; nj < NJ; ++nj)
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[mi][nj][i] = 0.0f;
 
-  int bcol[4];
+  int bcol[NJ];
 #pragma unroll
-  for (int nj = 0; nj < 4; ++nj) {
+  for (int nj = 0; nj < NJ; ++nj) {
     if constexpr (MODE == RM_GATEUP)
-      bcol[nj] = (nj < 2 ? 0 : RBN / 2) + wn * 64 + (nj & 1) * 32;
+      bcol[nj] = (nj < 2 ? 0 : BNT / 2) + wn * 64 + (nj & 1) * 32;
     else
-      bcol[nj] = wn * 128 + nj * 32;
+      bcol[nj] = wn * (32 * NJ) + nj * 32;
   }
 
   const int ksteps = Kdim / BK;
@@ -252,22 +256,22 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) ra[i] = *reinterpret_cast<const u32x4*>(ab + a_off[i]);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int64_t x = (MODE == RM_GATEUP && i >= 4) ? b1_off : 0;
+    for (int i = 0; i < NB; ++i) {
+      const int64_t x = (MODE == RM_GATEUP && i >= NB / 2) ? b1_off : 0;
       rb[i] = *reinterpret_cast<const u32x4*>(bb + x + b_off[i]);
     }
 #pragma unroll
     for (int i = 0; i < 2; ++i) *reinterpret_cast<u32x4*>(smem + kc_lds + i * 64 * BK) = ra[i];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(smem + RBM * BK + b_lds[i]) = rb[i];
+    for (int i = 0; i < NB; ++i) *reinterpret_cast<u32x4*>(smem + RBM * BK + b_lds[i]) = rb[i];
     if (ksteps > 1) {
       const uint16_t* ab1 = a_ptr(kofs(1));
       const uint16_t* bb1 = b_ptr(kofs(1));
 #pragma unroll
       for (int i = 0; i < 2; ++i) ra[i] = *reinterpret_cast<const u32x4*>(ab1 + a_off[i]);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int64_t x = (MODE == RM_GATEUP && i >= 4) ? b1_off : 0;
+      for (int i = 0; i < NB; ++i) {
+        const int64_t x = (MODE == RM_GATEUP && i >= NB / 2) ? b1_off : 0;
         rb[i] = *reinterpret_cast<const u32x4*>(bb1 + x + b_off[i]);
       }
     }
@@ -282,9 +286,9 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
   auto kstep = [&](int ks, auto has_next_t, auto has_next2_t) {
     constexpr bool has_next = decltype(has_next_t)::value;
     constexpr bool has_next2 = decltype(has_next2_t)::value;
-    const uint16_t* As = smem + (ks & 1) * R_STAGE;
+    const uint16_t* As = smem + (ks & 1) * STAGE;
     const uint16_t* Bs = As + RBM * BK;
-    uint16_t* An = smem + ((ks + 1) & 1) * R_STAGE;
+    uint16_t* An = smem + ((ks + 1) & 1) * STAGE;
     uint16_t* Bn = An + RBM * BK;
     const uint16_t* ab2 = has_next2 ? a_ptr(kofs(ks + 2)) : nullptr;
     const uint16_t* bb2 = has_next2 ? b_ptr(kofs(ks + 2)) : nullptr;
@@ -295,22 +299,25 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
       // same registers with the same chunks of tile ks+2.
       if constexpr (has_next) {
         if (kk < 2) *reinterpret_cast<u32x4*>(An + kc_lds + kk * 64 * BK) = ra[kk];
-        *reinterpret_cast<u32x4*>(Bn + b_lds[2 * kk]) = rb[2 * kk];
-        *reinterpret_cast<u32x4*>(Bn + b_lds[2 * kk + 1]) = rb[2 * kk + 1];
+#pragma unroll
+        for (int i = (kk * NB) / 4; i < ((kk + 1) * NB) / 4; ++i)
+          *reinterpret_cast<u32x4*>(Bn + b_lds[i]) = rb[i];
       }
       if constexpr (has_next2) {
         if (kk < 2) ra[kk] = *reinterpret_cast<const u32x4*>(ab2 + a_off[kk]);
-        const int64_t x = (MODE == RM_GATEUP && kk >= 2) ? b1_off : 0;
-        rb[2 * kk] = *reinterpret_cast<const u32x4*>(bb2 + x + b_off[2 * kk]);
-        rb[2 * kk + 1] = *reinterpret_cast<const u32x4*>(bb2 + x + b_off[2 * kk + 1]);
+#pragma unroll
+        for (int i = (kk * NB) / 4; i < ((kk + 1) * NB) / 4; ++i) {
+          const int64_t x = (MODE == RM_GATEUP && i >= NB / 2) ? b1_off : 0;
+          rb[i] = *reinterpret_cast<const u32x4*>(bb2 + x + b_off[i]);
+        }
       }
-      bf16x8 af[2], bf[4];
+      bf16x8 af[2], bf[NJ];
 #pragma unroll
       for (int mi = 0; mi < 2; ++mi) af[mi] = frag_kc(As, wm + mi * 32, kk, lane);
 #pragma unroll
-      for (int nj = 0; nj < 4; ++nj) {
+      for (int nj = 0; nj < NJ; ++nj) {
         if constexpr (B_KS)
-          bf[nj] = frag_ks<RBN>(Bs, bcol[nj], kk, lane);
+          bf[nj] = frag_ks<BNT>(Bs, bcol[nj], kk, lane);
         else
           bf[nj] = frag_kc(Bs, bcol[nj], kk, lane);
       }
@@ -320,7 +327,7 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
 #pragma unroll
       for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
-        for (int nj = 0; nj < 4; ++nj)
+        for (int nj = 0; nj < NJ; ++nj)
           acc[mi][nj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[nj], af[mi], acc[mi][nj], 0, 0, 0);
       phase_barrier();
     }
@@ -385,23 +392,24 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
       __builtin_amdgcn_wave_barrier();
     }
   } else {
-    using S = WaveStage<128>;
+    using S = WaveStage<32 * NJ>;
+    constexpr int CH = 4 * NJ;  // 16-byte chunks per row of the wave's sub-tile
 #pragma unroll
     for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
-      for (int nj = 0; nj < 4; ++nj)
+      for (int nj = 0; nj < NJ; ++nj)
 #pragma unroll
         for (int q = 0; q < 4; ++q)
           S::put4(st, mi, nj * 32, lane, q, acc[mi][nj][q * 4], acc[mi][nj][q * 4 + 1],
                   acc[mi][nj][q * 4 + 2], acc[mi][nj][q * 4 + 3]);
     __builtin_amdgcn_s_waitcnt(0xc07f);
     __builtin_amdgcn_wave_barrier();
-    const int c0 = n0 + wn * 128;
-    // 64 rows x 16 chunks = 1024 chunks, 16 per lane; a row's 256 bytes go out contiguously
+    const int c0 = n0 + wn * (32 * NJ);
+    // 64 rows x CH chunks, CH per lane; a row's bytes go out contiguously
 #pragma unroll 4
-    for (int it = 0; it < 16; ++it) {
+    for (int it = 0; it < CH; ++it) {
       const int idx = it * 64 + lane;
-      const int m = idx >> 4, c = idx & 15;
+      const int m = idx / CH, c = idx % CH;
       const int n = c0 + c * 8;
       if (wm + m < valid && n < Ncols) {
         const u32x4 v = *reinterpret_cast<const u32x4*>(st + m * S::PITCH + c * 8);
@@ -593,16 +601,19 @@ static unsigned round8(int64_t v) { return static_cast<unsigned>((v + 7) / 8 * 8
 constexpr int R_LDS_BYTES = 2 * R_STAGE * 2;  // 163840
 constexpr int W_LDS_BYTES = 8 * 64 * 136 * 2;  // 139264: the 8 epilogue regions (> 2 stages = 131072)
 
-template <int MODE>
+template <int MODE, int NJ>
 static int launch_row(RowArgs& a, int64_t tile_capacity, hipStream_t s, const char* what) {
   static bool configured = false;  // per process; the attribute is per function
   if (!configured) {
-    if (int rc = set_lds(row_tiled_kernel<MODE>, R_LDS_BYTES)) return rc;
+    if (int rc = set_lds(row_tiled_kernel<MODE, NJ>, R_LDS_BYTES)) return rc;
     configured = true;
   }
-  hipLaunchKernelGGL(row_tiled_kernel<MODE>, dim3(round8(tile_capacity * a.n_tiles)), dim3(NT), R_LDS_BYTES, s, a);
+  hipLaunchKernelGGL((row_tiled_kernel<MODE, NJ>), dim3(round8(tile_capacity * a.n_tiles)), dim3(NT), R_LDS_BYTES, s, a);
   return check_launch(what);
 }
+
+// 384-column tiles when they divide the width and 512-column tiles do not (F = 768).
+static bool narrow_tiles(int64_t width) { return width % 512 != 0 && width % 384 == 0; }
 
 int bf16_grouped_fwd(const void* rows, const void* w1, const void* w3, const void* w2,
                        const int32_t* seg_offsets, const int32_t* seg_counts,
@@ -616,13 +627,18 @@ int bf16_grouped_fwd(const void* rows, const void* w1, const void* w3, const voi
     a.a0 = (const uint16_t*)rows; a.b0 = (const uint16_t*)w1; a.b1 = (const uint16_t*)w3;
     a.o0 = (uint16_t*)gate; a.o1 = (uint16_t*)up; a.o2 = (uint16_t*)h;
     a.n_tiles = (int)((F + RBN / 2 - 1) / (RBN / 2));
-    if (int rc = launch_row<RM_GATEUP>(a, tile_capacity, s, "grouped gate/up")) return rc;
+    if (int rc = launch_row<RM_GATEUP, 4>(a, tile_capacity, s, "grouped gate/up")) return rc;
   }
   if (stages & STAGE_DOWN) {
     RowArgs b = a;
     b.a0 = (const uint16_t*)h; b.b0 = (const uint16_t*)w2; b.o0 = (uint16_t*)y;
-    b.n_tiles = (int)((D + RBN - 1) / RBN);
-    if (int rc = launch_row<RM_DOWN>(b, tile_capacity, s, "grouped down")) return rc;
+    if (narrow_tiles(D)) {
+      b.n_tiles = (int)(D / 384);
+      if (int rc = launch_row<RM_DOWN, 3>(b, tile_capacity, s, "grouped down")) return rc;
+    } else {
+      b.n_tiles = (int)((D + RBN - 1) / RBN);
+      if (int rc = launch_row<RM_DOWN, 4>(b, tile_capacity, s, "grouped down")) return rc;
+    }
   }
   return MI355_OK;
 }
@@ -641,15 +657,25 @@ int bf16_grouped_bwd(const void* dy, const void* rows, const void* w1, const voi
     a.a0 = (const uint16_t*)dy; a.b0 = (const uint16_t*)w2;
     a.gate = (const uint16_t*)gate; a.up = (const uint16_t*)up;
     a.o0 = (uint16_t*)dgate; a.o1 = (uint16_t*)dup;
-    a.n_tiles = (int)((F + RBN - 1) / RBN);
-    if (int rc = launch_row<RM_DH>(a, tile_capacity, s, "grouped dh")) return rc;
+    if (narrow_tiles(F)) {
+      a.n_tiles = (int)(F / 384);
+      if (int rc = launch_row<RM_DH, 3>(a, tile_capacity, s, "grouped dh")) return rc;
+    } else {
+      a.n_tiles = (int)((F + RBN - 1) / RBN);
+      if (int rc = launch_row<RM_DH, 4>(a, tile_capacity, s, "grouped dh")) return rc;
+    }
   }
   if (drows && (stages & STAGE_DX)) {
     RowArgs b = a;
     b.a0 = (const uint16_t*)dgate; b.a1 = (const uint16_t*)dup;
     b.b0 = (const uint16_t*)w1; b.b1 = (const uint16_t*)w3; b.o0 = (uint16_t*)drows;
-    b.n_tiles = (int)((D + RBN - 1) / RBN);
-    if (int rc = launch_row<RM_DX>(b, tile_capacity, s, "grouped drows")) return rc;
+    if (narrow_tiles(D)) {
+      b.n_tiles = (int)(D / 384);
+      if (int rc = launch_row<RM_DX, 3>(b, tile_capacity, s, "grouped drows")) return rc;
+    } else {
+      b.n_tiles = (int)((D + RBN - 1) / RBN);
+      if (int rc = launch_row<RM_DX, 4>(b, tile_capacity, s, "grouped drows")) return rc;
+    }
   }
   static bool wconfigured = false;
   if (!wconfigured) {

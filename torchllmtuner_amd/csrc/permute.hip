@@ -2,9 +2,9 @@
 //
 // Plan = a stable counting sort of the N = T*K assignment slots by expert id.
 //   1. plan_rank    each wave walks 512 consecutive slots in 64-slot chunks; within
-//                   a chunk, slots of the same expert are ranked by a ballot loop
-//                   (one iteration per distinct expert in the chunk), running
-//                   per-wave expert counts live in LDS.  Emits the rank of every
+//                   a chunk a slot's rank among equal experts is counted with 64
+//                   lane reads, and the running per-wave expert counts live in LDS
+//                   (one writer per expert and chunk).  Emits the rank of every
 //                   slot inside its wave and the wave's histogram.
 //   2. plan_scan    one workgroup: per-expert exclusive scan of the wave histograms
 //                   (ascending wave = ascending slot, which is what makes the sort
@@ -32,26 +32,28 @@ __global__ __launch_bounds__(256) void plan_rank_kernel(const int64_t* __restric
 
   const int gw = blockIdx.x * kWavesPerBlock + wave;
   const int begin = gw * kSlotsPerWave;
-  const unsigned long long lt_mask = (1ull << lane) - 1ull;
   for (int c = 0; c < kSlotsPerWave; c += kWave) {
     const int slot = begin + c + lane;
     const bool valid = slot < N;
     int e = valid ? static_cast<int>(ids[slot]) : -1;
     if (e < 0 || e >= E) e = valid ? 0 : -1;  // out-of-range ids are folded, never written OOB
-    unsigned long long todo = __ballot(valid);
-    int rank = 0;
-    while (todo) {
-      const int leader = __ffsll(static_cast<long long>(todo)) - 1;
-      const int e0 = __shfl(e, leader, kWave);
-      const unsigned long long same = __ballot(valid && e == e0);
-      const int base = my[e0];
-      if (e == e0) rank = base + __popcll(same & lt_mask);
-      __builtin_amdgcn_wave_barrier();
-      if (lane == leader) my[e0] = base + __popcll(same);
-      __builtin_amdgcn_wave_barrier();
-      todo &= ~same;
+    // rank among the chunk's lower lanes with the same expert, and whether a higher lane
+    // holds it too: 64 uniform-lane reads, no LDS round trip per distinct expert
+    int below = 0, above = 0;
+#pragma unroll 8
+    for (int j = 0; j < kWave; ++j) {
+      const int ej = __builtin_amdgcn_readlane(e, j);
+      const int same = (ej == e) ? 1 : 0;
+      below += (j < lane) ? same : 0;
+      above += (j > lane) ? same : 0;
     }
-    if (valid) rank_in_wave[slot] = rank;
+    if (valid) {
+      const int base = my[e];
+      rank_in_wave[slot] = base + below;
+      __builtin_amdgcn_wave_barrier();
+      if (above == 0) my[e] = base + below + 1;  // one writer per expert: its highest lane
+    }
+    __builtin_amdgcn_wave_barrier();
   }
   __syncthreads();
   for (int e = lane; e < E; e += kWave) wave_hist[static_cast<int64_t>(gw) * E + e] = my[e];
