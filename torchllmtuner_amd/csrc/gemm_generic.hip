@@ -8,6 +8,8 @@
 // that walks the operand's contiguous axis.
 #include "gemm_generic.h"
 
+#include <cstdint>
+
 namespace mi355 {
 
 namespace {
@@ -134,6 +136,107 @@ __global__ __launch_bounds__(256) void ggemm_kernel(GemmArgs g) {
   }
 }
 
+// ---- dense GEMM with 16-byte (fp32) / 8-byte (bf16) vector loads -------------------------
+// Same 64x64 tile and fp32 MFMA as above, 32-deep K slabs, for the DENSE mode when the
+// operands allow 4-element vector loads along their contiguous axis (the router
+// projections).  AV / BV: 0 = the K axis is contiguous, 1 = the M (resp. N) axis is.
+constexpr int VK = 32, VPITCH = 68;
+
+template <typename T>
+__device__ __forceinline__ void load4(const T* p, float (&v)[4]);
+template <>
+__device__ __forceinline__ void load4<float>(const float* p, float (&v)[4]) {
+  const float4 t = *reinterpret_cast<const float4*>(p);
+  v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+}
+template <>
+__device__ __forceinline__ void load4<uint16_t>(const uint16_t* p, float (&v)[4]) {
+  const uint2 t = *reinterpret_cast<const uint2*>(p);
+  v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
+  v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
+}
+
+template <typename TA, typename TB, typename TC, int AV, int BV>
+__global__ __launch_bounds__(256) void dense_vec_kernel(GemmArgs g) {
+  __shared__ __attribute__((aligned(16))) float As[VK][VPITCH];
+  __shared__ __attribute__((aligned(16))) float Bs[VK][VPITCH];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
+  const TA* A = static_cast<const TA*>(g.A);
+  const TB* B = static_cast<const TB*>(g.B);
+  const int m0 = blockIdx.x * TM, n0 = blockIdx.y * TN;
+  int k_begin = 0, k_end = g.K;
+  float* Cpartial = nullptr;
+  if (g.ksplit > 1) {
+    const int chunk = ((g.K + g.ksplit - 1) / g.ksplit + VK - 1) / VK * VK;
+    k_begin = blockIdx.z * chunk;
+    k_end = min(g.K, k_begin + chunk);
+    Cpartial = reinterpret_cast<float*>(g.C) + static_cast<int64_t>(blockIdx.z) * g.M * g.ldc;
+  }
+  // two 4-vectors of A and two of B per thread and slab
+  int am[2], ak[2], bk[2], bn[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int i = tid + j * 256;
+    if (AV == 0) { ak[j] = (i & 7) * 4; am[j] = i >> 3; } else { am[j] = (i & 15) * 4; ak[j] = i >> 4; }
+    if (BV == 0) { bk[j] = (i & 7) * 4; bn[j] = i >> 3; } else { bn[j] = (i & 15) * 4; bk[j] = i >> 4; }
+  }
+  float ra[2][4], rb[2][4];
+  auto load_slab = [&](int k0) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const bool a_ok = (m0 + am[j] < g.M) && (k0 + ak[j] < k_end);
+      if (a_ok) load4<TA>(A + static_cast<int64_t>(m0 + am[j]) * g.a_rs + static_cast<int64_t>(k0 + ak[j]) * g.a_cs, ra[j]);
+      else ra[j][0] = ra[j][1] = ra[j][2] = ra[j][3] = 0.0f;
+      const bool b_ok = (n0 + bn[j] < g.N) && (k0 + bk[j] < k_end);
+      if (b_ok) load4<TB>(B + static_cast<int64_t>(k0 + bk[j]) * g.b_rs + static_cast<int64_t>(n0 + bn[j]) * g.b_cs, rb[j]);
+      else rb[j][0] = rb[j][1] = rb[j][2] = rb[j][3] = 0.0f;
+    }
+  };
+  f32x16 acc;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+  if (k_begin < k_end) load_slab(k_begin);
+  for (int k0 = k_begin; k0 < k_end; k0 += VK) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      if (AV == 0) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) As[ak[j] + q][am[j]] = ra[j][q];
+      } else {
+        *reinterpret_cast<float4*>(&As[ak[j]][am[j]]) = make_float4(ra[j][0], ra[j][1], ra[j][2], ra[j][3]);
+      }
+      if (BV == 0) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) Bs[bk[j] + q][bn[j]] = rb[j][q];
+      } else {
+        *reinterpret_cast<float4*>(&Bs[bk[j]][bn[j]]) = make_float4(rb[j][0], rb[j][1], rb[j][2], rb[j][3]);
+      }
+    }
+    __syncthreads();
+    if (k0 + VK < k_end) load_slab(k0 + VK);
+#pragma unroll
+    for (int kk = 0; kk < VK; kk += 2) {
+      const float a = As[kk + (lane >> 5)][wm + (lane & 31)];
+      const float b = Bs[kk + (lane >> 5)][wn + (lane & 31)];
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc, 0, 0, 0);
+    }
+    __syncthreads();
+  }
+  const int n = n0 + wn + (lane & 31);
+  if (n >= g.N) return;
+  const float bias = g.bias ? g.bias[n] : 0.0f;
+  TC* C = static_cast<TC*>(g.C);
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int m = m0 + wm + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3);
+    if (m >= g.M) continue;
+    const int64_t off = static_cast<int64_t>(m) * g.ldc + n;
+    if (Cpartial) Cpartial[off] = acc[i];
+    else store_from_f32(C + off, acc[i] + bias);
+  }
+}
+
 template <typename TC>
 __global__ void splitk_reduce_kernel(const float* __restrict__ partial, TC* __restrict__ out,
                                      int64_t MN, int ksplit) {
@@ -155,9 +258,57 @@ int launch_c(const GemmArgs& a, int c_dtype, dim3 grid, hipStream_t s) {
 
 }  // namespace
 
+namespace {
+
+template <typename TA, typename TB, int AV, int BV>
+int launch_vec(const GemmArgs& a, int c_dtype, dim3 grid, hipStream_t s) {
+  if (c_dtype == MI355_F32 || a.ksplit > 1)
+    hipLaunchKernelGGL((dense_vec_kernel<TA, TB, float, AV, BV>), grid, dim3(256), 0, s, a);
+  else
+    hipLaunchKernelGGL((dense_vec_kernel<TA, TB, uint16_t, AV, BV>), grid, dim3(256), 0, s, a);
+  return check_launch("dense_vec_gemm");
+}
+
+template <typename TA, typename TB>
+int launch_vec_layout(const GemmArgs& a, int av, int bv, int c_dtype, dim3 grid, hipStream_t s) {
+  if (av == 0 && bv == 0) return launch_vec<TA, TB, 0, 0>(a, c_dtype, grid, s);
+  if (av == 0 && bv == 1) return launch_vec<TA, TB, 0, 1>(a, c_dtype, grid, s);
+  if (av == 1 && bv == 0) return launch_vec<TA, TB, 1, 0>(a, c_dtype, grid, s);
+  return launch_vec<TA, TB, 1, 1>(a, c_dtype, grid, s);
+}
+
+// The vector kernel applies to a dense, non-accumulating problem whose operands are
+// 4-element aligned along a unit-stride axis.
+bool vec_layout(const GemmArgs& a, int a_dtype, int b_dtype, int* av, int* bv) {
+  if (a.mode != GEMM_DENSE || a.accumulate) return false;
+  const int64_t asz = a_dtype == MI355_F32 ? 4 : 2, bsz = b_dtype == MI355_F32 ? 4 : 2;
+  if (reinterpret_cast<uintptr_t>(a.A) % (4 * asz) || reinterpret_cast<uintptr_t>(a.B) % (4 * bsz)) return false;
+  if (a.K % 4) return false;
+  if (a.a_cs == 1 && a.a_rs % 4 == 0) *av = 0;
+  else if (a.a_rs == 1 && a.a_cs % 4 == 0 && a.M % 4 == 0) *av = 1;
+  else return false;
+  if (a.b_rs == 1 && a.b_cs % 4 == 0) *bv = 0;
+  else if (a.b_cs == 1 && a.b_rs % 4 == 0 && a.N % 4 == 0) *bv = 1;
+  else return false;
+  if (a.ksplit > 1) {
+    const int chunk = ((a.K + a.ksplit - 1) / a.ksplit + VK - 1) / VK * VK;
+    if (chunk % 4) return false;
+  }
+  return true;
+}
+
+}  // namespace
+
 int launch_gemm(const GemmArgs& a, int a_dtype, int b_dtype, int c_dtype, dim3 grid,
                 hipStream_t s) {
   if (grid.x == 0 || grid.y == 0 || grid.z == 0) return MI355_OK;
+  int av = 0, bv = 0;
+  if (vec_layout(a, a_dtype, b_dtype, &av, &bv)) {
+    if (a_dtype == MI355_F32 && b_dtype == MI355_F32) return launch_vec_layout<float, float>(a, av, bv, c_dtype, grid, s);
+    if (a_dtype == MI355_BF16 && b_dtype == MI355_F32) return launch_vec_layout<uint16_t, float>(a, av, bv, c_dtype, grid, s);
+    if (a_dtype == MI355_F32 && b_dtype == MI355_BF16) return launch_vec_layout<float, uint16_t>(a, av, bv, c_dtype, grid, s);
+    if (a_dtype == MI355_BF16 && b_dtype == MI355_BF16) return launch_vec_layout<uint16_t, uint16_t>(a, av, bv, c_dtype, grid, s);
+  }
   if (a_dtype == MI355_F32 && b_dtype == MI355_F32) return launch_c<float, float>(a, c_dtype, grid, s);
   if (a_dtype == MI355_BF16 && b_dtype == MI355_F32) return launch_c<uint16_t, float>(a, c_dtype, grid, s);
   if (a_dtype == MI355_F32 && b_dtype == MI355_BF16) return launch_c<float, uint16_t>(a, c_dtype, grid, s);
