@@ -130,6 +130,9 @@ int mi355_router_select_bwd(const float* logits_TE, const int64_t* ids_TK,
  *   seg_counts    (El)    real (unpadded) rows per local segment
  *   row_of_slot   (N)     row of slot t*K+k, or -1 when not local
  *   slot_of_row   (row_capacity) slot held by each row, -1 for padding / unused
+ *   token_of_row  (row_capacity) token held by each row (slot / K), -1 for padding /
+ *                 unused; optional (NULL = skip): the gather index of the fused expert
+ *                 kernels below
  *   tile_expert, tile_row0 (tile_capacity each) and num_tiles (1): the list of
  *       tile_m-row tiles covering the real rows of every segment (local expert
  *       index and first row of each tile)
@@ -143,7 +146,7 @@ int mi355_permute_plan(const int64_t* ids_TK, int64_t T, int64_t K, int64_t E,
                        int64_t local_lo, int64_t local_hi, int64_t align,
                        int64_t tile_m, int32_t* counts_E, int32_t* seg_offsets,
                        int32_t* seg_counts, int32_t* row_of_slot,
-                       int32_t* slot_of_row, int64_t row_capacity,
+                       int32_t* slot_of_row, int32_t* token_of_row, int64_t row_capacity,
                        int32_t* tile_expert, int32_t* tile_row0, int32_t* num_tiles,
                        int64_t tile_capacity, void* workspace, void* stream);
 
@@ -221,13 +224,18 @@ int mi355_combine_bwd(const void* dout, const void* y, int dtype,
  * llmtuner/models/common/moe/experts.py:204-209, its _grouped_mm (:211-285) and
  * SwiGLU.forward, llmtuner/models/common/activation.py:36-37.
  * w1,w3: (El,F,D); w2: (El,D,F), all `dtype`, row-major.
+ * token_of_row (optional): when given, `rows` is the UNPERMUTED (T,D) token matrix and
+ * row r reads rows[token_of_row[r]] -- the gather of token_dispatch.py:197-199 fused
+ * into the operand loads, so the (R,D) expert-major copy is never written.  bf16 with
+ * D and F multiples of 64 only (MI355_EUNSUP otherwise).
  * gate/up/h are saved for the backward (each (row_capacity,F)).
  * bf16 uses MFMA tiles of tile_m rows (the plan's tile list must have been built
  * with the value mi355_grouped_tile_m(dtype) returns).
  */
 int64_t mi355_grouped_tile_m(int dtype);
-int mi355_grouped_swiglu_fwd(const void* rows, const void* w1, const void* w3,
-                             const void* w2, int dtype, const int32_t* seg_offsets,
+int mi355_grouped_swiglu_fwd(const void* rows, const int32_t* token_of_row,
+                             const void* w1, const void* w3, const void* w2, int dtype,
+                             const int32_t* seg_offsets,
                              const int32_t* seg_counts, const int32_t* tile_expert,
                              const int32_t* tile_row0, const int32_t* num_tiles,
                              int64_t tile_capacity, void* gate, void* up, void* h,
@@ -241,9 +249,12 @@ int mi355_grouped_swiglu_fwd(const void* rows, const void* w1, const void* w3,
  *   dw2[e] = dy_e^T . h_e;  dw1[e] = dgate_e^T . rows_e;  dw3[e] = dup_e^T . rows_e
  * dgate/dup are caller-provided scratch of (row_capacity,F) each.  Weight
  * gradients are written (not accumulated) in `dtype`; experts with no rows get
- * zeros.  Any of drows/dw1/dw3/dw2 may be NULL to skip it.
+ * zeros.  Any of drows/dw1/dw3/dw2 may be NULL to skip it.  token_of_row has the
+ * meaning it has in the forward (`rows` = the (T,D) token matrix); drows is always
+ * expert-major (row_capacity,D) and goes through mi355_permute_rows_bwd.
  */
-int mi355_grouped_swiglu_bwd(const void* dy, const void* rows, const void* w1,
+int mi355_grouped_swiglu_bwd(const void* dy, const void* rows,
+                             const int32_t* token_of_row, const void* w1,
                              const void* w3, const void* w2, const void* gate,
                              const void* up, const void* h, int dtype,
                              const int32_t* seg_offsets, const int32_t* seg_counts,
@@ -265,7 +276,8 @@ int mi355_grouped_swiglu_bwd(const void* dy, const void* rows, const void* w1,
 #define MI355_STAGE_DW2 16   /* dw2           <- dy, h        */
 #define MI355_STAGE_DW1 32   /* dw1           <- dgate, rows  */
 #define MI355_STAGE_DW3 64   /* dw3           <- dup, rows    */
-int mi355_grouped_swiglu_stage(int stage, const void* dy, const void* rows, const void* w1,
+int mi355_grouped_swiglu_stage(int stage, const void* dy, const void* rows,
+                               const int32_t* token_of_row, const void* w1,
                                const void* w3, const void* w2, void* gate, void* up,
                                void* h, void* y, const int32_t* seg_offsets,
                                const int32_t* seg_counts, const int32_t* tile_expert,

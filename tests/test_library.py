@@ -40,8 +40,8 @@ def test_argument_validation_reports_errors_without_a_gpu():
     rc = lib.mi355_router_select_fwd(None, None, None, None, None, 4, 0, 1, 0, 0, 1.0, 0, 0, 0, None)
     assert rc == -1
     assert b"E=0" in lib.mi355_moe_last_error()
-    rc = lib.mi355_permute_plan(None, 4, 2, 8, 5, 3, 1, 128, None, None, None, None, None, 8, None, None,
-                                None, 2, None, None)
+    rc = lib.mi355_permute_plan(None, 4, 2, 8, 5, 3, 1, 128, None, None, None, None, None, None, 8, None,
+                                None, None, 2, None, None)
     assert rc == -1 and b"local range" in lib.mi355_moe_last_error()
     with pytest.raises(ValueError, match="local range"):
         _lib.check(rc, "permute_plan")

@@ -30,21 +30,21 @@ SIGNATURES = {
     "mi355_router_select_fwd": (I, [P, P, P, P, P, L, L, L, I, I, F, I, I, I, P]),
     "mi355_router_select_bwd": (I, [P, P, P, P, P, L, L, L, I, I, F, I, P]),
     "mi355_permute_plan_workspace_bytes": (L, [L, L, L]),
-    "mi355_permute_plan": (I, [P, L, L, L, L, L, L, L, P, P, P, P, P, L, P, P, P, L, P, P]),
+    "mi355_permute_plan": (I, [P, L, L, L, L, L, L, L, P, P, P, P, P, P, L, P, P, P, L, P, P]),
     "mi355_segments_from_counts": (I, [P, L, L, L, P, P, P, P, P, L, P]),
     "mi355_permute_rows_fwd": (I, [P, I, P, P, P, L, L, L, L, P]),
     "mi355_permute_rows_bwd": (I, [P, I, P, P, L, L, L, P]),
     "mi355_combine_fwd": (I, [P, I, P, P, P, L, L, L, I, P]),
     "mi355_combine_bwd": (I, [P, P, I, P, P, P, P, P, P, L, L, L, L, P]),
     "mi355_grouped_tile_m": (L, [I]),
-    "mi355_grouped_swiglu_fwd": (I, [P, P, P, P, I, P, P, P, P, P, L, P, P, P, P, L, L, L, L, P]),
+    "mi355_grouped_swiglu_fwd": (I, [P, P, P, P, P, I, P, P, P, P, P, L, P, P, P, P, L, L, L, L, P]),
     "mi355_grouped_swiglu_stage": (
         I,
-        [I, P, P, P, P, P, P, P, P, P, P, P, P, P, P, L, P, P, P, P, P, P, L, L, L, L, P],
+        [I, P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, L, P, P, P, P, P, P, L, L, L, L, P],
     ),
     "mi355_grouped_swiglu_bwd": (
         I,
-        [P, P, P, P, P, P, P, P, I, P, P, P, P, P, L, P, P, P, P, P, P, L, L, L, L, P],
+        [P, P, P, P, P, P, P, P, P, I, P, P, P, P, P, L, P, P, P, P, P, P, L, L, L, L, P],
     ),
 }
 

@@ -12,13 +12,13 @@ namespace mi355 {
 constexpr int kTileM = 128;
 
 bool bf16_fast_path_ok(int64_t D, int64_t F);
-int bf16_grouped_fwd(const void* rows, const void* w1, const void* w3, const void* w2,
-                     const int32_t* seg_offsets, const int32_t* seg_counts,
+int bf16_grouped_fwd(const void* rows, const int32_t* token_of_row, const void* w1, const void* w3,
+                     const void* w2, const int32_t* seg_offsets, const int32_t* seg_counts,
                      const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* num_tiles,
                      int64_t tile_capacity, void* gate, void* up, void* h, void* y, int64_t D,
                      int64_t F, int stages, hipStream_t s);
-int bf16_grouped_bwd(const void* dy, const void* rows, const void* w1, const void* w3,
-                     const void* w2, const void* gate, const void* up, const void* h,
+int bf16_grouped_bwd(const void* dy, const void* rows, const int32_t* token_of_row, const void* w1,
+                     const void* w3, const void* w2, const void* gate, const void* up, const void* h,
                      const int32_t* seg_offsets, const int32_t* seg_counts,
                      const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* num_tiles,
                      int64_t tile_capacity, void* dgate, void* dup, void* drows, void* dw1,
@@ -119,8 +119,8 @@ extern "C" int64_t mi355_grouped_tile_m(int dtype) {
   return kTileM;
 }
 
-extern "C" int mi355_grouped_swiglu_fwd(const void* rows, const void* w1, const void* w3,
-                                        const void* w2, int dtype, const int32_t* seg_offsets,
+extern "C" int mi355_grouped_swiglu_fwd(const void* rows, const int32_t* token_of_row,
+                                        const void* w1, const void* w3, const void* w2, int dtype, const int32_t* seg_offsets,
                                         const int32_t* seg_counts, const int32_t* tile_expert,
                                         const int32_t* tile_row0, const int32_t* num_tiles,
                                         int64_t tile_capacity, void* gate, void* up, void* h, void* y,
@@ -133,9 +133,12 @@ extern "C" int mi355_grouped_swiglu_fwd(const void* rows, const void* w1, const 
                 "grouped_swiglu_fwd: null pointer");
   hipStream_t s = as_stream(stream);
   if (dtype == MI355_BF16 && bf16_fast_path_ok(D, F))
-    return bf16_grouped_fwd(rows, w1, w3, w2, seg_offsets, seg_counts,
+    return bf16_grouped_fwd(rows, token_of_row, w1, w3, w2, seg_offsets, seg_counts,
                                                              tile_expert, tile_row0, num_tiles,
                                                              tile_capacity, gate, up, h, y, D, F, 3, s);
+  if (token_of_row)
+    return fail(MI355_EUNSUP, "grouped_swiglu_fwd: the token gather needs bf16 with D and F multiples of 64; "
+                              "materialise the rows with mi355_permute_rows_fwd instead");
   const Seg sg{seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles, tile_capacity};
   // gate/up: B(k=d, n=f) = w[e][f][d]
   if (int rc = rowseg(sg, rows, D, w1, 1, D, F * D, gate, F, D, dtype, 0, s)) return rc;
@@ -152,7 +155,8 @@ extern "C" int mi355_grouped_swiglu_fwd(const void* rows, const void* w1, const 
   return rowseg(sg, h, F, w2, 1, F, D * F, y, D, F, dtype, 0, s);
 }
 
-extern "C" int mi355_grouped_swiglu_bwd(const void* dy, const void* rows, const void* w1,
+extern "C" int mi355_grouped_swiglu_bwd(const void* dy, const void* rows,
+                                        const int32_t* token_of_row, const void* w1,
                                         const void* w3, const void* w2, const void* gate,
                                         const void* up, const void* h, int dtype,
                                         const int32_t* seg_offsets, const int32_t* seg_counts,
@@ -169,8 +173,10 @@ extern "C" int mi355_grouped_swiglu_bwd(const void* dy, const void* rows, const 
   hipStream_t s = as_stream(stream);
   if (dtype == MI355_BF16 && bf16_fast_path_ok(D, F) && row_capacity > 0 && tile_capacity > 0)
     return bf16_grouped_bwd(
-        dy, rows, w1, w3, w2, gate, up, h, seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles,
+        dy, rows, token_of_row, w1, w3, w2, gate, up, h, seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles,
         tile_capacity, dgate, dup, drows, dw1, dw3, dw2, El, D, F, 0x7c, s);
+  if (token_of_row)
+    return fail(MI355_EUNSUP, "grouped_swiglu_bwd: the token gather needs bf16 with D and F multiples of 64");
   const Seg sg{seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles, tile_capacity};
   if (row_capacity > 0 && tile_capacity > 0) {
     // dh = dy . w2[e]: B(k=d, n=f) = w2[e][d][f]   (lands in dgate, rewritten in place below)
@@ -197,8 +203,8 @@ extern "C" int mi355_grouped_swiglu_bwd(const void* dy, const void* rows, const 
   return MI355_OK;
 }
 
-extern "C" int mi355_grouped_swiglu_stage(int stage, const void* dy, const void* rows, const void* w1,
-                                          const void* w3, const void* w2, void* gate, void* up,
+extern "C" int mi355_grouped_swiglu_stage(int stage, const void* dy, const void* rows,
+                                          const int32_t* token_of_row, const void* w1, const void* w3, const void* w2, void* gate, void* up,
                                           void* h, void* y, const int32_t* seg_offsets,
                                           const int32_t* seg_counts, const int32_t* tile_expert,
                                           const int32_t* tile_row0, const int32_t* num_tiles,
@@ -211,10 +217,10 @@ extern "C" int mi355_grouped_swiglu_stage(int stage, const void* dy, const void*
   if (row_capacity == 0 || tile_capacity == 0) return MI355_OK;
   hipStream_t s = as_stream(stream);
   if (stage <= 2)
-    return bf16_grouped_fwd(rows, w1, w3, w2, seg_offsets, seg_counts,
+    return bf16_grouped_fwd(rows, token_of_row, w1, w3, w2, seg_offsets, seg_counts,
                                                              tile_expert, tile_row0, num_tiles,
                                                              tile_capacity, gate, up, h, y, D, F, stage, s);
   return bf16_grouped_bwd(
-      dy, rows, w1, w3, w2, gate, up, h, seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles,
+      dy, rows, token_of_row, w1, w3, w2, gate, up, h, seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles,
       tile_capacity, dgate, dup, drows, dw1, dw3, dw2, El, D, F, stage, s);
 }

@@ -132,6 +132,7 @@ struct RowArgs {
   uint16_t* o2;        // GATEUP h
   const uint16_t* gate;  // DH
   const uint16_t* up;    // DH
+  const int32_t* a_src;  // GATEUP: row -> row of a0 to read (token gather), or null
   const int32_t* seg_offsets;
   const int32_t* seg_counts;
   const int32_t* tile_expert;
@@ -183,11 +184,15 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
   u32x4 ra[2], rb[NB];
   const int kc_row = tid >> 3, kc_chunk = tid & 7;
   const int kc_lds = kc_row * BK + ((kc_chunk ^ ((kc_row >> 1) & 7)) << 3);  // + i*64*BK (64 % 16 == 0)
-  const uint16_t* a_base0 = p.a0 + static_cast<int64_t>(row0) * lda + kc_chunk * 8;
+  const bool gather = (MODE == RM_GATEUP) && p.a_src != nullptr;
+  const uint16_t* a_base0 = p.a0 + (gather ? 0 : static_cast<int64_t>(row0) * lda) + kc_chunk * 8;
   const uint16_t* a_base1 = (MODE == RM_DX) ? p.a1 + static_cast<int64_t>(row0) * lda + kc_chunk * 8 : a_base0;
   int a_off[2];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) a_off[i] = min(kc_row + 64 * i, valid - 1) * lda;
+  for (int i = 0; i < 2; ++i) {
+    const int r = min(kc_row + 64 * i, valid - 1);
+    a_off[i] = (gather ? max(p.a_src[row0 + r], 0) : r) * lda;
+  }
 
   const uint16_t* b_base = B0;
   int b_off[NB];
@@ -455,6 +460,7 @@ struct WgradArgs {
   const uint16_t* a;  // (rows, M) row-major
   const uint16_t* b;  // (rows, N) row-major
   uint16_t* c;        // (El, M, N)
+  const int32_t* b_src;  // row -> row of b to read (token gather), or null
   const int32_t* seg_offsets;
   const int32_t* seg_counts;
   int M, N;
@@ -481,7 +487,13 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
   u32x4 ra[4], rb[4];
   const int ks_k = tid >> 5, ks_chunk = tid & 31;
   const uint16_t* a_base = p.a + static_cast<int64_t>(seg0) * M + min(m0 + ks_chunk * 8, M - 8);
-  const uint16_t* b_base = p.b + static_cast<int64_t>(seg0) * N + min(n0 + ks_chunk * 8, N - 8);
+  const uint16_t* b_base = p.b + (p.b_src ? 0 : static_cast<int64_t>(seg0) * N) + min(n0 + ks_chunk * 8, N - 8);
+  // With a gather, the source row of B's k-th row comes from an index array.  The
+  // indices of the step after the one being fetched are loaded one step early (tk), so
+  // no data load waits on an index load in the steady state.
+  const int32_t* b_src = p.b_src ? p.b_src + seg0 : nullptr;
+  auto src_row = [&](int k) -> int { return (b_src && k < cnt) ? max(b_src[k], 0) : k; };
+  int tk[4];
   int lds_off[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -504,7 +516,7 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
     for (int i = 0; i < 4; ++i) {
       const int k = ks_k + 16 * i;
       ra[i] = k < cnt ? *reinterpret_cast<const u32x4*>(a_base + static_cast<int64_t>(k) * M) : zero;
-      rb[i] = k < cnt ? *reinterpret_cast<const u32x4*>(b_base + static_cast<int64_t>(k) * N) : zero;
+      rb[i] = k < cnt ? *reinterpret_cast<const u32x4*>(b_base + static_cast<int64_t>(src_row(k)) * N) : zero;
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -516,10 +528,12 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
       for (int i = 0; i < 4; ++i) {
         const int k = BK + ks_k + 16 * i;
         ra[i] = k < cnt ? *reinterpret_cast<const u32x4*>(a_base + static_cast<int64_t>(k) * M) : zero;
-        rb[i] = k < cnt ? *reinterpret_cast<const u32x4*>(b_base + static_cast<int64_t>(k) * N) : zero;
+        rb[i] = k < cnt ? *reinterpret_cast<const u32x4*>(b_base + static_cast<int64_t>(src_row(k)) * N) : zero;
       }
     }
   }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) tk[i] = src_row(2 * BK + ks_k + 16 * i);
   __syncthreads();
 
   // The K extent here is one expert's rows (a handful of 64-row steps), so the loop is
@@ -542,7 +556,8 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
       if (has_next2) {
         const int k = kbase2 + ks_k + 16 * kk;
         ra[kk] = k < cnt ? *reinterpret_cast<const u32x4*>(a_base + static_cast<int64_t>(k) * M) : zero;
-        rb[kk] = k < cnt ? *reinterpret_cast<const u32x4*>(b_base + static_cast<int64_t>(k) * N) : zero;
+        rb[kk] = k < cnt ? *reinterpret_cast<const u32x4*>(b_base + static_cast<int64_t>(b_src ? tk[kk] : k) * N) : zero;
+        tk[kk] = src_row(k + BK);
       }
       bf16x8 af[2], bf[4];
 #pragma unroll
@@ -615,8 +630,8 @@ static int launch_row(RowArgs& a, int64_t tile_capacity, hipStream_t s, const ch
 // 384-column tiles when they divide the width and 512-column tiles do not (F = 768).
 static bool narrow_tiles(int64_t width) { return width % 512 != 0 && width % 384 == 0; }
 
-int bf16_grouped_fwd(const void* rows, const void* w1, const void* w3, const void* w2,
-                       const int32_t* seg_offsets, const int32_t* seg_counts,
+int bf16_grouped_fwd(const void* rows, const int32_t* token_of_row, const void* w1, const void* w3,
+                       const void* w2, const int32_t* seg_offsets, const int32_t* seg_counts,
                        const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* num_tiles,
                        int64_t tile_capacity, void* gate, void* up, void* h, void* y, int64_t D,
                        int64_t F, int stages, hipStream_t s) {
@@ -624,7 +639,7 @@ int bf16_grouped_fwd(const void* rows, const void* w1, const void* w3, const voi
   a.seg_offsets = seg_offsets; a.seg_counts = seg_counts; a.tile_expert = tile_expert;
   a.tile_row0 = tile_row0; a.num_tiles = num_tiles; a.D = (int)D; a.F = (int)F;
   if (stages & STAGE_GATEUP) {
-    a.a0 = (const uint16_t*)rows; a.b0 = (const uint16_t*)w1; a.b1 = (const uint16_t*)w3;
+    a.a0 = (const uint16_t*)rows; a.a_src = token_of_row; a.b0 = (const uint16_t*)w1; a.b1 = (const uint16_t*)w3;
     a.o0 = (uint16_t*)gate; a.o1 = (uint16_t*)up; a.o2 = (uint16_t*)h;
     a.n_tiles = (int)((F + RBN / 2 - 1) / (RBN / 2));
     if (int rc = launch_row<RM_GATEUP, 4>(a, tile_capacity, s, "grouped gate/up")) return rc;
@@ -643,8 +658,8 @@ int bf16_grouped_fwd(const void* rows, const void* w1, const void* w3, const voi
   return MI355_OK;
 }
 
-int bf16_grouped_bwd(const void* dy, const void* rows, const void* w1, const void* w3,
-                       const void* w2, const void* gate, const void* up, const void* h,
+int bf16_grouped_bwd(const void* dy, const void* rows, const int32_t* token_of_row, const void* w1,
+                       const void* w3, const void* w2, const void* gate, const void* up, const void* h,
                        const int32_t* seg_offsets, const int32_t* seg_counts,
                        const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* num_tiles,
                        int64_t tile_capacity, void* dgate, void* dup, void* drows, void* dw1,
@@ -682,18 +697,18 @@ int bf16_grouped_bwd(const void* dy, const void* rows, const void* w1, const voi
     if (int rc = set_lds(wgrad_kernel, W_LDS_BYTES)) return rc;
     wconfigured = true;
   }
-  auto wgrad = [&](const void* A, const void* B, void* C, int64_t M, int64_t N, const char* what) {
+  auto wgrad = [&](const void* A, const void* B, const int32_t* b_src, void* C, int64_t M, int64_t N, const char* what) {
     WgradArgs w{};
-    w.a = (const uint16_t*)A; w.b = (const uint16_t*)B; w.c = (uint16_t*)C;
+    w.a = (const uint16_t*)A; w.b = (const uint16_t*)B; w.c = (uint16_t*)C; w.b_src = b_src;
     w.seg_offsets = seg_offsets; w.seg_counts = seg_counts; w.M = (int)M; w.N = (int)N;
     w.m_tiles = (int)((M + WBM - 1) / WBM); w.n_tiles = (int)((N + WBN - 1) / WBN);
     w.total = (int)(El * w.m_tiles * w.n_tiles);
     hipLaunchKernelGGL(wgrad_kernel, dim3(round8(w.total)), dim3(NT), W_LDS_BYTES, s, w);
     return check_launch(what);
   };
-  if (dw2 && (stages & STAGE_DW2)) if (int rc = wgrad(dy, h, dw2, D, F, "grouped dw2")) return rc;
-  if (dw1 && (stages & STAGE_DW1)) if (int rc = wgrad(dgate, rows, dw1, F, D, "grouped dw1")) return rc;
-  if (dw3 && (stages & STAGE_DW3)) if (int rc = wgrad(dup, rows, dw3, F, D, "grouped dw3")) return rc;
+  if (dw2 && (stages & STAGE_DW2)) if (int rc = wgrad(dy, h, nullptr, dw2, D, F, "grouped dw2")) return rc;
+  if (dw1 && (stages & STAGE_DW1)) if (int rc = wgrad(dgate, rows, token_of_row, dw1, F, D, "grouped dw1")) return rc;
+  if (dw3 && (stages & STAGE_DW3)) if (int rc = wgrad(dup, rows, token_of_row, dw3, F, D, "grouped dw3")) return rc;
   return MI355_OK;
 }
 

@@ -187,8 +187,8 @@ __global__ void fill_i32_kernel(int32_t* p, int64_t n, int32_t v) {
 __global__ __launch_bounds__(256) void plan_rows_kernel(
     const int64_t* __restrict__ ids, const int32_t* __restrict__ rank_in_wave,
     const int32_t* __restrict__ wave_prefix, const int32_t* __restrict__ seg_offsets, int N, int E,
-    int lo, int hi, int32_t* __restrict__ row_of_slot, int32_t* __restrict__ slot_of_row,
-    int row_capacity) {
+    int lo, int hi, int K, int32_t* __restrict__ row_of_slot, int32_t* __restrict__ slot_of_row,
+    int32_t* __restrict__ token_of_row, int row_capacity) {
   const int slot = blockIdx.x * blockDim.x + threadIdx.x;
   if (slot >= N) return;
   int e = static_cast<int>(ids[slot]);
@@ -197,7 +197,12 @@ __global__ __launch_bounds__(256) void plan_rows_kernel(
   if (e >= lo && e < hi) {
     const int gw = slot / kSlotsPerWave;
     row = seg_offsets[e - lo] + wave_prefix[static_cast<int64_t>(gw) * E + e] + rank_in_wave[slot];
-    if (row >= 0 && row < row_capacity) slot_of_row[row] = slot; else row = -1;
+    if (row >= 0 && row < row_capacity) {
+      slot_of_row[row] = slot;
+      if (token_of_row) token_of_row[row] = slot / K;
+    } else {
+      row = -1;
+    }
   }
   row_of_slot[slot] = row;
 }
@@ -317,7 +322,7 @@ extern "C" int mi355_permute_plan(const int64_t* ids, int64_t T, int64_t K, int6
                                   int64_t lo, int64_t hi, int64_t align, int64_t tile_m,
                                   int32_t* counts_E, int32_t* seg_offsets, int32_t* seg_counts,
                                   int32_t* row_of_slot, int32_t* slot_of_row,
-                                  int64_t row_capacity, int32_t* tile_expert, int32_t* tile_row0,
+                                  int32_t* token_of_row, int64_t row_capacity, int32_t* tile_expert, int32_t* tile_row0,
                                   int32_t* num_tiles, int64_t tile_capacity, void* workspace,
                                   void* stream) {
   const int64_t N = T * K;
@@ -346,6 +351,11 @@ extern "C" int mi355_permute_plan(const int64_t* ids, int64_t T, int64_t K, int6
     hipLaunchKernelGGL(fill_i32_kernel, dim3((unsigned)((row_capacity + 255) / 256)), dim3(256), 0, s,
                        slot_of_row, row_capacity, -1);
     if (int rc = check_launch("plan_fill")) return rc;
+    if (token_of_row) {
+      hipLaunchKernelGGL(fill_i32_kernel, dim3((unsigned)((row_capacity + 255) / 256)), dim3(256), 0, s,
+                         token_of_row, row_capacity, -1);
+      if (int rc = check_launch("plan_fill")) return rc;
+    }
   }
   const int El = (int)(hi - lo);
   int32_t* wave_prefix = wave_hist + (int64_t)nwaves * E;
@@ -359,8 +369,8 @@ extern "C" int mi355_permute_plan(const int64_t* ids, int64_t T, int64_t K, int6
   if (int rc = check_launch("plan_scan")) return rc;
   if (N > 0) {
     hipLaunchKernelGGL(plan_rows_kernel, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, s, ids,
-                       rank_in_wave, wave_prefix, seg_offsets, (int)N, (int)E, (int)lo, (int)hi,
-                       row_of_slot, slot_of_row, (int)row_capacity);
+                       rank_in_wave, wave_prefix, seg_offsets, (int)N, (int)E, (int)lo, (int)hi, (int)K,
+                       row_of_slot, slot_of_row, token_of_row, (int)row_capacity);
     if (int rc = check_launch("plan_rows")) return rc;
   }
   return MI355_OK;

@@ -8,6 +8,7 @@ include/mi355_moe.h):
   route_select    scores -> top-k -> gather -> norm       (fused select, fused VJP)
   permute_rows    expert-major row gather                 (bwd: K-way row sum)
   grouped_swiglu  gate/up/SiLU*mul/down grouped GEMMs     (bwd: dX and dW GEMMs)
+                  (gather_grouped_swiglu fuses permute_rows into the GEMM operand loads)
   combine         weighted unpermute                      (bwd: dY and dScore)
 """
 
@@ -117,6 +118,37 @@ class GroupedSwiGLUFunction(torch.autograd.Function):
         return drows, dw1, dw3, dw2, None
 
 
+class GatherGroupedSwiGLUFunction(torch.autograd.Function):
+    """Token gather fused into the expert GEMMs: y rows from the unpermuted (T, D) tokens.
+
+    Forward never materialises the expert-major copy of the tokens: the gate/up kernel
+    reads ``x[token_of_row[r]]`` directly, and nothing of size (R, D) is kept for the
+    backward.  Backward rebuilds the rows once (the weight-gradient kernels measured
+    30 % slower reading their K rows through the index) and returns ``dx``, the K-way
+    row sum of the expert-major input gradient.
+    """
+
+    @staticmethod
+    def forward(ctx, x_TD, w1_EFD, w3_EFD, w2_EDF, plan):
+        y, gate, up, h = ops.grouped_swiglu_fwd(x_TD, w1_EFD, w3_EFD, w2_EDF, plan, gather=True)
+        ctx.save_for_backward(x_TD, w1_EFD, w3_EFD, w2_EDF, gate, up, h)
+        ctx.plan = plan
+        return y
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, dy):
+        x, w1, w3, w2, gate, up, h = ctx.saved_tensors
+        need_dw = any(ctx.needs_input_grad[1:4])
+        rows = ops.permute_rows_fwd(x, ctx.plan) if need_dw else x
+        drows, dw1, dw3, dw2 = ops.grouped_swiglu_bwd(
+            dy, rows, w1, w3, w2, gate, up, h, ctx.plan,
+            need_drows=ctx.needs_input_grad[0], need_dw=need_dw, gather=not need_dw,
+        )
+        dx = ops.permute_rows_bwd(drows, ctx.plan) if drows is not None else None
+        return dx, dw1, dw3, dw2, None
+
+
 class CombineFunction(torch.autograd.Function):
     """out[t] = sum_k weights[t,k] * y[row(t,k)]; backward gives dY and dWeights."""
 
@@ -152,6 +184,10 @@ def permute_rows(x_TD, plan):
 
 def grouped_swiglu(rows_RD, w1_EFD, w3_EFD, w2_EDF, plan):
     return GroupedSwiGLUFunction.apply(rows_RD, w1_EFD, w3_EFD, w2_EDF, plan)
+
+
+def gather_grouped_swiglu(x_TD, w1_EFD, w3_EFD, w2_EDF, plan):
+    return GatherGroupedSwiGLUFunction.apply(x_TD, w1_EFD, w3_EFD, w2_EDF, plan)
 
 
 def combine(y_RD, weights_TK, plan, round_terms=True):

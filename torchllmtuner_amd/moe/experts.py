@@ -126,6 +126,11 @@ class GroupedExperts(nn.Module):
         w1, w3, w2 = self._weights_as(x_RD.dtype)
         return Fn.grouped_swiglu(x_RD, w1, w3, w2, plan)
 
+    def compute_gathered(self, x_TD, plan: ops.PermutePlan):
+        """Expert outputs for every planned row, reading the tokens through the plan."""
+        w1, w3, w2 = self._weights_as(x_TD.dtype)
+        return Fn.gather_grouped_swiglu(x_TD, w1, w3, w2, plan)
+
 
 class RoutedExperts(nn.Module):
     """The dispatch/combine pair wrapped around the grouped expert weights."""
@@ -144,13 +149,18 @@ class RoutedExperts(nn.Module):
         return self.forward_planned(x_TD, topk_scores_TK, plan)
 
     def forward_planned(self, x_TD, topk_scores_TK, plan: ops.PermutePlan):
-        with (
-            self.dispatch_observation.measure(x_TD.device)
-            if self.dispatch_observation is not None
-            else nullcontext()
-        ):
-            rows = Fn.permute_rows(x_TD, plan)
-        y = self.inner_experts.compute_planned(rows, plan)
+        experts = self.inner_experts
+        if ops.gather_supported(x_TD, experts.hidden_dim) and x_TD.is_contiguous():
+            # the dispatch gather rides inside the expert kernels' operand loads
+            y = experts.compute_gathered(x_TD, plan)
+        else:
+            with (
+                self.dispatch_observation.measure(x_TD.device)
+                if self.dispatch_observation is not None
+                else nullcontext()
+            ):
+                rows = Fn.permute_rows(x_TD, plan)
+            y = experts.compute_planned(rows, plan)
         out = Fn.combine(y, topk_scores_TK, plan, not self.token_dispatcher.accumulate_in_fp32)
         return out.to(x_TD.dtype)
 

@@ -156,6 +156,7 @@ class PermutePlan:
     seg_counts: torch.Tensor
     row_of_slot: torch.Tensor | None
     slot_of_row: torch.Tensor | None
+    token_of_row: torch.Tensor | None
     tile_expert: torch.Tensor
     tile_row0: torch.Tensor
     num_tiles: torch.Tensor
@@ -196,17 +197,18 @@ def permute_plan(ids_TK, num_experts, local_lo=0, local_hi=None, align=1) -> Per
     tile_row0 = small[o:o + tile_cap]; o += tile_cap
     num_tiles = small[o:o + 1]
     row_of_slot = torch.empty(N, **i32)
-    slot_of_row = torch.empty(row_cap, **i32)
+    rows2 = torch.empty(2, row_cap, **i32)
+    slot_of_row, token_of_row = rows2[0], rows2[1]
     ws = torch.empty(lib.mi355_permute_plan_workspace_bytes(T, K, E), dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
         rc = lib.mi355_permute_plan(
             _p(ids_TK), T, K, E, lo, hi, align, tm, _p(counts_E), _p(seg_offsets), _p(seg_counts),
-            _p(row_of_slot), _p(slot_of_row), row_cap, _p(tile_expert), _p(tile_row0),
+            _p(row_of_slot), _p(slot_of_row), _p(token_of_row), row_cap, _p(tile_expert), _p(tile_row0),
             _p(num_tiles), tile_cap, _p(ws), _stream(dev),
         )
     _lib.check(rc, "permute_plan")
     return PermutePlan(T, K, E, lo, hi, align, tm, row_cap, tile_cap, counts_E, seg_offsets,
-                       seg_counts, row_of_slot, slot_of_row, tile_expert, tile_row0, num_tiles)
+                       seg_counts, row_of_slot, slot_of_row, token_of_row, tile_expert, tile_row0, num_tiles)
 
 
 def segments_from_counts(counts_e, total_rows: int) -> PermutePlan:
@@ -231,7 +233,7 @@ def segments_from_counts(counts_e, total_rows: int) -> PermutePlan:
         )
     _lib.check(rc, "segments_from_counts")
     return PermutePlan(0, 1, El, 0, El, 1, tm, total_rows, tile_cap, None, seg_offsets, seg_counts,
-                       None, None, tile_expert, tile_row0, num_tiles)
+                       None, None, None, tile_expert, tile_row0, num_tiles)
 
 
 # ------------------------------------------------------------------ row movers
@@ -297,10 +299,20 @@ def combine_bwd(dout_TD, y_RD, weights_TK, plan: PermutePlan, zero_padding=True)
 
 
 # ------------------------------------------------------------------ experts
-def grouped_swiglu_fwd(rows_RD, w1_EFD, w3_EFD, w2_EDF, plan: PermutePlan):
+def gather_supported(x_TD, hidden_dim: int) -> bool:
+    """The fused token gather exists for the bf16 MFMA kernels (D, F multiples of 64)."""
+    D = x_TD.shape[-1]
+    return (x_TD.dtype == torch.bfloat16 and D % 64 == 0 and hidden_dim % 64 == 0
+            and x_TD.shape[0] * D < 2**31)
+
+
+def grouped_swiglu_fwd(rows_RD, w1_EFD, w3_EFD, w2_EDF, plan: PermutePlan, gather=False):
+    """``gather=True``: ``rows_RD`` is the (T, D) token matrix, read through ``plan.token_of_row``."""
     dev = _dev(rows_RD, w1_EFD, w3_EFD, w2_EDF)
     rows_RD, w1_EFD, w3_EFD, w2_EDF = _c(rows_RD), _c(w1_EFD), _c(w3_EFD), _c(w2_EDF)
-    R, D = rows_RD.shape
+    D = rows_RD.shape[1]
+    R = plan.row_capacity if gather else rows_RD.shape[0]
+    tok = plan.token_of_row if gather else None
     El, F, D2 = w1_EFD.shape
     if D2 != D or w3_EFD.shape != w1_EFD.shape or w2_EDF.shape != (El, D, F):
         raise ValueError("expert weight shapes do not match (E,F,D)/(E,F,D)/(E,D,F)")
@@ -312,30 +324,33 @@ def grouped_swiglu_fwd(rows_RD, w1_EFD, w3_EFD, w2_EDF, plan: PermutePlan):
     gate, up, h, y = mk(F), mk(F), mk(F), mk(D)
     with torch.cuda.device(dev):
         rc = _lib.load().mi355_grouped_swiglu_fwd(
-            _p(rows_RD), _p(w1_EFD), _p(w3_EFD), _p(w2_EDF), _dt(rows_RD), _p(plan.seg_offsets),
-            _p(plan.seg_counts), _p(plan.tile_expert), _p(plan.tile_row0), _p(plan.num_tiles),
-            plan.tile_capacity, _p(gate), _p(up), _p(h), _p(y), El, D, F, R, _stream(dev),
+            _p(rows_RD), _p(tok), _p(w1_EFD), _p(w3_EFD), _p(w2_EDF), _dt(rows_RD),
+            _p(plan.seg_offsets), _p(plan.seg_counts), _p(plan.tile_expert), _p(plan.tile_row0),
+            _p(plan.num_tiles), plan.tile_capacity, _p(gate), _p(up), _p(h), _p(y), El, D, F, R,
+            _stream(dev),
         )
     _lib.check(rc, "grouped_swiglu_fwd")
     return y, gate, up, h
 
 
 def grouped_swiglu_bwd(dy_RD, rows_RD, w1_EFD, w3_EFD, w2_EDF, gate, up, h, plan: PermutePlan,
-                       need_drows=True, need_dw=True):
+                       need_drows=True, need_dw=True, gather=False):
     dev = _dev(dy_RD, rows_RD)
     dy_RD = _c(dy_RD)
     w1_EFD, w3_EFD, w2_EDF = _c(w1_EFD), _c(w3_EFD), _c(w2_EDF)
-    R, D = rows_RD.shape
+    D = rows_RD.shape[1]
+    R = dy_RD.shape[0]
+    tok = plan.token_of_row if gather else None
     El, F, _ = w1_EFD.shape
     dgate, dup = torch.empty_like(gate), torch.empty_like(up)
-    drows = torch.empty_like(rows_RD) if need_drows else None
+    drows = torch.empty(R, D, dtype=rows_RD.dtype, device=dev) if need_drows else None
     dw1 = torch.empty_like(w1_EFD) if need_dw else None
     dw3 = torch.empty_like(w3_EFD) if need_dw else None
     dw2 = torch.empty_like(w2_EDF) if need_dw else None
     with torch.cuda.device(dev):
         rc = _lib.load().mi355_grouped_swiglu_bwd(
-            _p(dy_RD), _p(rows_RD), _p(w1_EFD), _p(w3_EFD), _p(w2_EDF), _p(gate), _p(up), _p(h),
-            _dt(rows_RD), _p(plan.seg_offsets), _p(plan.seg_counts), _p(plan.tile_expert),
+            _p(dy_RD), _p(rows_RD), _p(tok), _p(w1_EFD), _p(w3_EFD), _p(w2_EDF), _p(gate), _p(up),
+            _p(h), _dt(rows_RD), _p(plan.seg_offsets), _p(plan.seg_counts), _p(plan.tile_expert),
             _p(plan.tile_row0), _p(plan.num_tiles), plan.tile_capacity, _p(dgate), _p(dup),
             _p(drows), _p(dw1), _p(dw3), _p(dw2), El, D, F, R, _stream(dev),
         )
@@ -354,12 +369,13 @@ def grouped_swiglu_stage(stage: str, buf: dict, plan: PermutePlan):
     """
     rows = buf["rows"]
     dev = _dev(rows)
-    R, D = rows.shape
+    D = rows.shape[1]
+    R = buf["gate"].shape[0]
     El, F, _ = buf["w1"].shape
     g = lambda k: _p(buf.get(k))
     with torch.cuda.device(dev):
         rc = _lib.load().mi355_grouped_swiglu_stage(
-            STAGES[stage], g("dy"), g("rows"), g("w1"), g("w3"), g("w2"), g("gate"), g("up"), g("h"),
+            STAGES[stage], g("dy"), g("rows"), g("token_of_row"), g("w1"), g("w3"), g("w2"), g("gate"), g("up"), g("h"),
             g("y"), _p(plan.seg_offsets), _p(plan.seg_counts), _p(plan.tile_expert),
             _p(plan.tile_row0), _p(plan.num_tiles), plan.tile_capacity, g("dgate"), g("dup"),
             g("drows"), g("dw1"), g("dw3"), g("dw2"), El, D, F, R, _stream(dev),
