@@ -26,6 +26,14 @@ if ROOT not in sys.path:
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 
+# HBM bytes per launch at the default workload, measured with rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE (scaled by a 256 MiB copy: x2.0 and x1.0); the table these come from is
+# profiles/moe_layer_qwen3_t8192_hbm_traffic.txt.  Only reported for the default workload.
+MEASURED_HBM_BYTES = {
+    "gate_up": 1646.5e6, "down": 946.3e6, "dh": 1253.3e6, "drows": 1623.5e6,
+    "dw2": 886.7e6, "dw1": 886.7e6, "dw3": 886.7e6,
+}
+
 WORKLOADS = {
     # name: T, D, E, K, F
     "qwen3-30b-a3b-moe-layer fwd+bwd T=8192 bf16": dict(T=8192, D=2048, E=128, K=8, F=768),
@@ -41,6 +49,8 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-tokens", type=int, default=1024)
     ap.add_argument("--stage-iters", type=int, default=10)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 256 MiB device-to-device copy (known traffic, for scaling rocprof FETCH_SIZE / WRITE_SIZE)")
     return ap.parse_args()
 
 
@@ -197,7 +207,7 @@ def main():
         "peak": PEAK_BF16_TFLOPS,
         "unit": "TFLOP/s",
         "frac": round(ach / PEAK_BF16_TFLOPS, 4),
-        "traffic": None,
+        "traffic": MEASURED_HBM_BYTES.get(dominant) if T == 8192 else None,
         "avg_launch_ms": round(stage_ms[dominant], 4),
         "all_grouped_gemms": {"TFLOP/s": round(gemm_flops / (gemm_ms * 1e-3) / 1e12, 1),
                               "frac": round(gemm_flops / (gemm_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4)},
@@ -222,6 +232,11 @@ def main():
         "roofline": roofline,
         "kernels": kernels,
     }
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(cfg, args.cpu_sample_tokens)
     print(json.dumps(result))
