@@ -33,10 +33,8 @@ __device__ inline void Vec<uint16_t>::unpack(const uint4& v, float (&f)[8]) {
 }
 template <>
 __device__ inline uint4 Vec<uint16_t>::pack(const float (&f)[8]) {
-  return make_uint4(f32_to_bf16(f[0]) | (uint32_t)f32_to_bf16(f[1]) << 16,
-                    f32_to_bf16(f[2]) | (uint32_t)f32_to_bf16(f[3]) << 16,
-                    f32_to_bf16(f[4]) | (uint32_t)f32_to_bf16(f[5]) << 16,
-                    f32_to_bf16(f[6]) | (uint32_t)f32_to_bf16(f[7]) << 16);
+  return make_uint4(pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
+                    pack_bf16x2(f[6], f[7]));
 }
 
 template <typename T>

@@ -31,11 +31,16 @@ inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s);
 __device__ __forceinline__ float bf16_to_f32(uint16_t v) {
   return __uint_as_float(static_cast<uint32_t>(v) << 16);
 }
+// gfx950 converts in hardware (v_cvt_pk_bf16_f32, round to nearest even, NaN stays NaN).
+typedef __bf16 mi355_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float mi355_f32x2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x40u);  // NaN
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return static_cast<uint16_t>(u >> 16);
+  return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));
+}
+// {lo, hi} -> one dword holding bf16(lo) | bf16(hi) << 16
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  const mi355_f32x2 v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, mi355_bf16x2));
 }
 __device__ __forceinline__ float round_bf16(float f) { return bf16_to_f32(f32_to_bf16(f)); }
 

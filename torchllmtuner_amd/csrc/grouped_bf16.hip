@@ -41,6 +41,7 @@
 //       c ^ ((k & 3) << 1); a fragment is two ds_read_b64_tr_b16 (LDS transpose
 //       reads: lane i of a 16-lane group supplies the address of row i/4, 8-byte
 //       piece i%4, and receives column i of the four rows).
+#include <algorithm>
 #include <cstdlib>
 #include <type_traits>
 
@@ -97,8 +98,12 @@ __device__ __forceinline__ void phase_barrier() {
   __builtin_amdgcn_sched_barrier(0);
 }
 
-__device__ __forceinline__ uint32_t pack2(float a, float b) {
-  return static_cast<uint32_t>(f32_to_bf16(a)) | (static_cast<uint32_t>(f32_to_bf16(b)) << 16);
+__device__ __forceinline__ uint32_t pack2(float a, float b) { return pack_bf16x2(a, b); }
+
+// 1 / (1 + e^-x) on the transcendental unit (v_exp_f32, v_rcp_f32: about 1 ulp each; every
+// use is rounded to bf16 right after)
+__device__ __forceinline__ float fast_sigmoid(float x) {
+  return __builtin_amdgcn_rcpf(1.0f + __expf(-x));
 }
 
 // ---- epilogue staging -----------------------------------------------------------------
@@ -156,10 +161,16 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
   constexpr bool B_KS = (MODE == RM_DH || MODE == RM_DX);
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
 
+  // Persistent workgroups: block b serves XCD b % 8 and walks that XCD's contiguous run
+  // of the tile list with stride gridDim/8, the order in which the hardware dispatcher
+  // would have started one-tile blocks.  A tile's stores drain while the next tile's
+  // operands are fetched, and no workgroup launch sits between two tiles.
   const int num_tiles = *p.num_tiles;
   const int total = num_tiles * p.n_tiles;
-  const int pid = xcd_remap(blockIdx.x, total);
-  if (pid < 0) return;
+  const int chunk = (total + 7) >> 3;
+  for (int within = blockIdx.x >> 3; within < chunk; within += gridDim.x >> 3) {
+  const int pid = (blockIdx.x & 7) * chunk + within;
+  if (pid >= total) break;
   const int tile = pid / p.n_tiles, nt = pid % p.n_tiles;
   const int e = p.tile_expert[tile];
   const int row0 = p.tile_row0[tile];
@@ -299,6 +310,16 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
     const uint16_t* bb2 = has_next2 ? b_ptr(kofs(ks + 2)) : nullptr;
 #pragma unroll
     for (int kk = 0; kk < BK / 16; ++kk) {
+      bf16x8 af[2], bf[NJ];
+#pragma unroll
+      for (int mi = 0; mi < 2; ++mi) af[mi] = frag_kc(As, wm + mi * 32, kk, lane);
+#pragma unroll
+      for (int nj = 0; nj < NJ; ++nj) {
+        if constexpr (B_KS)
+          bf[nj] = frag_ks<BNT>(Bs, bcol[nj], kk, lane);
+        else
+          bf[nj] = frag_kc(Bs, bcol[nj], kk, lane);
+      }
       // a quarter of the staging traffic rides along with each quarter of the MFMAs:
       // park the held chunks of tile ks+1 in the other LDS stage, then refill the
       // same registers with the same chunks of tile ks+2.
@@ -316,39 +337,20 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
           rb[i] = *reinterpret_cast<const u32x4*>(bb2 + x + b_off[i]);
         }
       }
-      bf16x8 af[2], bf[NJ];
-#pragma unroll
-      for (int mi = 0; mi < 2; ++mi) af[mi] = frag_kc(As, wm + mi * 32, kk, lane);
-#pragma unroll
-      for (int nj = 0; nj < NJ; ++nj) {
-        if constexpr (B_KS)
-          bf[nj] = frag_ks<BNT>(Bs, bcol[nj], kk, lane);
-        else
-          bf[nj] = frag_kc(Bs, bcol[nj], kk, lane);
-      }
-      // end of the memory phase: this wave's LDS traffic has landed; swap roles with the
-      // sibling group, which has just finished issuing its MFMAs
-      phase_barrier();
 #pragma unroll
       for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
         for (int nj = 0; nj < NJ; ++nj)
           acc[mi][nj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[nj], af[mi], acc[mi][nj], 0, 0, 0);
-      phase_barrier();
     }
+    __syncthreads();
   };
   using T_ = std::true_type;
   using F_ = std::false_type;
-  // Ping-pong: waves 4..7 run one phase behind waves 0..3 (wave w and w+4 share a SIMD),
-  // so each SIMD always has one wave in its MFMA phase while the other parks, fetches
-  // and reads fragments.  Every wave executes the same number of barriers.
-  if (wave >= 4) phase_barrier();
   int ks = 0;
   for (; ks + 2 < ksteps; ++ks) kstep(ks, T_{}, T_{});
   if (ks + 1 < ksteps) { kstep(ks, T_{}, F_{}); ++ks; }
   if (ks < ksteps) kstep(ks, F_{}, F_{});
-  if (wave < 4) phase_barrier();
-  __syncthreads();
 
   // ---- epilogue: through the wave's private LDS region, 16-byte coalesced rows ---------
   // acc[mi][nj][i]: output row = wm + mi*32 + (lane&31); output column within the nj-th
@@ -371,7 +373,7 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
           for (int r = 0; r < 4; ++r) {
             g[r] = round_bf16(acc[mi][j][q * 4 + r]);
             u[r] = round_bf16(acc[mi][j + 2][q * 4 + r]);
-            const float s = round_bf16(g[r] / (1.0f + __expf(-g[r])));
+            const float s = round_bf16(g[r] * fast_sigmoid(g[r]));
             h[r] = s * u[r];
           }
           S::put4(sg, 0, j * 32, lane, q, g[0], g[1], g[2], g[3]);
@@ -432,7 +434,7 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
               const float dh = __uint_as_float(hlf ? (v[w] & 0xffff0000u) : (v[w] << 16));
               const float g = __uint_as_float(hlf ? (gv[w] & 0xffff0000u) : (gv[w] << 16));
               const float u = __uint_as_float(hlf ? (uv[w] & 0xffff0000u) : (uv[w] << 16));
-              const float sig = 1.0f / (1.0f + __expf(-g));
+              const float sig = fast_sigmoid(g);
               const float s = round_bf16(g * sig);
               const float ds = round_bf16(dh * u);
               r_du[hlf] = dh * s;
@@ -448,6 +450,8 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
         }
       }
     }
+  }
+  __syncthreads();  // every wave is done with its staging region before the next tile's operands land
   }
 }
 
@@ -613,6 +617,19 @@ enum { STAGE_GATEUP = 1, STAGE_DOWN = 2, STAGE_DH = 4, STAGE_DX = 8, STAGE_DW2 =
 
 static unsigned round8(int64_t v) { return static_cast<unsigned>((v + 7) / 8 * 8); }
 
+// One workgroup per CU (a workgroup takes the whole LDS), rounded to whole XCD rounds.
+static unsigned resident_blocks() {
+  static unsigned n = 0;
+  if (n == 0) {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 8)
+      cus = 256;
+    n = static_cast<unsigned>(cus / 8 * 8);
+  }
+  return n;
+}
+
 constexpr int R_LDS_BYTES = 2 * R_STAGE * 2;  // 163840
 constexpr int W_LDS_BYTES = 8 * 64 * 136 * 2;  // 139264: the 8 epilogue regions (> 2 stages = 131072)
 
@@ -623,7 +640,8 @@ static int launch_row(RowArgs& a, int64_t tile_capacity, hipStream_t s, const ch
     if (int rc = set_lds(row_tiled_kernel<MODE, NJ>, R_LDS_BYTES)) return rc;
     configured = true;
   }
-  hipLaunchKernelGGL((row_tiled_kernel<MODE, NJ>), dim3(round8(tile_capacity * a.n_tiles)), dim3(NT), R_LDS_BYTES, s, a);
+  const unsigned blocks = std::min(round8(tile_capacity * a.n_tiles), resident_blocks());
+  hipLaunchKernelGGL((row_tiled_kernel<MODE, NJ>), dim3(blocks), dim3(NT), R_LDS_BYTES, s, a);
   return check_launch(what);
 }
 

@@ -257,10 +257,8 @@ __device__ __forceinline__ uint4 pack_vec<float>(const float (&a)[4]) {
 }
 template <>
 __device__ __forceinline__ uint4 pack_vec<uint16_t>(const float (&a)[8]) {
-  return make_uint4(f32_to_bf16(a[0]) | (uint32_t)f32_to_bf16(a[1]) << 16,
-                    f32_to_bf16(a[2]) | (uint32_t)f32_to_bf16(a[3]) << 16,
-                    f32_to_bf16(a[4]) | (uint32_t)f32_to_bf16(a[5]) << 16,
-                    f32_to_bf16(a[6]) | (uint32_t)f32_to_bf16(a[7]) << 16);
+  return make_uint4(pack_bf16x2(a[0], a[1]), pack_bf16x2(a[2], a[3]), pack_bf16x2(a[4], a[5]),
+                    pack_bf16x2(a[6], a[7]));
 }
 
 template <typename T>
