@@ -474,8 +474,11 @@ struct WgradArgs {
 
 __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
-  const int pid = xcd_remap(blockIdx.x, p.total);
-  if (pid < 0) return;
+  // persistent workgroups, same walk as the row-tiled kernels
+  const int chunk = (p.total + 7) >> 3;
+  for (int within = blockIdx.x >> 3; within < chunk; within += gridDim.x >> 3) {
+  const int pid = (blockIdx.x & 7) * chunk + within;
+  if (pid >= p.total) break;
   const int per_e = p.m_tiles * p.n_tiles;
   const int e = pid / per_e;
   const int rem = pid % per_e;
@@ -599,6 +602,8 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
       *reinterpret_cast<u32x4*>(C + static_cast<int64_t>(m) * N + n) =
           *reinterpret_cast<const u32x4*>(st + (idx >> 4) * S::PITCH + (idx & 15) * 8);
   }
+  __syncthreads();  // staging regions are free again before the next tile's operands land
+  }
 }
 
 template <typename K>
@@ -721,7 +726,7 @@ int bf16_grouped_bwd(const void* dy, const void* rows, const int32_t* token_of_r
     w.seg_offsets = seg_offsets; w.seg_counts = seg_counts; w.M = (int)M; w.N = (int)N;
     w.m_tiles = (int)((M + WBM - 1) / WBM); w.n_tiles = (int)((N + WBN - 1) / WBN);
     w.total = (int)(El * w.m_tiles * w.n_tiles);
-    hipLaunchKernelGGL(wgrad_kernel, dim3(round8(w.total)), dim3(NT), W_LDS_BYTES, s, w);
+    hipLaunchKernelGGL(wgrad_kernel, dim3(std::min(round8(w.total), resident_blocks())), dim3(NT), W_LDS_BYTES, s, w);
     return check_launch(what);
   };
   if (dw2 && (stages & STAGE_DW2)) if (int rc = wgrad(dy, h, nullptr, dw2, D, F, "grouped dw2")) return rc;
