@@ -89,8 +89,8 @@ __device__ __forceinline__ int xcd_remap(int bid, int total) {
   return (within < chunk && pid < total) ? pid : -1;
 }
 
-// Barrier between the memory phase and the MFMA phase of the ping-pong schedule: wait
-// for this wave's own LDS operations only (global loads stay in flight), then s_barrier.
+// Workgroup barrier that waits for this wave's own LDS operations only: global loads and
+// stores stay in flight across it.
 __device__ __forceinline__ void phase_barrier() {
   __builtin_amdgcn_sched_barrier(0);
   __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
@@ -474,33 +474,14 @@ struct WgradArgs {
 
 __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
-  // persistent workgroups, same walk as the row-tiled kernels
-  const int chunk = (p.total + 7) >> 3;
-  for (int within = blockIdx.x >> 3; within < chunk; within += gridDim.x >> 3) {
-  const int pid = (blockIdx.x & 7) * chunk + within;
-  if (pid >= p.total) break;
-  const int per_e = p.m_tiles * p.n_tiles;
-  const int e = pid / per_e;
-  const int rem = pid % per_e;
-  const int mt = rem / p.n_tiles, nt = rem % p.n_tiles;
-  const int m0 = mt * WBM, n0 = nt * WBN;
-  const int M = p.M, N = p.N;
-  const int seg0 = p.seg_offsets[e], cnt = p.seg_counts[e];
-
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = (wave >> 1) * 64, wn = (wave & 1) * 128;
+  const int M = p.M, N = p.N;
+  const int per_e = p.m_tiles * p.n_tiles;
 
   // KS tiles of 256 columns = 32 chunks per k row: k = (tid>>5) + 16*i, chunk tid&31
   u32x4 ra[4], rb[4];
   const int ks_k = tid >> 5, ks_chunk = tid & 31;
-  const uint16_t* a_base = p.a + static_cast<int64_t>(seg0) * M + min(m0 + ks_chunk * 8, M - 8);
-  const uint16_t* b_base = p.b + (p.b_src ? 0 : static_cast<int64_t>(seg0) * N) + min(n0 + ks_chunk * 8, N - 8);
-  // With a gather, the source row of B's k-th row comes from an index array.  The
-  // indices of the step after the one being fetched are loaded one step early (tk), so
-  // no data load waits on an index load in the steady state.
-  const int32_t* b_src = p.b_src ? p.b_src + seg0 : nullptr;
-  auto src_row = [&](int k) -> int { return (b_src && k < cnt) ? max(b_src[k], 0) : k; };
-  int tk[4];
   int lds_off[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -509,100 +490,149 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
   }
   const u32x4 zero = {0, 0, 0, 0};
 
-  f32x16 acc[2][4];
-#pragma unroll
-  for (int mi = 0; mi < 2; ++mi)
-#pragma unroll
-    for (int nj = 0; nj < 4; ++nj)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) acc[mi][nj][i] = 0.0f;
+  // Persistent workgroups, same walk as the row-tiled kernels.  The K extent is one
+  // expert's rows (a handful of 64-row steps), so what surrounds the K loop matters: the
+  // first operands of the next tile are requested before the epilogue of the current one
+  // and land while it runs.
+  const int chunk = (p.total + 7) >> 3;
+  const int stride = gridDim.x >> 3;
+  int within = blockIdx.x >> 3;
+  int pid = (blockIdx.x & 7) * chunk + within;
+  if (within >= chunk || pid >= p.total) return;
 
-  const int ksteps = (cnt + BK - 1) / BK;
-  if (ksteps > 0) {
+  // state of the tile whose operands are being fetched
+  int e = pid / per_e;
+  int m0 = ((pid % per_e) / p.n_tiles) * WBM, n0 = ((pid % per_e) % p.n_tiles) * WBN;
+  int cnt = p.seg_counts[e];
+  const uint16_t* a_base;
+  const uint16_t* b_base;
+  const int32_t* b_src;
+  auto set_bases = [&](int seg0) {
+    a_base = p.a + static_cast<int64_t>(seg0) * M + min(m0 + ks_chunk * 8, M - 8);
+    b_base = p.b + (p.b_src ? 0 : static_cast<int64_t>(seg0) * N) + min(n0 + ks_chunk * 8, N - 8);
+    b_src = p.b_src ? p.b_src + seg0 : nullptr;
+  };
+  // Loads of one K step, unconditional: rows past the segment re-read its last row and
+  // the A side is zeroed when it is parked, so the products vanish.  Needs cnt > 0.
+  auto issue = [&](int step) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int k = ks_k + 16 * i;
-      ra[i] = k < cnt ? *reinterpret_cast<const u32x4*>(a_base + static_cast<int64_t>(k) * M) : zero;
-      rb[i] = k < cnt ? *reinterpret_cast<const u32x4*>(b_base + static_cast<int64_t>(src_row(k)) * N) : zero;
+      const int k = min(step * BK + ks_k + 16 * i, cnt - 1);
+      ra[i] = *reinterpret_cast<const u32x4*>(a_base + static_cast<int64_t>(k) * M);
+      const int kb = b_src ? max(b_src[k], 0) : k;
+      rb[i] = *reinterpret_cast<const u32x4*>(b_base + static_cast<int64_t>(kb) * N);
     }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      *reinterpret_cast<u32x4*>(smem + lds_off[i]) = ra[i];
-      *reinterpret_cast<u32x4*>(smem + WBM * BK + lds_off[i]) = rb[i];
-    }
-    if (ksteps > 1) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int k = BK + ks_k + 16 * i;
-        ra[i] = k < cnt ? *reinterpret_cast<const u32x4*>(a_base + static_cast<int64_t>(k) * M) : zero;
-        rb[i] = k < cnt ? *reinterpret_cast<const u32x4*>(b_base + static_cast<int64_t>(src_row(k)) * N) : zero;
-      }
-    }
-  }
-#pragma unroll
-  for (int i = 0; i < 4; ++i) tk[i] = src_row(2 * BK + ks_k + 16 * i);
-  __syncthreads();
+  };
+  auto park = [&](int step, int i, uint16_t* An, uint16_t* Bn, int count) {
+    const bool live = step * BK + ks_k + 16 * i < count;
+    *reinterpret_cast<u32x4*>(An + lds_off[i]) = live ? ra[i] : zero;
+    *reinterpret_cast<u32x4*>(Bn + lds_off[i]) = rb[i];
+  };
+  set_bases(p.seg_offsets[e]);
+  if (cnt > 0) issue(0);
 
-  // The K extent here is one expert's rows (a handful of 64-row steps), so the loop is
-  // kept simple: one barrier per step, next tile parked and the one after fetched while
-  // the MFMAs of the current tile issue.
-  for (int ks = 0; ks < ksteps; ++ks) {
-    const uint16_t* As = smem + (ks & 1) * W_STAGE;
-    const uint16_t* Bs = As + WBM * BK;
-    uint16_t* An = smem + ((ks + 1) & 1) * W_STAGE;
-    uint16_t* Bn = An + WBM * BK;
-    const bool has_next = ks + 1 < ksteps;
-    const bool has_next2 = ks + 2 < ksteps;
-    const int kbase2 = (ks + 2) * BK;
+  for (;;) {
+    // the tile after this one: its segment is looked up now and used after the K loop
+    const int nwithin = within + stride;
+    const int npid = (blockIdx.x & 7) * chunk + nwithin;
+    const bool more = nwithin < chunk && npid < p.total;
+    const int fpid = more ? npid : pid;
+    const int ne = fpid / per_e;
+    const int nseg0 = p.seg_offsets[ne], ncnt = p.seg_counts[ne];
+    const int c_e = e, c_m0 = m0, c_n0 = n0, c_cnt = cnt;
+    const int ksteps = (cnt + BK - 1) / BK;
+
+    f32x16 acc[2][4];
 #pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk) {
-      if (has_next) {
-        *reinterpret_cast<u32x4*>(An + lds_off[kk]) = ra[kk];
-        *reinterpret_cast<u32x4*>(Bn + lds_off[kk]) = rb[kk];
-      }
-      if (has_next2) {
-        const int k = kbase2 + ks_k + 16 * kk;
-        ra[kk] = k < cnt ? *reinterpret_cast<const u32x4*>(a_base + static_cast<int64_t>(k) * M) : zero;
-        rb[kk] = k < cnt ? *reinterpret_cast<const u32x4*>(b_base + static_cast<int64_t>(b_src ? tk[kk] : k) * N) : zero;
-        tk[kk] = src_row(k + BK);
-      }
-      bf16x8 af[2], bf[4];
+    for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
-      for (int mi = 0; mi < 2; ++mi) af[mi] = frag_ks<256>(As, wm + mi * 32, kk, lane);
+      for (int nj = 0; nj < 4; ++nj)
 #pragma unroll
-      for (int nj = 0; nj < 4; ++nj) bf[nj] = frag_ks<256>(Bs, wn + nj * 32, kk, lane);
+        for (int i = 0; i < 16; ++i) acc[mi][nj][i] = 0.0f;
+
+    if (ksteps > 0) {
 #pragma unroll
-      for (int mi = 0; mi < 2; ++mi)
-#pragma unroll
-        for (int nj = 0; nj < 4; ++nj)
-          acc[mi][nj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[nj], af[mi], acc[mi][nj], 0, 0, 0);
-      __builtin_amdgcn_sched_barrier(0);
+      for (int i = 0; i < 4; ++i) park(0, i, smem, smem + WBM * BK, c_cnt);
+      if (ksteps > 1) issue(1);
     }
     __syncthreads();
-  }
 
-  using S = WaveStage<128>;
-  uint16_t* st = smem + wave * S::ELEMS;
+    // One K step: a quarter of the staging rides along with each quarter of the MFMAs.
+    // The flags are compile-time so that the loads of the steady state are unconditional
+    // and the compiler counts outstanding loads exactly.
+    auto kstep = [&](int ks, auto has_next_t, auto has_next2_t) {
+      constexpr bool has_next = decltype(has_next_t)::value;
+      constexpr bool has_next2 = decltype(has_next2_t)::value;
+      const uint16_t* As = smem + (ks & 1) * W_STAGE;
+      const uint16_t* Bs = As + WBM * BK;
+      uint16_t* An = smem + ((ks + 1) & 1) * W_STAGE;
+      uint16_t* Bn = An + WBM * BK;
 #pragma unroll
-  for (int mi = 0; mi < 2; ++mi)
+      for (int kk = 0; kk < BK / 16; ++kk) {
+        bf16x8 af[2], bf[4];
 #pragma unroll
-    for (int nj = 0; nj < 4; ++nj)
+        for (int mi = 0; mi < 2; ++mi) af[mi] = frag_ks<256>(As, wm + mi * 32, kk, lane);
 #pragma unroll
-      for (int q = 0; q < 4; ++q)
-        S::put4(st, mi, nj * 32, lane, q, acc[mi][nj][q * 4], acc[mi][nj][q * 4 + 1],
-                acc[mi][nj][q * 4 + 2], acc[mi][nj][q * 4 + 3]);
-  __builtin_amdgcn_s_waitcnt(0xc07f);
-  __builtin_amdgcn_wave_barrier();
-  uint16_t* C = p.c + static_cast<int64_t>(e) * M * N;
+        for (int nj = 0; nj < 4; ++nj) bf[nj] = frag_ks<256>(Bs, wn + nj * 32, kk, lane);
+        if constexpr (has_next) park(ks + 1, kk, An, Bn, c_cnt);
+        if constexpr (has_next2) {
+          const int k = min((ks + 2) * BK + ks_k + 16 * kk, c_cnt - 1);
+          ra[kk] = *reinterpret_cast<const u32x4*>(a_base + static_cast<int64_t>(k) * M);
+          const int kb = b_src ? max(b_src[k], 0) : k;
+          rb[kk] = *reinterpret_cast<const u32x4*>(b_base + static_cast<int64_t>(kb) * N);
+        }
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+          for (int nj = 0; nj < 4; ++nj)
+            acc[mi][nj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[nj], af[mi], acc[mi][nj], 0, 0, 0);
+      }
+      __syncthreads();
+    };
+    using T_ = std::true_type;
+    using F_ = std::false_type;
+    int ks = 0;
+    for (; ks + 2 < ksteps; ++ks) kstep(ks, T_{}, T_{});
+    if (ks + 1 < ksteps) { kstep(ks, T_{}, F_{}); ++ks; }
+    if (ks < ksteps) kstep(ks, F_{}, F_{});
+
+    // switch the fetch state to the next tile and request its first K step
+    if (more) {
+      e = ne;
+      m0 = ((npid % per_e) / p.n_tiles) * WBM;
+      n0 = ((npid % per_e) % p.n_tiles) * WBN;
+      cnt = ncnt;
+      set_bases(nseg0);
+      if (cnt > 0) issue(0);
+    }
+
+    using S = WaveStage<128>;
+    uint16_t* st = smem + wave * S::ELEMS;
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+      for (int nj = 0; nj < 4; ++nj)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          S::put4(st, mi, nj * 32, lane, q, acc[mi][nj][q * 4], acc[mi][nj][q * 4 + 1],
+                  acc[mi][nj][q * 4 + 2], acc[mi][nj][q * 4 + 3]);
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __builtin_amdgcn_wave_barrier();
+    uint16_t* C = p.c + static_cast<int64_t>(c_e) * M * N;
 #pragma unroll 4
-  for (int it = 0; it < 16; ++it) {
-    const int idx = it * 64 + lane;
-    const int m = m0 + wm + (idx >> 4), n = n0 + wn + (idx & 15) * 8;
-    if (m < M && n < N)
-      *reinterpret_cast<u32x4*>(C + static_cast<int64_t>(m) * N + n) =
-          *reinterpret_cast<const u32x4*>(st + (idx >> 4) * S::PITCH + (idx & 15) * 8);
-  }
-  __syncthreads();  // staging regions are free again before the next tile's operands land
+    for (int it = 0; it < 16; ++it) {
+      const int idx = it * 64 + lane;
+      const int m = c_m0 + wm + (idx >> 4), n = c_n0 + wn + (idx & 15) * 8;
+      if (m < M && n < N)
+        *reinterpret_cast<u32x4*>(C + static_cast<int64_t>(m) * N + n) =
+            *reinterpret_cast<const u32x4*>(st + (idx >> 4) * S::PITCH + (idx & 15) * 8);
+    }
+    // staging regions are free again before the next tile's operands are parked; only
+    // the LDS traffic is waited for, the tile's stores keep draining
+    phase_barrier();
+    if (!more) break;
+    within = nwithin;
+    pid = npid;
   }
 }
 
