@@ -153,41 +153,55 @@ struct RowArgs {
 constexpr int RBM = 128, RBN = 512;
 constexpr int R_STAGE = (RBM + RBN) * BK;  // elements per LDS stage (80 KiB)
 
-template <int MODE, int NJ>
+struct TileMeta {
+  int e, row0, valid, n0;
+};
+
+template <int MODE, int NJ, bool GATHER>
 __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
   constexpr int BNT = 128 * NJ;            // output columns of the tile (4 waves x NJ x 32)
   constexpr int NB = BNT / 64;             // 16-byte B chunks staged per thread and K step
   constexpr int STAGE = (RBM + BNT) * BK;  // elements per LDS stage
   constexpr bool B_KS = (MODE == RM_DH || MODE == RM_DX);
+  static_assert(!GATHER || MODE == RM_GATEUP, "only the gate/up product gathers its rows");
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
-
-  // Persistent workgroups: block b serves XCD b % 8 and walks that XCD's contiguous run
-  // of the tile list with stride gridDim/8, the order in which the hardware dispatcher
-  // would have started one-tile blocks.  A tile's stores drain while the next tile's
-  // operands are fetched, and no workgroup launch sits between two tiles.
-  const int num_tiles = *p.num_tiles;
-  const int total = num_tiles * p.n_tiles;
-  const int chunk = (total + 7) >> 3;
-  for (int within = blockIdx.x >> 3; within < chunk; within += gridDim.x >> 3) {
-  const int pid = (blockIdx.x & 7) * chunk + within;
-  if (pid >= total) break;
-  const int tile = pid / p.n_tiles, nt = pid % p.n_tiles;
-  const int e = p.tile_expert[tile];
-  const int row0 = p.tile_row0[tile];
-  const int valid = min(RBM, p.seg_offsets[e] + p.seg_counts[e] - row0);
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = (wave >> 2) * 64, wn = wave & 3;
   const int D = p.D, F = p.F;
-
   const int Kdim = (MODE == RM_GATEUP || MODE == RM_DH) ? D : (MODE == RM_DOWN ? F : 2 * F);
   const int lda = (MODE == RM_GATEUP || MODE == RM_DH) ? D : F;
   const int Ncols = (MODE == RM_GATEUP || MODE == RM_DH) ? F : D;  // output width
-  const int n0 = nt * (MODE == RM_GATEUP ? BNT / 2 : BNT);
   const int64_t wsz = static_cast<int64_t>(D) * F;
-  const uint16_t* B0 = p.b0 + e * wsz;
-  const uint16_t* B1 = (MODE == RM_GATEUP || MODE == RM_DX) ? p.b1 + e * wsz : B0;
-  const int64_t b1_off = B1 - B0;  // both weight stacks live in one flat address space
+  const int ksteps = Kdim / BK;
+
+  // Persistent workgroups: block b serves XCD b % 8 and walks that XCD's contiguous run
+  // of the tile list with stride gridDim/8, the order in which the hardware dispatcher
+  // would have started one-tile blocks.  Tile metadata is looked up two tiles ahead and
+  // the first operands of the next tile are requested before the epilogue of the current
+  // one, so neither lookup nor first fetch sits between two K loops; a tile's stores
+  // drain under the next tile's work.
+  const int num_tiles = *p.num_tiles;
+  const int total = num_tiles * p.n_tiles;
+  const int chunk = (total + 7) >> 3;
+  const int stride = gridDim.x >> 3;
+  const int pid_base = (blockIdx.x & 7) * chunk;
+  int within = blockIdx.x >> 3;
+  if (within >= chunk || pid_base + within >= total) return;
+  auto exists = [&](int w) { return w < chunk && pid_base + w < total; };
+  auto load_meta = [&](int w) -> TileMeta {
+    const int pid = pid_base + w;
+    const int tile = pid / p.n_tiles, nt = pid % p.n_tiles;
+    TileMeta m;
+    m.e = p.tile_expert[tile];
+    m.row0 = p.tile_row0[tile];
+    m.valid = min(RBM, p.seg_offsets[m.e] + p.seg_counts[m.e] - m.row0);
+    // a last tile that would overhang starts early instead and recomputes a few columns
+    // of its neighbour (same values), so no column is ever clamped
+    constexpr int W = (MODE == RM_GATEUP ? BNT / 2 : BNT);
+    m.n0 = min(nt * W, Ncols - W);
+    return m;
+  };
 
   // ---- global -> register staging: 16-byte chunks q = tid + 512*i ---------------------
   // KC tiles (8 chunks per row): row (tid>>3) + 64*i, chunk tid&7.
@@ -195,65 +209,18 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
   u32x4 ra[2], rb[NB];
   const int kc_row = tid >> 3, kc_chunk = tid & 7;
   const int kc_lds = kc_row * BK + ((kc_chunk ^ ((kc_row >> 1) & 7)) << 3);  // + i*64*BK (64 % 16 == 0)
-  const bool gather = (MODE == RM_GATEUP) && p.a_src != nullptr;
-  const uint16_t* a_base0 = p.a0 + (gather ? 0 : static_cast<int64_t>(row0) * lda) + kc_chunk * 8;
-  const uint16_t* a_base1 = (MODE == RM_DX) ? p.a1 + static_cast<int64_t>(row0) * lda + kc_chunk * 8 : a_base0;
-  int a_off[2];
-#pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int r = min(kc_row + 64 * i, valid - 1);
-    a_off[i] = (gather ? max(p.a_src[row0 + r], 0) : r) * lda;
-  }
-
-  const uint16_t* b_base = B0;
-  int b_off[NB];
   int b_lds[NB];
-  if constexpr (!B_KS) {
-    b_base += kc_chunk * 8;
 #pragma unroll
-    for (int i = 0; i < NB; ++i) {
-      const int r = kc_row + 64 * i;
-      if constexpr (MODE == RM_GATEUP)
-        b_off[i] = min(n0 + (r % (BNT / 2)), F - 1) * D;  // first half of the rows from w1, second from w3
-      else
-        b_off[i] = min(n0 + r, D - 1) * F;  // DOWN: w2[e] is (D,F); a tile row is an output column d
+  for (int i = 0; i < NB; ++i) {
+    if constexpr (!B_KS) {
       b_lds[i] = kc_lds + i * 64 * BK;
-    }
-  } else {
-    // DH: B(k=d, n=f) = w2[e][d][f], ld F.  DX: B(k=f, n=d) = w1/w3[e][f][d], ld D.
-    // (b_off carries both the k row and the clamped column of each chunk)
-    constexpr int CPR = BNT / 8;  // chunks per k row
-#pragma unroll
-    for (int i = 0; i < NB; ++i) {
+    } else {
+      constexpr int CPR = BNT / 8;  // chunks per k row
       const int q = tid + NT * i;
       const int k = q / CPR, cc = q % CPR;
-      b_off[i] = k * Ncols + min(n0 + cc * 8, Ncols - 8);
       b_lds[i] = k * BNT + ((cc ^ ((k & 3) << 1)) << 3);
     }
   }
-
-  // pointers for the K step being fetched
-  auto a_ptr = [&](int k0) -> const uint16_t* {
-    if constexpr (MODE == RM_DX) return (k0 >= F ? a_base1 + (k0 - F) : a_base0 + k0);
-    return a_base0 + k0;
-  };
-  auto b_ptr = [&](int k0) -> const uint16_t* {
-    if constexpr (MODE == RM_DX) {
-      const int kk0 = k0 >= F ? k0 - F : k0;
-      return b_base + (k0 >= F ? b1_off : 0) + static_cast<int64_t>(kk0) * Ncols;
-    }
-    if constexpr (B_KS) return b_base + static_cast<int64_t>(k0) * Ncols;
-    return b_base + k0;
-  };
-
-  f32x16 acc[2][NJ];
-#pragma unroll
-  for (int mi = 0; mi < 2; ++mi)
-#pragma unroll
-    for (int nj = 0; nj < NJ; ++nj)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) acc[mi][nj][i] = 0.0f;
-
   int bcol[NJ];
 #pragma unroll
   for (int nj = 0; nj < NJ; ++nj) {
@@ -263,35 +230,111 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
       bcol[nj] = wn * (32 * NJ) + nj * 32;
   }
 
-  const int ksteps = Kdim / BK;
-  auto kofs = [&](int ks) { return ks * BK; };
-  // prologue: tile 0 -> LDS stage 0, tile 1 -> registers
-  {
-    const uint16_t* ab = a_ptr(kofs(0));
-    const uint16_t* bb = b_ptr(kofs(0));
+  // Operand addresses are a wave-uniform 64-bit base (tile, K step, chunk index) plus a
+  // 32-bit per-thread byte offset, the form global loads take without any 64-bit vector
+  // arithmetic.  The B offsets never change; the A offsets follow the tile's rows.
+  constexpr bool B_REGULAR = !B_KS || (NT % (BNT / 8) == 0);  // chunk index -> fixed row stride
+  constexpr int NBV = B_REGULAR ? 1 : NB;
+  const int ldb = B_KS ? Ncols : (MODE == RM_GATEUP ? D : F);
+  uint32_t voffB[NBV];
+  if constexpr (!B_KS) {
+    voffB[0] = static_cast<uint32_t>(kc_row * ldb + kc_chunk * 8) * 2u;
+  } else {
+    constexpr int CPR = BNT / 8;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) ra[i] = *reinterpret_cast<const u32x4*>(ab + a_off[i]);
-#pragma unroll
-    for (int i = 0; i < NB; ++i) {
-      const int64_t x = (MODE == RM_GATEUP && i >= NB / 2) ? b1_off : 0;
-      rb[i] = *reinterpret_cast<const u32x4*>(bb + x + b_off[i]);
-    }
-#pragma unroll
-    for (int i = 0; i < 2; ++i) *reinterpret_cast<u32x4*>(smem + kc_lds + i * 64 * BK) = ra[i];
-#pragma unroll
-    for (int i = 0; i < NB; ++i) *reinterpret_cast<u32x4*>(smem + RBM * BK + b_lds[i]) = rb[i];
-    if (ksteps > 1) {
-      const uint16_t* ab1 = a_ptr(kofs(1));
-      const uint16_t* bb1 = b_ptr(kofs(1));
-#pragma unroll
-      for (int i = 0; i < 2; ++i) ra[i] = *reinterpret_cast<const u32x4*>(ab1 + a_off[i]);
-#pragma unroll
-      for (int i = 0; i < NB; ++i) {
-        const int64_t x = (MODE == RM_GATEUP && i >= NB / 2) ? b1_off : 0;
-        rb[i] = *reinterpret_cast<const u32x4*>(bb1 + x + b_off[i]);
-      }
+    for (int i = 0; i < NBV; ++i) {
+      const int q = tid + NT * i;
+      voffB[i] = static_cast<uint32_t>((q / CPR) * ldb + (q % CPR) * 8) * 2u;
     }
   }
+  // state of the tile whose operands are being fetched
+  const char* ubA0;  // A rows (k = 0)
+  const char* ubA1;  // DX: second half of the contraction (dup)
+  const char* ubB0;  // B tile origin in the first weight stack
+  int64_t b1_bytes;  // second weight stack - first (one flat address space)
+  uint32_t voffA[2];
+  // source rows of the A tile: the tile's own rows, or token rows through the gather index
+  auto load_asrc = [&](const TileMeta& m, int (&asrc)[2]) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int r = max(min(kc_row + 64 * i, m.valid - 1), 0);
+      asrc[i] = GATHER ? p.a_src[m.row0 + r] : r;
+    }
+  };
+  auto setup = [&](const TileMeta& m, const int (&asrc)[2]) {
+    const int64_t arow = GATHER ? 0 : static_cast<int64_t>(m.row0) * lda;
+    ubA0 = reinterpret_cast<const char*>(p.a0 + arow);
+    ubA1 = (MODE == RM_DX) ? reinterpret_cast<const char*>(p.a1 + arow) : ubA0;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) voffA[i] = static_cast<uint32_t>(max(asrc[i], 0) * lda + kc_chunk * 8) * 2u;
+    const uint16_t* B0 = p.b0 + m.e * wsz;
+    const uint16_t* B1 = (MODE == RM_GATEUP || MODE == RM_DX) ? p.b1 + m.e * wsz : B0;
+    b1_bytes = (B1 - B0) * 2;
+    // KC: the tile's first weight row is n0; KS: its first column is n0
+    ubB0 = reinterpret_cast<const char*>(B0 + (B_KS ? static_cast<int64_t>(m.n0) : static_cast<int64_t>(m.n0) * ldb));
+  };
+  // chunk i of the A / B tile of the K step that starts at k0
+  auto load_a = [&](int k0, int i) -> u32x4 {
+    const char* base = ubA0 + static_cast<int64_t>(k0) * 2;
+    if constexpr (MODE == RM_DX) base = (k0 >= F ? ubA1 + static_cast<int64_t>(k0 - F) * 2 : base);
+    return *reinterpret_cast<const u32x4*>(base + voffA[i]);
+  };
+  auto load_b = [&](int k0, int i) -> u32x4 {
+    const char* base = ubB0;
+    if constexpr (MODE == RM_GATEUP) {
+      // rows 0..BNT/2 of the tile come from w1, the rest from w3, same f range
+      base += (i >= NB / 2 ? b1_bytes : 0) + (static_cast<int64_t>(64 * (i % (NB / 2))) * ldb + k0) * 2;
+    } else if constexpr (MODE == RM_DOWN) {
+      base += (static_cast<int64_t>(64 * i) * ldb + k0) * 2;
+    } else {
+      int kk0 = k0;
+      if constexpr (MODE == RM_DX) {
+        if (k0 >= F) { kk0 = k0 - F; base += b1_bytes; }
+      }
+      base += static_cast<int64_t>(kk0 + (B_REGULAR ? i * (NT / (BNT / 8)) : 0)) * ldb * 2;
+    }
+    return *reinterpret_cast<const u32x4*>(base + voffB[B_REGULAR ? 0 : i]);
+  };
+  auto kofs = [&](int ks) { return ks * BK; };
+  // request every chunk of K step `step` of the fetch tile
+  auto issue = [&](int step) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) ra[i] = load_a(kofs(step), i);
+#pragma unroll
+    for (int i = 0; i < NB; ++i) rb[i] = load_b(kofs(step), i);
+  };
+
+  TileMeta cur = load_meta(within);
+  TileMeta nxt = load_meta(exists(within + stride) ? within + stride : within);
+  {
+    int asrc[2];
+    load_asrc(cur, asrc);
+    setup(cur, asrc);
+    issue(0);
+  }
+
+  for (;;) {
+  const bool more = exists(within + stride);
+  // the tile after the next: looked up now, used one tile later
+  const TileMeta nxt2 = load_meta(exists(within + 2 * stride) ? within + 2 * stride : within);
+  int nsrc[2];
+  load_asrc(nxt, nsrc);
+  const int row0 = cur.row0, valid = cur.valid, n0 = cur.n0;
+
+  f32x16 acc[2][NJ];
+#pragma unroll
+  for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+    for (int nj = 0; nj < NJ; ++nj)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[mi][nj][i] = 0.0f;
+
+  // K step 0 (requested before the previous epilogue) -> LDS stage 0, K step 1 -> registers
+#pragma unroll
+  for (int i = 0; i < 2; ++i) *reinterpret_cast<u32x4*>(smem + kc_lds + i * 64 * BK) = ra[i];
+#pragma unroll
+  for (int i = 0; i < NB; ++i) *reinterpret_cast<u32x4*>(smem + RBM * BK + b_lds[i]) = rb[i];
+  if (ksteps > 1) issue(1);
   __syncthreads();
 
   // One K step.  HAS_NEXT: the registers hold tile ks+1 and are parked in the other LDS
@@ -306,8 +349,6 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
     const uint16_t* Bs = As + RBM * BK;
     uint16_t* An = smem + ((ks + 1) & 1) * STAGE;
     uint16_t* Bn = An + RBM * BK;
-    const uint16_t* ab2 = has_next2 ? a_ptr(kofs(ks + 2)) : nullptr;
-    const uint16_t* bb2 = has_next2 ? b_ptr(kofs(ks + 2)) : nullptr;
 #pragma unroll
     for (int kk = 0; kk < BK / 16; ++kk) {
       bf16x8 af[2], bf[NJ];
@@ -330,12 +371,9 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
           *reinterpret_cast<u32x4*>(Bn + b_lds[i]) = rb[i];
       }
       if constexpr (has_next2) {
-        if (kk < 2) ra[kk] = *reinterpret_cast<const u32x4*>(ab2 + a_off[kk]);
+        if (kk < 2) ra[kk] = load_a(kofs(ks + 2), kk);
 #pragma unroll
-        for (int i = (kk * NB) / 4; i < ((kk + 1) * NB) / 4; ++i) {
-          const int64_t x = (MODE == RM_GATEUP && i >= NB / 2) ? b1_off : 0;
-          rb[i] = *reinterpret_cast<const u32x4*>(bb2 + x + b_off[i]);
-        }
+        for (int i = (kk * NB) / 4; i < ((kk + 1) * NB) / 4; ++i) rb[i] = load_b(kofs(ks + 2), i);
       }
 #pragma unroll
       for (int mi = 0; mi < 2; ++mi)
@@ -351,6 +389,13 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
   for (; ks + 2 < ksteps; ++ks) kstep(ks, T_{}, T_{});
   if (ks + 1 < ksteps) { kstep(ks, T_{}, F_{}); ++ks; }
   if (ks < ksteps) kstep(ks, F_{}, F_{});
+
+  // switch the fetch state to the next tile and request its first K step: the loads
+  // are in flight while the epilogue below runs
+  if (more) {
+    setup(nxt, nsrc);
+    issue(0);
+  }
 
   // ---- epilogue: through the wave's private LDS region, 16-byte coalesced rows ---------
   // acc[mi][nj][i]: output row = wm + mi*32 + (lane&31); output column within the nj-th
@@ -451,7 +496,13 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
       }
     }
   }
-  __syncthreads();  // every wave is done with its staging region before the next tile's operands land
+  // every wave is done with its staging region before the next tile's operands are parked;
+  // only LDS traffic is waited for, the tile's stores keep draining
+  phase_barrier();
+  if (!more) break;
+  within += stride;
+  cur = nxt;
+  nxt = nxt2;
   }
 }
 
@@ -645,8 +696,9 @@ int set_lds(K kernel, int bytes) {
 
 }  // namespace
 
-// The MFMA path needs whole 64-wide K steps and 16-byte aligned rows.
-bool bf16_fast_path_ok(int64_t D, int64_t F) { return D % 64 == 0 && F % 64 == 0 && D >= 64 && F >= 64; }
+// The MFMA path needs whole 64-wide K steps, 16-byte aligned rows, and outputs at least
+// one tile wide (a last tile that would overhang is shifted back, never clamped).
+bool bf16_fast_path_ok(int64_t D, int64_t F) { return D % 64 == 0 && F % 64 == 0 && D >= 384 && F >= 384; }
 
 enum { STAGE_GATEUP = 1, STAGE_DOWN = 2, STAGE_DH = 4, STAGE_DX = 8, STAGE_DW2 = 16, STAGE_DW1 = 32, STAGE_DW3 = 64 };
 
@@ -668,20 +720,21 @@ static unsigned resident_blocks() {
 constexpr int R_LDS_BYTES = 2 * R_STAGE * 2;  // 163840
 constexpr int W_LDS_BYTES = 8 * 64 * 136 * 2;  // 139264: the 8 epilogue regions (> 2 stages = 131072)
 
-template <int MODE, int NJ>
+template <int MODE, int NJ, bool GATHER = false>
 static int launch_row(RowArgs& a, int64_t tile_capacity, hipStream_t s, const char* what) {
   static bool configured = false;  // per process; the attribute is per function
   if (!configured) {
-    if (int rc = set_lds(row_tiled_kernel<MODE, NJ>, R_LDS_BYTES)) return rc;
+    if (int rc = set_lds(row_tiled_kernel<MODE, NJ, GATHER>, R_LDS_BYTES)) return rc;
     configured = true;
   }
   const unsigned blocks = std::min(round8(tile_capacity * a.n_tiles), resident_blocks());
-  hipLaunchKernelGGL((row_tiled_kernel<MODE, NJ>), dim3(blocks), dim3(NT), R_LDS_BYTES, s, a);
+  hipLaunchKernelGGL((row_tiled_kernel<MODE, NJ, GATHER>), dim3(blocks), dim3(NT), R_LDS_BYTES, s, a);
   return check_launch(what);
 }
 
-// 384-column tiles when they divide the width and 512-column tiles do not (F = 768).
-static bool narrow_tiles(int64_t width) { return width % 512 != 0 && width % 384 == 0; }
+// 384-column tiles when they divide the width and 512-column tiles do not (F = 768), or
+// when the output is narrower than 512 columns.
+static bool narrow_tiles(int64_t width) { return width < 512 || (width % 512 != 0 && width % 384 == 0); }
 
 int bf16_grouped_fwd(const void* rows, const int32_t* token_of_row, const void* w1, const void* w3,
                        const void* w2, const int32_t* seg_offsets, const int32_t* seg_counts,
@@ -695,13 +748,17 @@ int bf16_grouped_fwd(const void* rows, const int32_t* token_of_row, const void* 
     a.a0 = (const uint16_t*)rows; a.a_src = token_of_row; a.b0 = (const uint16_t*)w1; a.b1 = (const uint16_t*)w3;
     a.o0 = (uint16_t*)gate; a.o1 = (uint16_t*)up; a.o2 = (uint16_t*)h;
     a.n_tiles = (int)((F + RBN / 2 - 1) / (RBN / 2));
-    if (int rc = launch_row<RM_GATEUP, 4>(a, tile_capacity, s, "grouped gate/up")) return rc;
+    if (token_of_row) {
+      if (int rc = launch_row<RM_GATEUP, 4, true>(a, tile_capacity, s, "grouped gate/up")) return rc;
+    } else {
+      if (int rc = launch_row<RM_GATEUP, 4>(a, tile_capacity, s, "grouped gate/up")) return rc;
+    }
   }
   if (stages & STAGE_DOWN) {
     RowArgs b = a;
     b.a0 = (const uint16_t*)h; b.b0 = (const uint16_t*)w2; b.o0 = (uint16_t*)y;
     if (narrow_tiles(D)) {
-      b.n_tiles = (int)(D / 384);
+      b.n_tiles = (int)((D + 383) / 384);
       if (int rc = launch_row<RM_DOWN, 3>(b, tile_capacity, s, "grouped down")) return rc;
     } else {
       b.n_tiles = (int)((D + RBN - 1) / RBN);
@@ -726,7 +783,7 @@ int bf16_grouped_bwd(const void* dy, const void* rows, const int32_t* token_of_r
     a.gate = (const uint16_t*)gate; a.up = (const uint16_t*)up;
     a.o0 = (uint16_t*)dgate; a.o1 = (uint16_t*)dup;
     if (narrow_tiles(F)) {
-      a.n_tiles = (int)(F / 384);
+      a.n_tiles = (int)((F + 383) / 384);
       if (int rc = launch_row<RM_DH, 3>(a, tile_capacity, s, "grouped dh")) return rc;
     } else {
       a.n_tiles = (int)((F + RBN - 1) / RBN);
@@ -738,7 +795,7 @@ int bf16_grouped_bwd(const void* dy, const void* rows, const int32_t* token_of_r
     b.a0 = (const uint16_t*)dgate; b.a1 = (const uint16_t*)dup;
     b.b0 = (const uint16_t*)w1; b.b1 = (const uint16_t*)w3; b.o0 = (uint16_t*)drows;
     if (narrow_tiles(D)) {
-      b.n_tiles = (int)(D / 384);
+      b.n_tiles = (int)((D + 383) / 384);
       if (int rc = launch_row<RM_DX, 3>(b, tile_capacity, s, "grouped drows")) return rc;
     } else {
       b.n_tiles = (int)((D + RBN - 1) / RBN);
