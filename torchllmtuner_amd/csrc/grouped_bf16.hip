@@ -168,6 +168,7 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = (wave >> 2) * 64, wn = wave & 3;
+  const int wave_m = __builtin_amdgcn_readfirstlane(wm);  // the same value, known to be wave-uniform
   const int D = p.D, F = p.F;
   const int Kdim = (MODE == RM_GATEUP || MODE == RM_DH) ? D : (MODE == RM_DOWN ? F : 2 * F);
   const int lda = (MODE == RM_GATEUP || MODE == RM_DH) ? D : F;
@@ -342,6 +343,10 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
   // so that every load of the steady-state loop is unconditional: the compiler can then
   // count outstanding loads exactly and wait only for the three oldest before each park,
   // instead of draining the queue (vmcnt(0)) once per K step.
+  // The last tile of an expert is partly empty: a wave skips the MFMAs of its 32-row
+  // blocks that hold no real rows (a wave-uniform branch; operands are still staged and
+  // every barrier met).
+  const int act = min(max((valid - wave_m + 31) >> 5, 0), 2);
   auto kstep = [&](int ks, auto has_next_t, auto has_next2_t) {
     constexpr bool has_next = decltype(has_next_t)::value;
     constexpr bool has_next2 = decltype(has_next2_t)::value;
@@ -376,10 +381,13 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
         for (int i = (kk * NB) / 4; i < ((kk + 1) * NB) / 4; ++i) rb[i] = load_b(kofs(ks + 2), i);
       }
 #pragma unroll
-      for (int mi = 0; mi < 2; ++mi)
+      for (int mi = 0; mi < 2; ++mi) {
+        if (mi < act) {
 #pragma unroll
-        for (int nj = 0; nj < NJ; ++nj)
-          acc[mi][nj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[nj], af[mi], acc[mi][nj], 0, 0, 0);
+          for (int nj = 0; nj < NJ; ++nj)
+            acc[mi][nj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[nj], af[mi], acc[mi][nj], 0, 0, 0);
+        }
+      }
     }
     __syncthreads();
   };
@@ -409,6 +417,7 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
     const int f0 = n0 + wn * 64;
 #pragma unroll
     for (int mi = 0; mi < 2; ++mi) {
+      if (wave_m + mi * 32 >= valid) continue;  // no real rows in this half (uniform per wave)
 #pragma unroll
       for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -443,7 +452,7 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
       __builtin_amdgcn_s_waitcnt(0xc07f);
       __builtin_amdgcn_wave_barrier();
     }
-  } else {
+  } else if (wave_m < valid) {
     using S = WaveStage<32 * NJ>;
     constexpr int CH = 4 * NJ;  // 16-byte chunks per row of the wave's sub-tile
 #pragma unroll
