@@ -71,6 +71,38 @@ def time_events(fn, iters, warmup=2):
     return start.elapsed_time(stop) / iters
 
 
+def sustained_mfma(dev):
+    """What the matrix cores hold on v_mfma_f32_32x32x16_bf16 with register-resident
+    operands of random bits (libmi355probe.so): rate and core clock, both under the
+    card's own power management.  Returns None when the probe library is not built."""
+    import ctypes
+
+    import torch
+
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "torchllmtuner_amd", "libmi355probe.so")
+    if not os.path.exists(path):
+        return None
+    lib = ctypes.CDLL(path)
+    lib.mi355_probe_mfma.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                     ctypes.c_void_p]
+    lib.mi355_probe_mfma.restype = ctypes.c_int
+    blocks, iters = 4 * torch.cuda.get_device_properties(dev).multi_processor_count, 100000
+    sink = torch.zeros(1, dtype=torch.float32, device=dev)
+    clocks = torch.zeros(2 * blocks, dtype=torch.int64, device=dev)
+    out = {}
+    for label, rnd in (("random_bits", 1), ("constant_bits", 0)):
+        def launch():
+            rc = lib.mi355_probe_mfma(sink.data_ptr(), clocks.data_ptr(), blocks, iters, rnd,
+                                      torch.cuda.current_stream().cuda_stream)
+            assert rc == 0
+        ms = time_events(launch, 3, warmup=1)
+        flops = blocks * 8.0 * iters * 8 * 32768
+        c = clocks.view(blocks, 2).double()
+        out[label] = {"TFLOP/s": round(flops / (ms * 1e-3) / 1e12, 1),
+                      "core_clock_mhz": round(float((c[:, 0] / c[:, 1]).mean()) * 100.0, 0)}
+    return out
+
+
 def cpu_baseline(cfg, sample_tokens):
     """The oracle's forward+backward on host cores over ``sample_tokens`` tokens."""
     import torch
@@ -212,6 +244,13 @@ def main():
         "all_grouped_gemms": {"TFLOP/s": round(gemm_flops / (gemm_ms * 1e-3) / 1e12, 1),
                               "frac": round(gemm_flops / (gemm_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4)},
     }
+
+    probe = sustained_mfma(dev)
+    if probe is not None:
+        # the same instruction with operands in registers: the rate the card holds under
+        # its own power management, next to the data-sheet peak above
+        roofline["sustained_mfma"] = probe
+        roofline["frac_of_sustained"] = round(ach / probe["random_bits"]["TFLOP/s"], 4)
 
     result = {
         "metric": "MoE layer fwd+bwd tokens/s (Qwen3-30B-A3B shape, 1 GPU)",

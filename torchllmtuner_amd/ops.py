@@ -300,10 +300,11 @@ def combine_bwd(dout_TD, y_RD, weights_TK, plan: PermutePlan, zero_padding=True)
 
 # ------------------------------------------------------------------ experts
 def gather_supported(x_TD, hidden_dim: int) -> bool:
-    """The fused token gather exists for the bf16 MFMA kernels (D, F multiples of 64)."""
+    """The fused token gather exists for the bf16 MFMA kernels (D, F multiples of 64, at
+    least 384: the library's own condition for that path)."""
     D = x_TD.shape[-1]
     return (x_TD.dtype == torch.bfloat16 and D % 64 == 0 and hidden_dim % 64 == 0
-            and x_TD.shape[0] * D < 2**31)
+            and D >= 384 and hidden_dim >= 384 and x_TD.shape[0] * D < 2**31)
 
 
 def grouped_swiglu_fwd(rows_RD, w1_EFD, w3_EFD, w2_EDF, plan: PermutePlan, gather=False):
