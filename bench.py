@@ -188,14 +188,14 @@ def main():
         w1, w3, w2 = ie.w1_EFD.detach(), ie.w3_EFD.detach(), ie.w2_EDF.detach()
         y, gate, up, h = ops.grouped_swiglu_fwd(rows, w1, w3, w2, plan)
         dy, _ = ops.combine_bwd(gout, y, scores, plan)
-        fwd_buf = dict(rows=x, token_of_row=plan.token_of_row, w1=w1, w3=w3, w2=w2, gate=gate, up=up, h=h, y=y)
-        buf = dict(rows=rows, w1=w1, w3=w3, w2=w2, gate=gate, up=up, h=h, y=y, dy=dy,
+        # as in the training step: the token matrix is read through the gather index
+        # (gate/up A operand, dW1/dW3 B operand); no expert-major copy of the tokens
+        buf = dict(rows=x, token_of_row=plan.token_of_row, w1=w1, w3=w3, w2=w2, gate=gate, up=up, h=h, y=y, dy=dy,
                    dgate=torch.empty_like(gate), dup=torch.empty_like(up), drows=torch.empty_like(rows),
                    dw1=torch.empty_like(w1), dw3=torch.empty_like(w3), dw2=torch.empty_like(w2))
         R_rows = int(plan.total_rows.item())
         it = args.stage_iters
-        stage_ms = {s: time_events(lambda s=s: ops.grouped_swiglu_stage(s, fwd_buf if s == 'gate_up' else buf, plan), it)
-                    for s in ops.STAGES}
+        stage_ms = {s: time_events(lambda s=s: ops.grouped_swiglu_stage(s, buf, plan), it) for s in ops.STAGES}
         logits = ops.router_gate_fwd(x, block.router.gate.weight)
         other_ms = {
             "router_gate_fwd": time_events(lambda: ops.router_gate_fwd(x, block.router.gate.weight), it),
@@ -224,6 +224,8 @@ def main():
         kernels[f"grouped_{s}"] = {"ms": round(ms, 4), "TFLOP/s": round(tf, 1), "frac_mfma": round(tf / PEAK_BF16_TFLOPS, 4)}
     for s, ms in other_ms.items():
         ent = {"ms": round(ms, 4)}
+        if s == "permute_rows_fwd":
+            ent["in_step"] = False  # public dispatcher API only: the fused step gathers inside the GEMMs
         if s in other_bytes:
             gbs = other_bytes[s] / (ms * 1e-3) / 1e9
             ent.update({"GB/s": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4)})

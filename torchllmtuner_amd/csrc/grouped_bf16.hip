@@ -532,6 +532,7 @@ struct WgradArgs {
   int total;  // El * m_tiles * n_tiles
 };
 
+template <bool GATHER>
 __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -553,53 +554,73 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
   // Persistent workgroups, same walk as the row-tiled kernels.  The K extent is one
   // expert's rows (a handful of 64-row steps), so what surrounds the K loop matters: the
   // first operands of the next tile are requested before the epilogue of the current one
-  // and land while it runs.
+  // and land while it runs, segment bounds are looked up two tiles ahead, and with a
+  // gathered B operand the row indices of a K step are fetched one step before its data.
   const int chunk = (p.total + 7) >> 3;
   const int stride = gridDim.x >> 3;
+  const int pid_base = (blockIdx.x & 7) * chunk;
   int within = blockIdx.x >> 3;
-  int pid = (blockIdx.x & 7) * chunk + within;
-  if (within >= chunk || pid >= p.total) return;
+  if (within >= chunk || pid_base + within >= p.total) return;
+  auto exists = [&](int w) { return w < chunk && pid_base + w < p.total; };
 
   // state of the tile whose operands are being fetched
+  int pid = pid_base + within;
   int e = pid / per_e;
   int m0 = ((pid % per_e) / p.n_tiles) * WBM, n0 = ((pid % per_e) % p.n_tiles) * WBN;
-  int cnt = p.seg_counts[e];
+  int seg0 = p.seg_offsets[e], cnt = p.seg_counts[e];
   const uint16_t* a_base;
   const uint16_t* b_base;
-  const int32_t* b_src;
-  auto set_bases = [&](int seg0) {
+  auto set_bases = [&]() {
     a_base = p.a + static_cast<int64_t>(seg0) * M + min(m0 + ks_chunk * 8, M - 8);
-    b_base = p.b + (p.b_src ? 0 : static_cast<int64_t>(seg0) * N) + min(n0 + ks_chunk * 8, N - 8);
-    b_src = p.b_src ? p.b_src + seg0 : nullptr;
+    b_base = p.b + (GATHER ? 0 : static_cast<int64_t>(seg0) * N) + min(n0 + ks_chunk * 8, N - 8);
+  };
+  // B row of this thread's chunk i in K step `step` of segment (s0, c): its own row, or
+  // (gather) the source row from the index array.  Needs c > 0.
+  auto row_index = [&](int s0, int c, int step, int i) -> int {
+    const int k = min(step * BK + ks_k + 16 * i, c - 1);
+    return GATHER ? max(p.b_src[s0 + k], 0) : k;
   };
   // Loads of one K step, unconditional: rows past the segment re-read its last row and
   // the A side is zeroed when it is parked, so the products vanish.  Needs cnt > 0.
-  auto issue = [&](int step) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int k = min(step * BK + ks_k + 16 * i, cnt - 1);
-      ra[i] = *reinterpret_cast<const u32x4*>(a_base + static_cast<int64_t>(k) * M);
-      const int kb = b_src ? max(b_src[k], 0) : k;
-      rb[i] = *reinterpret_cast<const u32x4*>(b_base + static_cast<int64_t>(kb) * N);
-    }
+  auto load_ab = [&](int step, int i, int brow) {
+    const int k = min(step * BK + ks_k + 16 * i, cnt - 1);
+    ra[i] = *reinterpret_cast<const u32x4*>(a_base + static_cast<int64_t>(k) * M);
+    rb[i] = *reinterpret_cast<const u32x4*>(b_base + static_cast<int64_t>(brow) * N);
   };
   auto park = [&](int step, int i, uint16_t* An, uint16_t* Bn, int count) {
     const bool live = step * BK + ks_k + 16 * i < count;
     *reinterpret_cast<u32x4*>(An + lds_off[i]) = live ? ra[i] : zero;
     *reinterpret_cast<u32x4*>(Bn + lds_off[i]) = rb[i];
   };
-  set_bases(p.seg_offsets[e]);
-  if (cnt > 0) issue(0);
+  int bidx[4];  // B rows of the K step that is requested next
+  set_bases();
+  if (cnt > 0) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) load_ab(0, i, row_index(seg0, cnt, 0, i));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) bidx[i] = row_index(seg0, cnt, 1, i);
+  }
+  // segment of the next tile (the one after it is looked up inside the loop)
+  int nseg0, ncnt;
+  {
+    const int ne = (pid_base + (exists(within + stride) ? within + stride : within)) / per_e;
+    nseg0 = p.seg_offsets[ne];
+    ncnt = p.seg_counts[ne];
+  }
 
   for (;;) {
-    // the tile after this one: its segment is looked up now and used after the K loop
-    const int nwithin = within + stride;
-    const int npid = (blockIdx.x & 7) * chunk + nwithin;
-    const bool more = nwithin < chunk && npid < p.total;
-    const int fpid = more ? npid : pid;
-    const int ne = fpid / per_e;
-    const int nseg0 = p.seg_offsets[ne], ncnt = p.seg_counts[ne];
-    const int c_e = e, c_m0 = m0, c_n0 = n0, c_cnt = cnt;
+    const bool more = exists(within + stride);
+    const int npid = pid_base + within + stride;
+    // two tiles ahead: segment bounds, used one tile later
+    const int e2 = (pid_base + (exists(within + 2 * stride) ? within + 2 * stride : within)) / per_e;
+    const int n2seg0 = p.seg_offsets[e2], n2cnt = p.seg_counts[e2];
+    // next tile: B rows of its first K step (its bounds were looked up a tile ago)
+    int nidx[4];
+    if (ncnt > 0) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) nidx[i] = row_index(nseg0, ncnt, 0, i);
+    }
+    const int c_e = e, c_m0 = m0, c_n0 = n0, c_cnt = cnt, c_seg0 = seg0;
     const int ksteps = (cnt + BK - 1) / BK;
 
     f32x16 acc[2][4];
@@ -613,7 +634,12 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
     if (ksteps > 0) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) park(0, i, smem, smem + WBM * BK, c_cnt);
-      if (ksteps > 1) issue(1);
+      if (ksteps > 1) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) load_ab(1, i, bidx[i]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) bidx[i] = row_index(c_seg0, c_cnt, 2, i);
+      }
     }
     __syncthreads();
 
@@ -636,10 +662,8 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
         for (int nj = 0; nj < 4; ++nj) bf[nj] = frag_ks<256>(Bs, wn + nj * 32, kk, lane);
         if constexpr (has_next) park(ks + 1, kk, An, Bn, c_cnt);
         if constexpr (has_next2) {
-          const int k = min((ks + 2) * BK + ks_k + 16 * kk, c_cnt - 1);
-          ra[kk] = *reinterpret_cast<const u32x4*>(a_base + static_cast<int64_t>(k) * M);
-          const int kb = b_src ? max(b_src[k], 0) : k;
-          rb[kk] = *reinterpret_cast<const u32x4*>(b_base + static_cast<int64_t>(kb) * N);
+          load_ab(ks + 2, kk, bidx[kk]);
+          bidx[kk] = row_index(c_seg0, c_cnt, ks + 3, kk);
         }
 #pragma unroll
         for (int mi = 0; mi < 2; ++mi)
@@ -658,12 +682,18 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
 
     // switch the fetch state to the next tile and request its first K step
     if (more) {
-      e = ne;
+      e = npid / per_e;
       m0 = ((npid % per_e) / p.n_tiles) * WBM;
       n0 = ((npid % per_e) % p.n_tiles) * WBN;
+      seg0 = nseg0;
       cnt = ncnt;
-      set_bases(nseg0);
-      if (cnt > 0) issue(0);
+      set_bases();
+      if (cnt > 0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) load_ab(0, i, nidx[i]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) bidx[i] = row_index(seg0, cnt, 1, i);
+      }
     }
 
     using S = WaveStage<128>;
@@ -691,8 +721,9 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
     // the LDS traffic is waited for, the tile's stores keep draining
     phase_barrier();
     if (!more) break;
-    within = nwithin;
-    pid = npid;
+    within += stride;
+    nseg0 = n2seg0;
+    ncnt = n2cnt;
   }
 }
 
@@ -813,7 +844,8 @@ int bf16_grouped_bwd(const void* dy, const void* rows, const int32_t* token_of_r
   }
   static bool wconfigured = false;
   if (!wconfigured) {
-    if (int rc = set_lds(wgrad_kernel, W_LDS_BYTES)) return rc;
+    if (int rc = set_lds(wgrad_kernel<false>, W_LDS_BYTES)) return rc;
+    if (int rc = set_lds(wgrad_kernel<true>, W_LDS_BYTES)) return rc;
     wconfigured = true;
   }
   auto wgrad = [&](const void* A, const void* B, const int32_t* b_src, void* C, int64_t M, int64_t N, const char* what) {
@@ -822,7 +854,11 @@ int bf16_grouped_bwd(const void* dy, const void* rows, const int32_t* token_of_r
     w.seg_offsets = seg_offsets; w.seg_counts = seg_counts; w.M = (int)M; w.N = (int)N;
     w.m_tiles = (int)((M + WBM - 1) / WBM); w.n_tiles = (int)((N + WBN - 1) / WBN);
     w.total = (int)(El * w.m_tiles * w.n_tiles);
-    hipLaunchKernelGGL(wgrad_kernel, dim3(std::min(round8(w.total), resident_blocks())), dim3(NT), W_LDS_BYTES, s, w);
+    const dim3 grid(std::min(round8(w.total), resident_blocks()));
+    if (b_src)
+      hipLaunchKernelGGL(wgrad_kernel<true>, grid, dim3(NT), W_LDS_BYTES, s, w);
+    else
+      hipLaunchKernelGGL(wgrad_kernel<false>, grid, dim3(NT), W_LDS_BYTES, s, w);
     return check_launch(what);
   };
   if (dw2 && (stages & STAGE_DW2)) if (int rc = wgrad(dy, h, nullptr, dw2, D, F, "grouped dw2")) return rc;

@@ -123,9 +123,9 @@ class GatherGroupedSwiGLUFunction(torch.autograd.Function):
 
     Forward never materialises the expert-major copy of the tokens: the gate/up kernel
     reads ``x[token_of_row[r]]`` directly, and nothing of size (R, D) is kept for the
-    backward.  Backward rebuilds the rows once (the weight-gradient kernels measured
-    30 % slower reading their K rows through the index) and returns ``dx``, the K-way
-    row sum of the expert-major input gradient.
+    backward.  The weight-gradient kernels read their K rows through the same index (the
+    row numbers of a K step are fetched one step ahead of its data), and ``dx`` is the
+    K-way row sum of the expert-major input gradient.
     """
 
     @staticmethod
@@ -139,11 +139,9 @@ class GatherGroupedSwiGLUFunction(torch.autograd.Function):
     @once_differentiable
     def backward(ctx, dy):
         x, w1, w3, w2, gate, up, h = ctx.saved_tensors
-        need_dw = any(ctx.needs_input_grad[1:4])
-        rows = ops.permute_rows_fwd(x, ctx.plan) if need_dw else x
         drows, dw1, dw3, dw2 = ops.grouped_swiglu_bwd(
-            dy, rows, w1, w3, w2, gate, up, h, ctx.plan,
-            need_drows=ctx.needs_input_grad[0], need_dw=need_dw, gather=not need_dw,
+            dy, x, w1, w3, w2, gate, up, h, ctx.plan,
+            need_drows=ctx.needs_input_grad[0], need_dw=any(ctx.needs_input_grad[1:4]), gather=True,
         )
         dx = ops.permute_rows_bwd(drows, ctx.plan) if drows is not None else None
         return dx, dw1, dw3, dw2, None
