@@ -58,9 +58,14 @@ const char* mi355_moe_last_error(void);
  * Replaces RouterGateLinearFunction.forward and RouterGateLinear.forward,
  * llmtuner/models/common/linear.py:107-131,179-183.
  * x: (T,D) x_dtype row-major; w: (E,D) w_dtype; logit_bias: (E) fp32 or NULL.
+ * workspace: mi355_router_gate_fwd_workspace_bytes() bytes or NULL.  With a workspace,
+ * bf16 x, fp32 w and D, E multiples of 64, each fp32 weight is written as three bf16
+ * pieces (24 mantissa bits) and the product runs as three bf16 MFMAs with fp32
+ * accumulation; otherwise the strided fp32-MFMA kernel is used.
  */
+int64_t mi355_router_gate_fwd_workspace_bytes(int64_t T, int64_t D, int64_t E);
 int mi355_router_gate_fwd(const void* x, int x_dtype, const void* w, int w_dtype,
-                          const float* logit_bias, float* logits_TE,
+                          const float* logit_bias, float* logits_TE, void* workspace,
                           int64_t T, int64_t D, int64_t E, void* stream);
 
 /*
@@ -68,7 +73,8 @@ int mi355_router_gate_fwd(const void* x, int x_dtype, const void* w, int w_dtype
  * dw[e][d] = sum_t dlogits[t][e] * x[t][d]   (written in w_dtype; NULL = skip)
  * both accumulated in fp32.  Replaces RouterGateLinearFunction.backward,
  * linear.py:133-151.  workspace: mi355_router_gate_bwd_workspace_bytes() bytes
- * (split-K partial sums for dw), may be NULL when dw is NULL.
+ * (bf16 weight pieces, split-K partial sums for dw); NULL selects the strided
+ * fp32-MFMA kernels and is only valid when dw is NULL or T is small.
  */
 int64_t mi355_router_gate_bwd_workspace_bytes(int64_t T, int64_t D, int64_t E);
 int mi355_router_gate_bwd(const float* dlogits_TE, const void* x, int x_dtype,

@@ -28,7 +28,10 @@ def ops():
 
 # ---------------------------------------------------------------- router gate
 @pytest.mark.parametrize("T,D,E,xdt", [(3, 8, 4, torch.float32), (512, 256, 8, torch.float32),
-                                       (1000, 320, 72, torch.bfloat16), (0, 16, 4, torch.float32)])
+                                       (1000, 320, 72, torch.bfloat16), (0, 16, 4, torch.float32),
+                                       # bf16 tokens, D and E multiples of 64: the three-piece bf16 MFMA path
+                                       (1000, 320, 64, torch.bfloat16), (2048, 2048, 128, torch.bfloat16),
+                                       (77, 192, 192, torch.bfloat16), (8192, 128, 256, torch.bfloat16)])
 def test_router_gate_fwd_bwd(ops, T, D, E, xdt):
     print(f"router_gate T={T} D={D} E={E} {xdt}", flush=True)
     g = torch.Generator().manual_seed(0)

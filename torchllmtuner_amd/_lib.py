@@ -24,7 +24,8 @@ F = c_float
 SIGNATURES = {
     "mi355_moe_abi_version": (I, []),
     "mi355_moe_last_error": (c_char_p, []),
-    "mi355_router_gate_fwd": (I, [P, I, P, I, P, P, L, L, L, P]),
+    "mi355_router_gate_fwd_workspace_bytes": (L, [L, L, L]),
+    "mi355_router_gate_fwd": (I, [P, I, P, I, P, P, P, L, L, L, P]),
     "mi355_router_gate_bwd_workspace_bytes": (L, [L, L, L]),
     "mi355_router_gate_bwd": (I, [P, P, I, P, I, P, P, P, L, L, L, P]),
     "mi355_router_select_fwd": (I, [P, P, P, P, P, L, L, L, I, I, F, I, I, I, P]),

@@ -45,85 +45,19 @@
 #include <cstdlib>
 #include <type_traits>
 
+#include "bf16_tiles.h"
 #include "common.h"
 
 namespace mi355 {
 namespace {
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef short s16x4 __attribute__((ext_vector_type(4)));
-typedef short s16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
-
-constexpr int BK = 64;
 constexpr int NT = 512;  // threads per workgroup
-
-#define LDS_PTR(p) ((__attribute__((address_space(3))) s16x4*)(p))
-
-// ---- fragment reads -----------------------------------------------------------------
-__device__ __forceinline__ bf16x8 frag_kc(const uint16_t* tile, int row, int kk, int lane) {
-  const int r = row + (lane & 31);
-  const int c = kk * 2 + (lane >> 5);
-  return *reinterpret_cast<const bf16x8*>(tile + r * BK + ((c ^ ((r >> 1) & 7)) << 3));
-}
-
-template <int COLS>
-__device__ __forceinline__ bf16x8 frag_ks(const uint16_t* tile, int col, int kk, int lane) {
-  const int g = lane >> 4, i = lane & 15;
-  const int k = kk * 16 + 8 * (g >> 1) + (i >> 2);  // k & 3 == i >> 2 for both reads
-  const int c = col + 16 * (g & 1) + 4 * (i & 3);
-  const int off = (((c >> 3) ^ ((k & 3) << 1)) << 3) + (c & 7);
-  const uint16_t* p = tile + k * COLS + off;
-  const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(p));
-  const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(p + 4 * COLS));
-  const s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-  return __builtin_bit_cast(bf16x8, v);
-}
-
-__device__ __forceinline__ int xcd_remap(int bid, int total) {
-  const int chunk = (total + 7) >> 3;
-  const int within = bid >> 3;
-  const int pid = (bid & 7) * chunk + within;
-  return (within < chunk && pid < total) ? pid : -1;
-}
-
-// Workgroup barrier that waits for this wave's own LDS operations only: global loads and
-// stores stay in flight across it.
-__device__ __forceinline__ void phase_barrier() {
-  __builtin_amdgcn_sched_barrier(0);
-  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
-  __builtin_amdgcn_s_barrier();
-  __builtin_amdgcn_sched_barrier(0);
-}
-
-__device__ __forceinline__ uint32_t pack2(float a, float b) { return pack_bf16x2(a, b); }
 
 // 1 / (1 + e^-x) on the transcendental unit (v_exp_f32, v_rcp_f32: about 1 ulp each; every
 // use is rounded to bf16 right after)
 __device__ __forceinline__ float fast_sigmoid(float x) {
   return __builtin_amdgcn_rcpf(1.0f + __expf(-x));
 }
-
-// ---- epilogue staging -----------------------------------------------------------------
-// A wave parks its 64 x W sub-tile (bf16) in its private LDS region, [64][W + 8], then
-// streams it out as 16-byte row pieces.  acc was produced with the weight fragment as
-// the first MFMA operand: lane = output row (lane & 31), registers = output columns.
-template <int W>
-struct WaveStage {
-  static constexpr int PITCH = W + 8;
-  static constexpr int ELEMS = 64 * PITCH;
-  // element (row m of 64, col n of W) for register i of the accumulator tile (mi, nj-th 32 columns)
-  __device__ static __forceinline__ void put4(uint16_t* st, int mi, int col0, int lane, int q,
-                                              float v0, float v1, float v2, float v3) {
-    const int m = mi * 32 + (lane & 31);
-    const int n = col0 + q * 8 + (lane >> 5) * 4;
-    u32x2 pk = {pack2(v0, v1), pack2(v2, v3)};
-    *reinterpret_cast<u32x2*>(st + m * PITCH + n) = pk;
-  }
-};
-
 
 enum RowMode { RM_GATEUP = 0, RM_DOWN = 1, RM_DH = 2, RM_DX = 3 };
 

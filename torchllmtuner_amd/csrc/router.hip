@@ -283,14 +283,23 @@ int check_router_args(int64_t T, int64_t E, int64_t K) {
 
 using namespace mi355;
 
+extern "C" int64_t mi355_router_gate_fwd_workspace_bytes(int64_t T, int64_t D, int64_t E) {
+  (void)T;
+  return (D >= 1 && E >= 1 && router_x3_ok(MI355_BF16, MI355_F32, D, E)) ? router_x3_fwd_workspace(D, E) : 0;
+}
+
 extern "C" int mi355_router_gate_fwd(const void* x, int x_dtype, const void* w, int w_dtype,
-                                     const float* logit_bias, float* logits, int64_t T, int64_t D,
-                                     int64_t E, void* stream) {
+                                     const float* logit_bias, float* logits, void* workspace,
+                                     int64_t T, int64_t D, int64_t E, void* stream) {
   MI355_REQUIRE(T >= 0 && D >= 1 && E >= 1, "router_gate_fwd: bad shape T=%lld D=%lld E=%lld",
                 (long long)T, (long long)D, (long long)E);
   MI355_REQUIRE(T < (1ll << 31) && D < (1ll << 31), "router_gate_fwd: shape exceeds int32");
   if (T == 0) return MI355_OK;
   MI355_REQUIRE(x && w && logits, "router_gate_fwd: null pointer");
+  // bf16 tokens against fp32 weights: three bf16 MFMAs per product, fp32-exact operands
+  if (workspace && router_x3_ok(x_dtype, w_dtype, D, E))
+    return router_x3_fwd(x, static_cast<const float*>(w), logit_bias, logits, workspace, T, D, E,
+                         as_stream(stream));
   GemmArgs g{};
   g.A = x; g.B = w; g.C = logits; g.bias = logit_bias;
   g.a_rs = D; g.a_cs = 1;
@@ -311,8 +320,11 @@ static int gate_bwd_ksplit(int64_t T, int64_t D, int64_t E) {
 }
 
 extern "C" int64_t mi355_router_gate_bwd_workspace_bytes(int64_t T, int64_t D, int64_t E) {
+  if (T < 0 || D < 1 || E < 1) return 0;
   const int s = gate_bwd_ksplit(T, D, E);
-  return s > 1 ? (int64_t)s * E * D * 4 : 0;
+  const int64_t strided = s > 1 ? (int64_t)s * E * D * 4 : 0;
+  const int64_t x3 = router_x3_ok(MI355_BF16, MI355_F32, D, E) ? router_x3_bwd_workspace(T, D, E) : 0;
+  return strided > x3 ? strided : x3;
 }
 
 extern "C" int mi355_router_gate_bwd(const float* dlogits, const void* x, int x_dtype,
@@ -322,6 +334,10 @@ extern "C" int mi355_router_gate_bwd(const float* dlogits, const void* x, int x_
   MI355_REQUIRE(T >= 0 && D >= 1 && E >= 1 && T < (1ll << 31) && D < (1ll << 31),
                 "router_gate_bwd: bad shape");
   hipStream_t s = as_stream(stream);
+  if (workspace && router_x3_ok(x_dtype, w_dtype, D, E)) {
+    MI355_REQUIRE(dlogits && w && (x || !dw), "router_gate_bwd: null pointer");
+    return router_x3_bwd(dlogits, x, static_cast<const float*>(w), dx, static_cast<float*>(dw), workspace, T, D, E, s);
+  }
   if (dx && T > 0) {
     GemmArgs g{};
     g.A = dlogits; g.B = w; g.C = dx;

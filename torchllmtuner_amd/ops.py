@@ -68,9 +68,12 @@ def router_gate_fwd(x_TD, w_ED, logit_bias_E=None):
         raise ValueError(f"gate weight {tuple(w_ED.shape)} does not match input dim {D}")
     bias = None if logit_bias_E is None else _c(logit_bias_E.float())
     out = torch.empty(T, E, dtype=torch.float32, device=dev)
+    lib = _lib.load()
+    nbytes = lib.mi355_router_gate_fwd_workspace_bytes(T, D, E)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev) if nbytes else None
     with torch.cuda.device(dev):
-        rc = _lib.load().mi355_router_gate_fwd(
-            _p(x_TD), _dt(x_TD), _p(w_ED), _dt(w_ED), _p(bias), _p(out), T, D, E, _stream(dev)
+        rc = lib.mi355_router_gate_fwd(
+            _p(x_TD), _dt(x_TD), _p(w_ED), _dt(w_ED), _p(bias), _p(out), _p(ws), T, D, E, _stream(dev)
         )
     _lib.check(rc, "router_gate_fwd")
     return out
@@ -84,11 +87,8 @@ def router_gate_bwd(dlogits_TE, x_TD, w_ED, need_dx=True, need_dw=True):
     lib = _lib.load()
     dx = torch.empty_like(x_TD) if need_dx else None
     dw = torch.empty_like(w_ED) if need_dw else None
-    ws = None
-    if need_dw:
-        nbytes = lib.mi355_router_gate_bwd_workspace_bytes(T, D, E)
-        if nbytes:
-            ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    nbytes = lib.mi355_router_gate_bwd_workspace_bytes(T, D, E)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev) if nbytes else None
     with torch.cuda.device(dev):
         rc = lib.mi355_router_gate_bwd(
             _p(dlogits_TE), _p(x_TD), _dt(x_TD), _p(w_ED), _dt(w_ED), _p(dx), _p(dw), _p(ws),
