@@ -30,8 +30,8 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # WRITE_SIZE (scaled by a 256 MiB copy: x2.0 and x1.0); the table these come from is
 # profiles/moe_layer_qwen3_t8192_hbm_traffic.txt.  Only reported for the default workload.
 MEASURED_HBM_BYTES = {
-    "gate_up": 1646.5e6, "down": 946.3e6, "dh": 1253.3e6, "drows": 1623.5e6,
-    "dw2": 886.7e6, "dw1": 886.7e6, "dw3": 886.7e6,
+    "gate_up": 2189.8e6, "down": 1015.6e6, "dh": 1383.4e6, "drows": 2100.3e6,
+    "dw2": 831.1e6, "dw1": 895.9e6, "dw3": 895.9e6,
 }
 
 WORKLOADS = {
@@ -49,6 +49,8 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-tokens", type=int, default=1024)
     ap.add_argument("--stage-iters", type=int, default=10)
+    ap.add_argument("--no-probe", action="store_true",
+                    help="skip the sustained-MFMA probe (about 0.8 s of matrix-core work)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (known traffic, for scaling rocprof FETCH_SIZE / WRITE_SIZE)")
     return ap.parse_args()
@@ -247,7 +249,7 @@ def main():
                               "frac": round(gemm_flops / (gemm_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4)},
     }
 
-    probe = sustained_mfma(dev)
+    probe = None if args.no_probe else sustained_mfma(dev)
     if probe is not None:
         # the same instruction with operands in registers: the rate the card holds under
         # its own power management, next to the data-sheet peak above

@@ -7,24 +7,38 @@
 //   drows    dgate . w1 + dup . w3      A KC, B KS   (one accumulator, K = 2F)
 //   dw*      a_e^T . b_e                A KS, B KS   K = the expert's rows
 //
-// Shape of the kernels.  Measured on MI355X these GEMMs are bound by the number of
-// cache-line requests a CU's vector L1 keeps in flight (about 50 x 128 B at ~600 clk
-// average L2 latency = 13 B/clk/CU), not by the matrix cores: what matters is bytes
-// requested per flop.  Hence 128x512 output tiles for the row-tiled products and
-// 256x256 for the weight gradients, eight waves per workgroup (two per SIMD), one
-// workgroup per CU with the 160 KiB of LDS holding two stages of the operand tiles.
-// Row tiles come from the permutation plan's tile list (128 rows of one expert each)
-// and block ids are remapped so that each XCD walks a contiguous run of tiles: the
-// blocks that share an expert's weights share an L2.
+// Shape of the kernels.  128x512 output tiles for the row-tiled products (384 wide when
+// that divides the width and 512 does not) and 256x256 for the weight gradients, eight
+// waves per workgroup (two per SIMD, each wave a 64x128 accumulator tile), one workgroup
+// per CU with the 160 KiB of LDS holding two stages of the operand tiles.  Row tiles come
+// from the permutation plan's tile list (128 rows of one expert each).
 //
-// Row-tiled main loop: a ping-pong schedule.  Waves 4..7 run one phase behind waves
-// 0..3 (wave w and w+4 share a SIMD); a phase is either "memory" (park 2-3 chunks of
-// the next tile in the other LDS stage, fetch the same chunks of the tile after it,
-// read this step's fragments) or "MFMA" (8 matrix instructions), separated by
-// s_barrier with only the wave's own LDS traffic waited for, so global loads stay in
-// flight across barriers.  The pipeline tail is peeled at compile time: every load
-// of the steady-state loop is unconditional, which lets the compiler count
-// outstanding loads exactly instead of draining the queue once per K step.
+// What bounds them, measured on MI355X.  With operands of random bits the card's power
+// management holds the core clock near 1.5-1.9 GHz (2.4 GHz with constant operands): a
+// register-resident MFMA loop sustains 1.45-1.95 PFLOP/s instead of the 2.5 PFLOP/s of the
+// data sheet, the same loop fed from LDS and staging its operands from L2 about 1.0-1.1.
+// The K loops here run at that rate; operand traffic is not the limit (L2 delivers
+// 50 B/clk/CU to a tile-shaped read pattern, HBM 10 B/clk/CU, and making every operand
+// cache-resident changes nothing).  What is left is everything around the K loop, hence:
+//   * persistent workgroups: block b serves XCD b % 8 and walks that XCD's contiguous
+//     run of tiles with stride gridDim/8, so the tiles in flight on an XCD are
+//     neighbours that share an expert's weights in its L2, and no workgroup launch sits
+//     between two tiles;
+//   * tile metadata looked up two tiles ahead, the first K step of the next tile
+//     requested before the epilogue of the current one; the barrier between tiles waits
+//     for LDS traffic only, so a tile's stores drain under the next tile's work;
+//   * hardware bf16 conversion and transcendental-unit sigmoid in the epilogues (they
+//     were VALU bound);
+//   * a wave skips the MFMAs of 32-row blocks that hold no real rows (last tile of an
+//     expert).
+//
+// K loop: one barrier per K step of 64.  Per quarter step a wave reads its fragments,
+// parks a quarter of the next step's operands (held in registers) in the other LDS
+// stage, refills those registers with the step after, and issues its MFMAs.  The
+// pipeline tail is peeled at compile time: every load of the steady state is
+// unconditional, so the compiler counts outstanding loads exactly instead of draining
+// the queue once per K step.  Operand addresses are a wave-uniform 64-bit base plus a
+// fixed 32-bit per-thread offset.
 //
 // MFMA: v_mfma_f32_32x32x16_bf16.  Per lane 8 bf16 of each operand (row lane%32,
 // k = 8*(lane/32)..+7), 16 fp32 of the result (column lane%32, rows
@@ -33,14 +47,7 @@
 // output columns of one output row: epilogues pack them and go through LDS to
 // write 16-byte, fully coalesced rows.
 //
-// LDS layouts (no padding, XOR swizzles; 16-byte chunks):
-//   KC  contraction axis contiguous in HBM: [row][64 k], chunk c of row r stored at
-//       c ^ ((r >> 1) & 7); a fragment is one ds_read_b128 (measured conflict-free;
-//       the key r & 7 costs a 2-way conflict).
-//   KS  contraction axis strided in HBM: [k][cols], chunk c of row k stored at
-//       c ^ ((k & 3) << 1); a fragment is two ds_read_b64_tr_b16 (LDS transpose
-//       reads: lane i of a 16-lane group supplies the address of row i/4, 8-byte
-//       piece i%4, and receives column i of the four rows).
+// The LDS layouts (KC / KS) and fragment reads are in bf16_tiles.h.
 #include <algorithm>
 #include <cstdlib>
 #include <type_traits>
