@@ -191,3 +191,105 @@ def test_dispatcher_api_matches_reference_contract():
                                                 torch.zeros(2, 2, dtype=torch.long, device=DEV), counts.to(DEV))
     with pytest.raises(RuntimeError, match="no CPU implementation"):
         moe.LocalTokenDispatcher(4, 2).dispatch(x, sc, ids, counts)
+
+
+def test_full_size_properties_qwen3_t8192():
+    """The benchmark's own size (T=8192, D=2048, E=128, K=8, F=768, bf16), too large for the
+    CPU oracle: size-independent properties instead.
+
+    * the plan is a permutation of the T*K slots, counts add up, every row maps back;
+    * scaling w2 by 2 (exact in bf16) scales the output by exactly 2, bit for bit;
+    * a sample of tokens recomputed token by token in fp32 on the device agrees within
+      the bf16 bar; a sample of experts' weight gradients recomputed from the same
+      intermediates with plain matmuls agrees within it too;
+    * two runs give bit-identical outputs and gradients (no atomics anywhere).
+    """
+    print("block full size T=8192", flush=True)
+    from torchllmtuner_amd import ops
+
+    T, D, E, K, F = 8192, 2048, 128, 8, 768
+    spec = R.RouterSpec(E, K, score_func="softmax", route_norm=True)
+    p = make_params(E, D, F, torch.bfloat16, seed=3)
+    block = build_block(p, spec, D, F, torch.bfloat16, DEV)
+    block.train()
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(T, D, generator=g).bfloat16().to(DEV)
+    gout = torch.randn(T, D, generator=g).bfloat16().to(DEV)
+
+    def run():
+        block.zero_grad(set_to_none=True)
+        xin = x.clone().requires_grad_()
+        out = block(xin)
+        out.backward(gout)
+        ie = block.routed_experts.inner_experts
+        return out.detach(), xin.grad, ie.w1_EFD.grad.clone(), ie.w3_EFD.grad.clone(), ie.w2_EDF.grad.clone(), \
+            block.router.gate.weight.grad.clone()
+
+    first = run()
+    second = run()
+    for a, b in zip(first, second):
+        assert torch.equal(a, b), "two runs on the same inputs differ"
+    out, dx, dw1, dw3, dw2, dwr = first
+    for t in first:
+        assert torch.isfinite(t.float()).all()
+
+    # --- plan: permutation, counts
+    with torch.no_grad():
+        scores, ids = block.router.route(x)
+        plan = block.routed_experts.token_dispatcher.plan(ids)
+    N = T * K
+    assert int(plan.counts_E.sum()) == N and int(plan.total_rows) == N
+    ros = plan.row_of_slot.long()
+    assert torch.equal(torch.sort(ros).values, torch.arange(N, device=DEV))
+    assert torch.equal(plan.slot_of_row.long()[ros], torch.arange(N, device=DEV))
+    assert torch.equal(plan.token_of_row.long(), plan.slot_of_row.long() // K)
+    sorted_ids = ids.reshape(-1)[plan.slot_of_row.long()]
+    assert bool((sorted_ids[1:] >= sorted_ids[:-1]).all()), "rows are not expert-major"
+    assert torch.equal(torch.bincount(ids.reshape(-1), minlength=E).int(), plan.counts_E)
+    assert bool((ids.sort(-1).values[:, 1:] != ids.sort(-1).values[:, :-1]).all()), "an expert chosen twice"
+
+    # --- exact linearity in w2 (power-of-two scaling commutes with every rounding)
+    ie = block.routed_experts.inner_experts
+    with torch.no_grad():
+        ie.w2_EDF.mul_(2.0)
+        out2 = block(x)
+        ie.w2_EDF.mul_(0.5)
+    assert torch.equal(out2, out * 2), "output is not exactly linear in w2"
+
+    # --- sampled tokens, recomputed one by one in fp32 on the device
+    w1, w3, w2 = ie.w1_EFD.detach(), ie.w3_EFD.detach(), ie.w2_EDF.detach()
+    sample = torch.randint(0, T, (48,), generator=g).tolist()
+    ref = torch.zeros(len(sample), D, device=DEV)
+    bf = lambda v: v.bfloat16().float()
+    for i, t in enumerate(sample):
+        xt = x[t].float()
+        for k in range(K):
+            e = int(ids[t, k])
+            gate, up = bf(w1[e].float() @ xt), bf(w3[e].float() @ xt)
+            h = bf(bf(torch.nn.functional.silu(gate)) * up)
+            ref[i] += float(scores[t, k]) * bf(w2[e].float() @ h)
+    assert rel_l2(out[sample].float(), ref) < 2e-2
+
+    # --- sampled experts: weight gradients from plain matmuls over the same intermediates
+    with torch.no_grad():
+        rows = ops.permute_rows_fwd(x, plan)
+        y, gate, up, h = ops.grouped_swiglu_fwd(rows, w1, w3, w2, plan)
+        dy, dsc = ops.combine_bwd(gout, y, scores, plan)
+    off = plan.seg_offsets.cpu().tolist()
+    for e in (0, 57, 127):
+        sl = slice(off[e], off[e + 1])
+        gf, uf, dyf = gate[sl].float(), up[sl].float(), dy[sl].float()
+        want_dw2 = dyf.T @ h[sl].float()
+        dh = bf(dyf @ w2[e].float())
+        sig = torch.sigmoid(gf)
+        dup = bf(dh * bf(gf * sig))
+        dgate = bf(bf(dh * uf) * (sig * (1 + gf * (1 - sig))))
+        assert rel_l2(dw2[e].float(), want_dw2) < 2e-2
+        assert rel_l2(dw1[e].float(), dgate.T @ rows[sl].float()) < 2e-2
+        assert rel_l2(dw3[e].float(), dup.T @ rows[sl].float()) < 2e-2
+    # router score gradient of the sampled tokens: <y[row], dout[t]>
+    for t in sample[:8]:
+        for k in range(K):
+            r = int(plan.row_of_slot[t * K + k])
+            want = float((y[r].float() * gout[t].float()).sum())
+            assert abs(float(dsc[t, k]) - want) <= 2e-2 * max(1.0, abs(want))
