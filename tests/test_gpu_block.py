@@ -293,3 +293,112 @@ def test_full_size_properties_qwen3_t8192():
             r = int(plan.row_of_slot[t * K + k])
             want = float((y[r].float() * gout[t].float()).sum())
             assert abs(float(dsc[t, k]) - want) <= 2e-2 * max(1.0, abs(want))
+
+
+def _sampled_token_reference(x, ids, weights, w1, w3, w2, sample, lo=0, hi=None):
+    """Token-by-token fp32 recomputation on the device with the bf16 rounding points of the
+    expert MLP; experts outside [lo, hi) contribute nothing (one rank's share)."""
+    bf = lambda v: v.bfloat16().float()
+    hi = w1.shape[0] + lo if hi is None else hi
+    ref = torch.zeros(len(sample), x.shape[1], device=x.device)
+    for i, t in enumerate(sample):
+        xt = x[t].float()
+        for k in range(ids.shape[1]):
+            e = int(ids[t, k])
+            if not lo <= e < hi:
+                continue
+            gate, up = bf(w1[e - lo].float() @ xt), bf(w3[e - lo].float() @ xt)
+            h = bf(bf(torch.nn.functional.silu(gate)) * up)
+            ref[i] += float(weights[t, k]) * bf(w2[e - lo].float() @ h)
+    return ref
+
+
+def test_full_size_properties_skewed_padded_t16384():
+    """T=16384 at the Qwen3 shape, Zipf(1.2)-skewed routing, 128-row padded segments: layout
+    invariants of the padded plan, determinism, sampled-token recomputation."""
+    print("block full size padded T=16384", flush=True)
+    T, D, E, K, F = 16384, 2048, 128, 8, 768
+    spec = R.RouterSpec(E, K, score_func="softmax", route_norm=True)
+    p = make_params(E, D, F, torch.bfloat16, seed=5)
+    p.router_logit_bias_E = -1.2 * torch.log(torch.arange(1, E + 1, dtype=torch.float32))
+    block = build_block(p, spec, D, F, torch.bfloat16, DEV, dispatcher="padded", pad_multiple=128)
+    block.train()
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn(T, D, generator=g).bfloat16().to(DEV)
+    gout = torch.randn(T, D, generator=g).bfloat16().to(DEV)
+
+    def run():
+        block.zero_grad(set_to_none=True)
+        xin = x.clone().requires_grad_()
+        out = block(xin)
+        out.backward(gout)
+        return out.detach(), xin.grad, block.routed_experts.inner_experts.w2_EDF.grad.clone()
+
+    first, second = run(), run()
+    for a, b in zip(first, second):
+        assert torch.equal(a, b) and torch.isfinite(a.float()).all()
+    with torch.no_grad():
+        scores, ids = block.router.route(x)
+        plan = block.routed_experts.token_dispatcher.plan(ids)
+    counts = torch.bincount(ids.reshape(-1), minlength=E)
+    assert torch.equal(plan.counts_E.long(), counts)
+    top = counts.sort(descending=True).values
+    assert float(top[: E // 5].sum()) / (T * K) > 0.45, "the load is not skewed"
+    padded = plan.seg_offsets[1:] - plan.seg_offsets[:-1]
+    assert torch.equal(padded.long(), counts + (-counts % 128))
+    total = int(plan.total_rows)
+    sor = plan.slot_of_row[:total].long()
+    real = sor >= 0
+    assert int(real.sum()) == T * K
+    assert torch.equal(torch.sort(sor[real]).values, torch.arange(T * K, device=DEV))
+    # padding sits at the end of each segment
+    off = plan.seg_offsets.long()
+    e_of_row = torch.bucketize(torch.arange(total, device=DEV), off[1:], right=True)
+    within = torch.arange(total, device=DEV) - off[e_of_row]
+    assert torch.equal(real, within < counts.to(DEV)[e_of_row])
+    ie = block.routed_experts.inner_experts
+    sample = torch.randint(0, T, (32,), generator=g).tolist()
+    ref = _sampled_token_reference(x, ids, scores, ie.w1_EFD.detach(), ie.w3_EFD.detach(), ie.w2_EDF.detach(), sample)
+    assert rel_l2(first[0][sample].float(), ref) < 2e-2
+
+
+def test_full_size_properties_deepseek_local_share():
+    """The DeepSeek-V3-shaped block at full size: T=4096, D=7168, 256 experts in 8 groups
+    (4 kept), sigmoid + bias, top-8, scale 2.5, F=2048, experts 0-31 computed here, one
+    shared expert of width 2048.  Group confinement, full-E statistics, sampled recomputation."""
+    print("block full size deepseek share", flush=True)
+    T, D, E, K, F = 4096, 7168, 256, 8, 2048
+    spec = R.RouterSpec(E, K, score_func="sigmoid", route_norm=True, route_scale=2.5,
+                        num_expert_groups=8, num_limited_groups=4)
+    p = make_params(E, D, F, torch.bfloat16, seed=7, shared_F=F, El=32)
+    p.expert_bias_E = torch.rand(E, generator=torch.Generator().manual_seed(2)) * 0.2 - 0.1
+    block = build_block(p, spec, D, F, torch.bfloat16, DEV, load_balance_coeff=1e-3, dispatcher="share", local=(0, 32))
+    block.train()
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(T, D, generator=g).bfloat16().to(DEV)
+    gout = torch.randn(T, D, generator=g).bfloat16().to(DEV)
+    xin = x.clone().requires_grad_()
+    out = block(xin)
+    out.backward(gout)
+    assert torch.isfinite(out.float()).all() and torch.isfinite(xin.grad.float()).all()
+    assert int(block.tokens_per_expert_E.sum().item()) == T * K
+    with torch.no_grad():
+        scores, ids = block.router.route(x, block.expert_bias_E)
+    groups = ids // 32
+    assert int(max(len(set(r)) for r in groups.cpu().tolist())) <= 4, "a token left its 4 groups"
+    assert bool((ids.sort(-1).values[:, 1:] != ids.sort(-1).values[:, :-1]).all())
+    torch.testing.assert_close(scores.sum(-1), torch.full((T,), 2.5, device=DEV), rtol=1e-5, atol=1e-5)
+    ie = block.routed_experts.inner_experts
+    sample = torch.randint(0, T, (24,), generator=g).tolist()
+    ref = _sampled_token_reference(x, ids, scores, ie.w1_EFD.detach(), ie.w3_EFD.detach(), ie.w2_EDF.detach(),
+                                   sample, lo=0, hi=32)
+    sh = block.shared_experts
+    bf = lambda v: v.bfloat16().float()
+    for i, t in enumerate(sample):
+        xt = x[t].float()
+        gate, up = bf(sh.gate_proj.weight.float() @ xt), bf(sh.up_proj.weight.float() @ xt)
+        ref[i] += bf(sh.down_proj.weight.float() @ bf(bf(torch.nn.functional.silu(gate)) * up))
+    assert rel_l2(out.detach()[sample].float(), ref) < 2e-2
+    local_rows = int((ids < 32).sum())
+    assert 0 < local_rows < T * K
+    assert ie.w1_EFD.grad is not None and torch.isfinite(ie.w1_EFD.grad.float()).all()
