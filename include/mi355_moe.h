@@ -112,6 +112,28 @@ int mi355_router_select_bwd(const float* logits_TE, const int64_t* ids_TK,
                             int score_func, int route_norm, float route_scale,
                             int select_mode, void* stream);
 
+/*
+ * Per-forward load-balance loss on the dense score map and the routing map:
+ *   f_e = E * counts_e / max(sum counts, 1e-12),  counts_e = sum_t map[t][e]
+ *   p_e = sum_t s[t][e] / max(sum_e s[t][e], 1e-12)   (padding tokens contribute 0)
+ *   loss = sum_e f_e * p_e            (the value is T * L_bal; the caller's 1/tokens
+ *                                      normalisation makes it coeff * L_bal)
+ * Replaces MicrobatchWiseLoadBalanceLoss.forward up to inject(),
+ * llmtuner/models/common/moe/auxiliary_loss.py:147-162 (single process: no token-axis
+ * reduction).  routing_map_TE: (T,E) bytes, non-zero = chosen; padding_mask_T: (T) bytes
+ * or NULL; loss: 1 float; f_E: (E) floats kept for the backward; workspace:
+ * mi355_balance_loss_workspace_bytes().  E <= 1024.
+ * The backward writes d loss / d scores * grad_loss[0] into dscores_TE (the map carries no
+ * gradient): (f_j - sum_e f_e s'_e) / S_t, zero rows for padding tokens.
+ */
+int64_t mi355_balance_loss_workspace_bytes(int64_t T, int64_t E);
+int mi355_balance_loss_fwd(const float* scores_TE, const uint8_t* routing_map_TE,
+                           const uint8_t* padding_mask_T, float* loss, float* f_E,
+                           void* workspace, int64_t T, int64_t E, void* stream);
+int mi355_balance_loss_bwd(const float* scores_TE, const float* f_E,
+                           const uint8_t* padding_mask_T, const float* grad_loss,
+                           float* dscores_TE, int64_t T, int64_t E, void* stream);
+
 /* ------------------------------------------------------- permutation plan */
 
 /*

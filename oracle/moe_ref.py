@@ -284,6 +284,22 @@ def combine(y_RD, tok_R, s_sorted_R, x_TD, accumulate_in_fp32=False):
     return out.to(x_TD.dtype)
 
 
+def balance_loss(scores_TE, routing_map_TE, padding_mask_T=None):
+    """``MicrobatchWiseLoadBalanceLoss.forward`` up to ``inject``
+    (llmtuner/models/common/moe/auxiliary_loss.py:147-162), one process: counts from the
+    (already padding-filtered) map, ``f = normalize(counts, p=1) * E``, per-token
+    L1-normalised scores with padding rows zeroed, ``loss = sum f * p``."""
+    import torch.nn.functional as F
+
+    counts_E = routing_map_TE.to(scores_TE.dtype).sum(dim=0)
+    f_E = F.normalize(counts_E, p=1, dim=0) * scores_TE.size(-1)
+    probs_TE = F.normalize(scores_TE, p=1, dim=-1)
+    if padding_mask_T is not None:
+        probs_TE = probs_TE * ~padding_mask_T.unsqueeze(-1)
+    p_E = probs_TE.sum(dim=0)
+    return (f_E * p_E).sum()
+
+
 def shared_expert(x_TD, gate_w_FD, up_w_FD, down_w_DF):
     """The HF dense MLP reused as the shared expert (block_conversion.py:278-291)."""
     return F.linear(F.silu(F.linear(x_TD, gate_w_FD)) * F.linear(x_TD, up_w_FD), down_w_DF)

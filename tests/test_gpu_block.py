@@ -402,3 +402,47 @@ def test_full_size_properties_deepseek_local_share():
     local_rows = int((ids < 32).sum())
     assert 0 < local_rows < T * K
     assert ie.w1_EFD.grad is not None and torch.isfinite(ie.w1_EFD.grad.float()).all()
+
+
+@pytest.mark.parametrize("score_func,with_padding", [("sigmoid", True), ("softmax", False)])
+def test_balance_loss_hook_injects_the_reference_gradient(score_func, with_padding):
+    """An attached MicrobatchWiseLoadBalanceLoss adds coeff / tokens * d(sum f p) to the
+    router's gradient path and accumulates its metric; fp32 so the bar is 1e-5."""
+    print(f"block aux loss {score_func}", flush=True)
+    from torchllmtuner_amd import moe
+
+    T, D, E, K, F = 320, 128, 8, 2, 64
+    coeff, denom = 3000.0, 300.0  # large on purpose: the aux term must be visible next to the main gradient
+    spec = R.RouterSpec(E, K, score_func=score_func, route_norm=True)
+    p = make_params(E, D, F, torch.float32, seed=11, std=0.1)
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(T, D, generator=g)
+    gout = torch.randn(T, D, generator=g)
+    pad = (torch.rand(T, generator=g) < 0.15) if with_padding else None
+
+    leaves = {k: getattr(p, k).clone().requires_grad_() for k in ("router_w_ED", "w1_EFD", "w3_EFD", "w2_EDF")}
+    xr = x.clone().requires_grad_()
+    ref, aux = R.moe_forward(xr, R.MoEParams(**leaves), spec)
+    rmap = R.routing_map(aux["ids_TK"], E)
+    if pad is not None:
+        rmap = rmap & ~pad[:, None]
+    raw = R.balance_loss(R.score(aux["logits"], score_func), rmap, pad)
+    ((ref * gout).sum() + raw * (coeff / denom)).backward()
+
+    block = build_block(p, spec, D, F, torch.float32, DEV)
+    block.router.aux_loss = moe.MicrobatchWiseLoadBalanceLoss(coeff=coeff).to(DEV)
+    block.train()
+    moe.AuxLoss.set_step_denominator(torch.tensor(denom), model_parts=[block])
+    xd = x.to(DEV).requires_grad_()
+    out = block(xd, padding_mask=None if pad is None else pad.to(DEV))
+    out.backward(gout.to(DEV))
+    assert rel_max(out, ref) < 1e-5
+    assert abs(float(block.router.aux_loss.instance_acc) - float(raw.detach()) / denom) < 1e-5 * max(1.0, float(raw.detach()) / denom)
+    assert rel_max(block.router.gate.weight.grad, leaves["router_w_ED"].grad) < 1e-5
+    assert rel_max(xd.grad, xr.grad) < 1e-5
+    # and it is the aux term that moved the router gradient
+    block.zero_grad(set_to_none=True)
+    block.router.aux_loss = None
+    xd2 = x.to(DEV).requires_grad_()
+    block(xd2).backward(gout.to(DEV))
+    assert rel_max(block.router.gate.weight.grad, leaves["router_w_ED"].grad) > 1e-4

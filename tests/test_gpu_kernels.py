@@ -304,3 +304,31 @@ def test_grouped_experts_bf16_generic_shapes(ops, counts, D, Fd):
 def test_grouped_experts_bf16_mfma(ops, counts, D, Fd):
     print(f"experts bf16 mfma {counts} D={D} F={Fd}", flush=True)
     _experts_case(ops, torch.bfloat16, counts, D, Fd, std=0.05)
+
+
+# ---------------------------------------------------------------- balance loss
+@pytest.mark.parametrize("T,E,K,padded", [(12, 4, 2, False), (1000, 128, 8, True), (4096, 256, 8, True),
+                                          (0, 8, 2, False), (77, 320, 5, False)])
+def test_balance_loss_fwd_bwd(ops, T, E, K, padded):
+    print(f"balance loss T={T} E={E}", flush=True)
+    g = torch.Generator().manual_seed(3)
+    s = torch.rand(T, E, generator=g)
+    m = torch.zeros(T, E, dtype=torch.bool)
+    if T:
+        m.scatter_(-1, torch.topk(s, K).indices, True)
+    pad = None
+    if padded:
+        pad = torch.rand(T, generator=g) < 0.1
+        m &= ~pad[:, None]
+    sr = s.clone().requires_grad_()
+    ref = R.balance_loss(sr, m, pad)
+    loss, f_E = ops.balance_loss_fwd(s.to(DEV), m.to(DEV), None if pad is None else pad.to(DEV))
+    assert abs(float(loss) - float(ref.detach())) <= 1e-5 * max(1.0, abs(float(ref.detach())))
+    if T == 0:
+        return
+    ref.backward()
+    grad = ops.balance_loss_bwd(s.to(DEV), f_E, torch.tensor(1.0, device=DEV), None if pad is None else pad.to(DEV))
+    assert rel_max(grad, sr.grad) < FP32_TOL
+    # twice the upstream gradient, twice the result
+    grad2 = ops.balance_loss_bwd(s.to(DEV), f_E, torch.tensor(2.0, device=DEV), None if pad is None else pad.to(DEV))
+    assert torch.equal(grad2, grad * 2)

@@ -392,3 +392,44 @@ def test_block_analytic_experts():
             y = p.w2_EDF[e] @ (F.silu(p.w1_EFD[e] @ x[t]) * (p.w3_EFD[e] @ x[t]))
             want[t] += aux["scores_TK"][t, k].double() * (e + 1) * y
     torch.testing.assert_close(out, want, rtol=1e-10, atol=1e-12)
+
+
+# ---- per-forward load-balance loss --------------------------------------------
+def _routing_from_scores(scores_TE, k):
+    routing = torch.zeros_like(scores_TE, dtype=torch.bool)
+    routing.scatter_(-1, torch.topk(scores_TE.detach(), k).indices, True)
+    return routing
+
+
+def test_balance_loss_matches_the_paper_formula_and_invariants():
+    # tests/unit_tests/cpu/models/test_aux_loss.py:465-571
+    torch.manual_seed(0)
+    T, E, K = 12, 4, 2
+    s = torch.rand(T, E)
+    m = _routing_from_scores(s, K)
+    counts = m.float().sum(0)
+    f = (E / (K * T)) * counts                      # eq. 18 with T explicit
+    p = (s / s.sum(-1, keepdim=True)).sum(0)        # eq. 19 times T
+    torch.testing.assert_close(R.balance_loss(s, m), (f * p).sum(), atol=1e-6, rtol=0)
+    # scale and token-order invariance
+    torch.testing.assert_close(R.balance_loss(s * 1000.0, m), R.balance_loss(s, m), rtol=1e-5, atol=0)
+    perm = torch.randperm(T)
+    torch.testing.assert_close(R.balance_loss(s[perm], m[perm]), R.balance_loss(s, m), rtol=1e-6, atol=0)
+    # even load, uniform scores: f_i = 1, sum_i p_i = T
+    T2, E2 = 8, 4
+    even = torch.zeros(T2, E2, dtype=torch.bool)
+    even[torch.arange(T2), torch.arange(T2) % E2] = True
+    assert R.balance_loss(torch.ones(T2, E2), even).item() == pytest.approx(float(T2))
+    # padding rows drop out of p; the gradient reaches the scores, not the map
+    pad = torch.zeros(T, dtype=torch.bool); pad[3] = pad[7] = True
+    keep = ~pad
+    torch.testing.assert_close(R.balance_loss(s, m & keep[:, None], pad),
+                               R.balance_loss(s[keep], m[keep]), rtol=1e-6, atol=0)
+    sg = s.clone().requires_grad_()
+    R.balance_loss(sg, m).backward()
+    assert sg.grad.abs().sum() > 0
+    # closed-form gradient: (f_j - <f, s'_t>) / S_t
+    S = s.sum(-1, keepdim=True)
+    fE = counts / counts.sum() * E
+    want = (fE[None, :] - (s / S * fE).sum(-1, keepdim=True)) / S
+    torch.testing.assert_close(sg.grad, want, rtol=1e-5, atol=1e-6)

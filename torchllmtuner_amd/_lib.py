@@ -28,6 +28,9 @@ SIGNATURES = {
     "mi355_router_gate_fwd": (I, [P, I, P, I, P, P, P, L, L, L, P]),
     "mi355_router_gate_bwd_workspace_bytes": (L, [L, L, L]),
     "mi355_router_gate_bwd": (I, [P, P, I, P, I, P, P, P, L, L, L, P]),
+    "mi355_balance_loss_workspace_bytes": (L, [L, L]),
+    "mi355_balance_loss_fwd": (I, [P, P, P, P, P, P, L, L, P]),
+    "mi355_balance_loss_bwd": (I, [P, P, P, P, P, L, L, P]),
     "mi355_router_select_fwd": (I, [P, P, P, P, P, L, L, L, I, I, F, I, I, I, P]),
     "mi355_router_select_bwd": (I, [P, P, P, P, P, L, L, L, I, I, F, I, P]),
     "mi355_permute_plan_workspace_bytes": (L, [L, L, L]),

@@ -1,6 +1,7 @@
 """The native MoE block (router, dispatchers, grouped experts) on MI355X kernels."""
 
 from .activation import SwiGLU
+from .auxiliary_loss import AuxLoss, MicrobatchWiseLoadBalanceLoss
 from .experts import DenseSwiGLU, DispatchObservation, ExpertErrorCapture, GroupedExperts, RoutedExperts
 from .layer import MoE
 from .linear import RouterGateLinear
@@ -13,6 +14,7 @@ from .token_dispatch import (
 )
 
 __all__ = [
+    "AuxLoss",
     "DenseSwiGLU",
     "DispatchObservation",
     "ExpertErrorCapture",
@@ -20,6 +22,7 @@ __all__ = [
     "LocalDispatchMetadata",
     "LocalShareTokenDispatcher",
     "LocalTokenDispatcher",
+    "MicrobatchWiseLoadBalanceLoss",
     "MoE",
     "PaddedTokenDispatcher",
     "RoutedExperts",

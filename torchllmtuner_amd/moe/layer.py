@@ -13,20 +13,19 @@ from __future__ import annotations
 
 import math
 from collections.abc import Iterator
-from contextvars import ContextVar
 from numbers import Real
 
 import torch
 import torch.nn as nn
 
+from .auxiliary_loss import in_checkpoint_recompute
 from .experts import RoutedExperts
 from .routing import TokenChoiceTopKRouter
 
 __all__ = ["MoE", "in_checkpoint_recompute"]
 
-# Set by an activation-checkpointing wrapper while it replays a forward; counter
-# updates are skipped there (llmtuner/models/common/aux_loss.py:47-68).
-in_checkpoint_recompute: ContextVar[bool] = ContextVar("in_checkpoint_recompute", default=False)
+# in_checkpoint_recompute is set by an activation-checkpointing wrapper while it replays a
+# forward; counter updates are skipped there (llmtuner/models/common/aux_loss.py:47-68).
 
 
 class MoE(nn.Module):

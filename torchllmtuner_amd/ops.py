@@ -137,6 +137,42 @@ def router_select_bwd(logits_TE, ids_TK, dweights_TK, dscores_TE, score_func, ro
     return out
 
 
+def balance_loss_fwd(scores_TE, routing_map_TE, padding_mask_T=None):
+    """Returns (loss 0-d fp32, f_E) of the per-forward load-balance loss."""
+    dev = _dev(scores_TE, routing_map_TE, padding_mask_T)
+    if scores_TE.dtype != torch.float32:
+        raise TypeError("router scores must be float32")
+    scores_TE = _c(scores_TE)
+    T, E = scores_TE.shape
+    if routing_map_TE.shape != scores_TE.shape:
+        raise ValueError(f"routing map {tuple(routing_map_TE.shape)} does not match scores {tuple(scores_TE.shape)}")
+    as_bytes = lambda m: _c(m).view(torch.uint8) if m.dtype == torch.bool else _c(m.ne(0)).view(torch.uint8)
+    rmap = as_bytes(routing_map_TE)
+    pad = None if padding_mask_T is None else as_bytes(padding_mask_T)
+    lib = _lib.load()
+    out = torch.empty(1 + E, dtype=torch.float32, device=dev)
+    ws = torch.empty(max(lib.mi355_balance_loss_workspace_bytes(T, E), 4), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        rc = lib.mi355_balance_loss_fwd(_p(scores_TE), _p(rmap), _p(pad), _p(out), out[1:].data_ptr(), _p(ws),
+                                        T, E, _stream(dev))
+    _lib.check(rc, "balance_loss_fwd")
+    return out[0], out[1:]
+
+
+def balance_loss_bwd(scores_TE, f_E, grad_loss, padding_mask_T=None):
+    dev = _dev(scores_TE, f_E, grad_loss, padding_mask_T)
+    scores_TE = _c(scores_TE)
+    T, E = scores_TE.shape
+    pad = None if padding_mask_T is None else _c(padding_mask_T).view(torch.uint8)
+    g = _c(grad_loss.float().reshape(1))
+    out = torch.empty_like(scores_TE)
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_balance_loss_bwd(_p(scores_TE), _p(_c(f_E)), _p(pad), _p(g), _p(out), T, E,
+                                                _stream(dev))
+    _lib.check(rc, "balance_loss_bwd")
+    return out
+
+
 # ------------------------------------------------------------------ plan
 @dataclass
 class PermutePlan:
