@@ -2,6 +2,12 @@
 
 from .activation import SwiGLU
 from .auxiliary_loss import AuxLoss, MicrobatchWiseLoadBalanceLoss
+from .convert import (
+    hf_expert_state_to_native,
+    moe_from_packed_experts,
+    native_ep_expert_key,
+    native_expert_state_to_hf,
+)
 from .experts import DenseSwiGLU, DispatchObservation, ExpertErrorCapture, GroupedExperts, RoutedExperts
 from .layer import MoE
 from .linear import RouterGateLinear
@@ -29,4 +35,8 @@ __all__ = [
     "RouterGateLinear",
     "SwiGLU",
     "TokenChoiceTopKRouter",
+    "hf_expert_state_to_native",
+    "moe_from_packed_experts",
+    "native_ep_expert_key",
+    "native_expert_state_to_hf",
 ]
