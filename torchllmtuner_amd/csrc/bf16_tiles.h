@@ -8,7 +8,7 @@
 //       c ^ ((r >> 1) & 7); a fragment is one ds_read_b128 (measured conflict-free;
 //       the key r & 7 costs a 2-way conflict).
 //   KS  contraction axis strided in HBM: [k][cols], chunk c of row k stored at
-//       c ^ ((k & 3) << 1); a fragment is two ds_read_b64_tr_b16 (LDS transpose
+//       c ^ ((k & 3) << 2) (16 chunks or more per row); a fragment is two ds_read_b64_tr_b16 (LDS transpose
 //       reads: lane i of a 16-lane group supplies the address of row i/4, 8-byte
 //       piece i%4, and receives column i of the four rows).
 // v_mfma_f32_32x32x16_bf16 takes per lane 8 bf16 of each operand (row lane%32,
@@ -27,6 +27,11 @@ typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int BK = 64;
 
+// KS swizzle key of LDS row k, in 16-byte chunks: a transpose read touches four
+// consecutive k rows and 64 bytes of each per 32 lanes, and rows are a multiple of
+// 256 bytes apart, so each row's four chunks are moved to their own quarter of the banks.
+__device__ __forceinline__ int ks_key(int k) { return (k & 3) << 2; }
+
 #define LDS_PTR(p) ((__attribute__((address_space(3))) s16x4*)(p))
 
 // ---- fragment reads -----------------------------------------------------------------
@@ -41,7 +46,7 @@ __device__ __forceinline__ bf16x8 frag_ks(const uint16_t* tile, int col, int kk,
   const int g = lane >> 4, i = lane & 15;
   const int k = kk * 16 + 8 * (g >> 1) + (i >> 2);  // k & 3 == i >> 2 for both reads
   const int c = col + 16 * (g & 1) + 4 * (i & 3);
-  const int off = (((c >> 3) ^ ((k & 3) << 1)) << 3) + (c & 7);
+  const int off = (((c >> 3) ^ ks_key(k)) << 3) + (c & 7);
   const uint16_t* p = tile + k * COLS + off;
   const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(p));
   const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(p + 4 * COLS));

@@ -160,7 +160,7 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
       constexpr int CPR = BNT / 8;  // chunks per k row
       const int q = tid + NT * i;
       const int k = q / CPR, cc = q % CPR;
-      b_lds[i] = k * BNT + ((cc ^ ((k & 3) << 1)) << 3);
+      b_lds[i] = k * BNT + ((cc ^ ks_key(k)) << 3);
     }
   }
   int bcol[NJ];
@@ -488,7 +488,7 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int k = ks_k + 16 * i;
-    lds_off[i] = k * 256 + ((ks_chunk ^ ((k & 3) << 1)) << 3);
+    lds_off[i] = k * 256 + ((ks_chunk ^ ks_key(k)) << 3);
   }
   const u32x4 zero = {0, 0, 0, 0};
 

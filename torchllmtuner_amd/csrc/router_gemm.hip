@@ -24,7 +24,7 @@ __device__ __forceinline__ int kc_off(int row, int chunk) {
 }
 template <int COLS>
 __device__ __forceinline__ int ks_off(int k, int chunk) {
-  return k * COLS + ((chunk ^ ((k & 3) << 1)) << 3);
+  return k * COLS + ((chunk ^ ks_key(k)) << 3);
 }
 
 // 8 consecutive fp32 -> three 16-byte chunks of bf16 pieces (hi, mid, lo)
