@@ -22,6 +22,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
@@ -54,6 +55,34 @@ __device__ __forceinline__ bf16x8 frag_ks(const uint16_t* tile, int col, int kk,
   return __builtin_bit_cast(bf16x8, v);
 }
 
+// ---- fragments for v_mfma_f32_16x16x32_bf16 -------------------------------------------
+// Per lane 8 bf16 of each operand: row lane%16, k = 8*(lane/16)..+7 of a 32-wide K block;
+// 4 fp32 of the result: column lane%16, rows 4*(lane/16) + i.  With random operand bits
+// this shape sustains about 14 % more than 32x32x16 on MI355X (a quarter of the
+// accumulator bytes per instruction for half the flops, and power is what limits both).
+__device__ __forceinline__ bf16x8 frag16_kc(const uint16_t* tile, int row, int kk32, int lane) {
+  const int r = row + (lane & 15);
+  const int c = kk32 * 4 + (lane >> 4);
+  return *reinterpret_cast<const bf16x8*>(tile + r * BK + ((c ^ ((r >> 1) & 7)) << 3));
+}
+
+// KS key for the 16x16x32 reader: 32 lanes of a transpose read touch rows k..k+3 and
+// k+8..k+11, 32 bytes of each, so the eight rows get an eighth of the banks each.
+__device__ __forceinline__ int ks_key16(int k) { return ((k & 3) << 2) | (((k >> 3) & 1) << 1); }
+
+template <int COLS>
+__device__ __forceinline__ bf16x8 frag16_ks(const uint16_t* tile, int col, int kk32, int lane) {
+  const int g = lane >> 4, i = lane & 15;
+  const int k = kk32 * 32 + 8 * g + (i >> 2);  // key of row k + 4 equals that of row k
+  const int c = col + 4 * (i & 3);
+  const int off = (((c >> 3) ^ ks_key16(k)) << 3) + (c & 7);
+  const uint16_t* p = tile + k * COLS + off;
+  const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(p));
+  const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(p + 4 * COLS));
+  const s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(bf16x8, v);
+}
+
 // Workgroup barrier that waits for this wave's own LDS operations only: global loads and
 // stores stay in flight across it.
 __device__ __forceinline__ void phase_barrier() {
@@ -78,6 +107,15 @@ struct WaveStage {
                                               float v0, float v1, float v2, float v3) {
     const int m = mi * 32 + (lane & 31);
     const int n = col0 + q * 8 + (lane >> 5) * 4;
+    u32x2 pk = {pack2(v0, v1), pack2(v2, v3)};
+    *reinterpret_cast<u32x2*>(st + m * PITCH + n) = pk;
+  }
+  // the same for a 16 x 16 accumulator tile (mi-th 16 rows): lane = row lane & 15,
+  // registers = columns col0 + 4 * (lane >> 4) .. + 3
+  __device__ static __forceinline__ void put16(uint16_t* st, int mi, int col0, int lane, float v0, float v1,
+                                               float v2, float v3) {
+    const int m = mi * 16 + (lane & 15);
+    const int n = col0 + 4 * (lane >> 4);
     u32x2 pk = {pack2(v0, v1), pack2(v2, v3)};
     *reinterpret_cast<u32x2*>(st + m * PITCH + n) = pk;
   }

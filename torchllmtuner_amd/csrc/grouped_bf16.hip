@@ -40,9 +40,10 @@
 // the queue once per K step.  Operand addresses are a wave-uniform 64-bit base plus a
 // fixed 32-bit per-thread offset.
 //
-// MFMA: v_mfma_f32_32x32x16_bf16.  Per lane 8 bf16 of each operand (row lane%32,
-// k = 8*(lane/32)..+7), 16 fp32 of the result (column lane%32, rows
-// 8*(i/4) + 4*(lane/32) + i%4).  The weight tile is passed as the FIRST operand
+// MFMA of the row-tiled kernels: v_mfma_f32_16x16x32_bf16.  Per lane 8 bf16 of each operand (row lane%16,
+// k = 8*(lane/16)..+7), 4 fp32 of the result (column lane%16, rows 4*(lane/16) + i).
+// With random operand bits this shape sustains about 14 % more than 32x32x16 on this
+// card (2.17 against 1.90 PFLOP/s register-resident, +7 % in a whole K loop).  The weight tile is passed as the FIRST operand
 // and the activation tile as the second, so a lane ends up with four CONSECUTIVE
 // output columns of one output row: epilogues pack them and go through LDS to
 // write 16-byte, fully coalesced rows.
@@ -160,16 +161,19 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
       constexpr int CPR = BNT / 8;  // chunks per k row
       const int q = tid + NT * i;
       const int k = q / CPR, cc = q % CPR;
-      b_lds[i] = k * BNT + ((cc ^ ks_key(k)) << 3);
+      b_lds[i] = k * BNT + ((cc ^ ks_key16(k)) << 3);
     }
   }
-  int bcol[NJ];
+  // a wave's 64 x (32 NJ) accumulator tile is 4 x NJ2 MFMA tiles of 16 x 16; with
+  // gate/up the first NJ column tiles are gate columns, the last NJ the same f of up
+  constexpr int NJ2 = 2 * NJ;
+  int bcol[NJ2];
 #pragma unroll
-  for (int nj = 0; nj < NJ; ++nj) {
+  for (int nj = 0; nj < NJ2; ++nj) {
     if constexpr (MODE == RM_GATEUP)
-      bcol[nj] = (nj < 2 ? 0 : BNT / 2) + wn * 64 + (nj & 1) * 32;
+      bcol[nj] = (nj < NJ ? 0 : BNT / 2) + wn * (16 * NJ) + (nj % NJ) * 16;
     else
-      bcol[nj] = wn * (32 * NJ) + nj * 32;
+      bcol[nj] = wn * (32 * NJ) + nj * 16;
   }
 
   // Operand addresses are a wave-uniform 64-bit base (tile, K step, chunk index) plus a
@@ -263,13 +267,13 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
   load_asrc(nxt, nsrc);
   const int row0 = cur.row0, valid = cur.valid, n0 = cur.n0;
 
-  f32x16 acc[2][NJ];
+  f32x4 acc[4][NJ2];
 #pragma unroll
-  for (int mi = 0; mi < 2; ++mi)
+  for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
-    for (int nj = 0; nj < NJ; ++nj)
+    for (int nj = 0; nj < NJ2; ++nj)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) acc[mi][nj][i] = 0.0f;
+      for (int i = 0; i < 4; ++i) acc[mi][nj][i] = 0.0f;
 
   // K step 0 (requested before the previous epilogue) -> LDS stage 0, K step 1 -> registers
 #pragma unroll
@@ -284,10 +288,10 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
   // so that every load of the steady-state loop is unconditional: the compiler can then
   // count outstanding loads exactly and wait only for the three oldest before each park,
   // instead of draining the queue (vmcnt(0)) once per K step.
-  // The last tile of an expert is partly empty: a wave skips the MFMAs of its 32-row
+  // The last tile of an expert is partly empty: a wave skips the MFMAs of its 16-row
   // blocks that hold no real rows (a wave-uniform branch; operands are still staged and
   // every barrier met).
-  const int act = min(max((valid - wave_m + 31) >> 5, 0), 2);
+  const int act = min(max((valid - wave_m + 15) >> 4, 0), 4);
   auto kstep = [&](int ks, auto has_next_t, auto has_next2_t) {
     constexpr bool has_next = decltype(has_next_t)::value;
     constexpr bool has_next2 = decltype(has_next2_t)::value;
@@ -296,37 +300,43 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
     uint16_t* An = smem + ((ks + 1) & 1) * STAGE;
     uint16_t* Bn = An + RBM * BK;
 #pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk) {
-      bf16x8 af[2], bf[NJ];
+    for (int kk = 0; kk < BK / 32; ++kk) {
+      bf16x8 af[4];
 #pragma unroll
-      for (int mi = 0; mi < 2; ++mi) af[mi] = frag_kc(As, wm + mi * 32, kk, lane);
+      for (int mi = 0; mi < 4; ++mi) af[mi] = frag16_kc(As, wm + mi * 16, kk, lane);
 #pragma unroll
-      for (int nj = 0; nj < NJ; ++nj) {
-        if constexpr (B_KS)
-          bf[nj] = frag_ks<BNT>(Bs, bcol[nj], kk, lane);
-        else
-          bf[nj] = frag_kc(Bs, bcol[nj], kk, lane);
-      }
-      // a quarter of the staging traffic rides along with each quarter of the MFMAs:
-      // park the held chunks of tile ks+1 in the other LDS stage, then refill the
-      // same registers with the same chunks of tile ks+2.
-      if constexpr (has_next) {
-        if (kk < 2) *reinterpret_cast<u32x4*>(An + kc_lds + kk * 64 * BK) = ra[kk];
+      for (int hb = 0; hb < 2; ++hb) {
+        bf16x8 bf[NJ];
 #pragma unroll
-        for (int i = (kk * NB) / 4; i < ((kk + 1) * NB) / 4; ++i)
-          *reinterpret_cast<u32x4*>(Bn + b_lds[i]) = rb[i];
-      }
-      if constexpr (has_next2) {
-        if (kk < 2) ra[kk] = load_a(kofs(ks + 2), kk);
+        for (int b = 0; b < NJ; ++b) {
+          if constexpr (B_KS)
+            bf[b] = frag16_ks<BNT>(Bs, bcol[hb * NJ + b], kk, lane);
+          else
+            bf[b] = frag16_kc(Bs, bcol[hb * NJ + b], kk, lane);
+        }
+        // a quarter of the staging traffic rides along with each quarter of the MFMAs:
+        // park the held chunks of tile ks+1 in the other LDS stage, then refill the
+        // same registers with the same chunks of tile ks+2.
+        const int q = kk * 2 + hb;
+        if constexpr (has_next) {
+          if (q < 2) *reinterpret_cast<u32x4*>(An + kc_lds + q * 64 * BK) = ra[q];
 #pragma unroll
-        for (int i = (kk * NB) / 4; i < ((kk + 1) * NB) / 4; ++i) rb[i] = load_b(kofs(ks + 2), i);
-      }
+          for (int i = (q * NB) / 4; i < ((q + 1) * NB) / 4; ++i)
+            *reinterpret_cast<u32x4*>(Bn + b_lds[i]) = rb[i];
+        }
+        if constexpr (has_next2) {
+          if (q < 2) ra[q] = load_a(kofs(ks + 2), q);
 #pragma unroll
-      for (int mi = 0; mi < 2; ++mi) {
-        if (mi < act) {
+          for (int i = (q * NB) / 4; i < ((q + 1) * NB) / 4; ++i) rb[i] = load_b(kofs(ks + 2), i);
+        }
 #pragma unroll
-          for (int nj = 0; nj < NJ; ++nj)
-            acc[mi][nj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[nj], af[mi], acc[mi][nj], 0, 0, 0);
+        for (int mi = 0; mi < 4; ++mi) {
+          if (mi < act) {
+#pragma unroll
+            for (int b = 0; b < NJ; ++b)
+              acc[mi][hb * NJ + b] =
+                  __builtin_amdgcn_mfma_f32_16x16x32_bf16(bf[b], af[mi], acc[mi][hb * NJ + b], 0, 0, 0);
+          }
         }
       }
     }
@@ -347,8 +357,8 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
   }
 
   // ---- epilogue: through the wave's private LDS region, 16-byte coalesced rows ---------
-  // acc[mi][nj][i]: output row = wm + mi*32 + (lane&31); output column within the nj-th
-  // 32-column group = (i>>2)*8 + (lane>>5)*4 + (i&3).
+  // acc[mi][nj][i]: output row = wm + mi*16 + (lane&15); output column within the nj-th
+  // 16-column tile = 4*(lane>>4) + i.
   uint16_t* st = smem + wave * (64 * 136);  // 8 waves x 17 KiB < 160 KiB; the barrier ending the K loop freed the tiles
   if constexpr (MODE == RM_GATEUP) {
     // per 32-row half: three 32 x 64 tiles gate | up | h at columns 0, 64, 128 of a
@@ -357,23 +367,24 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
     uint16_t* sg = smem + wave * (32 * S::PITCH);
     const int f0 = n0 + wn * 64;
 #pragma unroll
-    for (int mi = 0; mi < 2; ++mi) {
-      if (wave_m + mi * 32 >= valid) continue;  // no real rows in this half (uniform per wave)
+    for (int half = 0; half < 2; ++half) {
+      if (wave_m + half * 32 >= valid) continue;  // no real rows in this half (uniform per wave)
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int ml = 0; ml < 2; ++ml)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
+        for (int j = 0; j < NJ; ++j) {
+          const int mi = half * 2 + ml;
           float g[4], u[4], h[4];
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            g[r] = round_bf16(acc[mi][j][q * 4 + r]);
-            u[r] = round_bf16(acc[mi][j + 2][q * 4 + r]);
+            g[r] = round_bf16(acc[mi][j][r]);
+            u[r] = round_bf16(acc[mi][j + NJ][r]);
             const float s = round_bf16(g[r] * fast_sigmoid(g[r]));
             h[r] = s * u[r];
           }
-          S::put4(sg, 0, j * 32, lane, q, g[0], g[1], g[2], g[3]);
-          S::put4(sg, 0, 64 + j * 32, lane, q, u[0], u[1], u[2], u[3]);
-          S::put4(sg, 0, 128 + j * 32, lane, q, h[0], h[1], h[2], h[3]);
+          S::put16(sg, ml, j * 16, lane, g[0], g[1], g[2], g[3]);
+          S::put16(sg, ml, 64 + j * 16, lane, u[0], u[1], u[2], u[3]);
+          S::put16(sg, ml, 128 + j * 16, lane, h[0], h[1], h[2], h[3]);
         }
       __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the wave's own LDS writes have landed
       __builtin_amdgcn_wave_barrier();
@@ -383,7 +394,7 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
         const int idx = it * 64 + lane;
         const int m = idx / 24, rem = idx % 24, t = rem >> 3, c = rem & 7;
         const int f = f0 + c * 8;
-        const int mr = wm + mi * 32 + m;
+        const int mr = wm + half * 32 + m;
         if (mr < valid && f < F) {
           const u32x4 v = *reinterpret_cast<const u32x4*>(sg + m * S::PITCH + t * 64 + c * 8);
           uint16_t* dst = (t == 0 ? p.o0 : (t == 1 ? p.o1 : p.o2)) + static_cast<int64_t>(row0 + mr) * F + f;
@@ -397,13 +408,10 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
     using S = WaveStage<32 * NJ>;
     constexpr int CH = 4 * NJ;  // 16-byte chunks per row of the wave's sub-tile
 #pragma unroll
-    for (int mi = 0; mi < 2; ++mi)
+    for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
-      for (int nj = 0; nj < NJ; ++nj)
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-          S::put4(st, mi, nj * 32, lane, q, acc[mi][nj][q * 4], acc[mi][nj][q * 4 + 1],
-                  acc[mi][nj][q * 4 + 2], acc[mi][nj][q * 4 + 3]);
+      for (int nj = 0; nj < NJ2; ++nj)
+        S::put16(st, mi, nj * 16, lane, acc[mi][nj][0], acc[mi][nj][1], acc[mi][nj][2], acc[mi][nj][3]);
     __builtin_amdgcn_s_waitcnt(0xc07f);
     __builtin_amdgcn_wave_barrier();
     const int c0 = n0 + wn * (32 * NJ);
@@ -564,6 +572,8 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
     const int c_e = e, c_m0 = m0, c_n0 = n0, c_cnt = cnt, c_seg0 = seg0;
     const int ksteps = (cnt + BK - 1) / BK;
 
+    // 64 x 128 per wave as 2 x 4 tiles of v_mfma_f32_32x32x16_bf16: with both operands read
+    // through LDS transposes the 16x16x32 shape of the row-tiled kernels measured slower here
     f32x16 acc[2][4];
 #pragma unroll
     for (int mi = 0; mi < 2; ++mi)

@@ -17,8 +17,6 @@
 namespace mi355 {
 namespace {
 
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-
 __device__ __forceinline__ int kc_off(int row, int chunk) {
   return row * BK + ((chunk ^ ((row >> 1) & 7)) << 3);
 }
