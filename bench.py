@@ -86,22 +86,25 @@ def sustained_mfma(dev):
         return None
     lib = ctypes.CDLL(path)
     lib.mi355_probe_mfma.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
-                                     ctypes.c_void_p]
+                                     ctypes.c_int, ctypes.c_void_p]
     lib.mi355_probe_mfma.restype = ctypes.c_int
-    blocks, iters = 4 * torch.cuda.get_device_properties(dev).multi_processor_count, 100000
+    blocks = 4 * torch.cuda.get_device_properties(dev).multi_processor_count
     sink = torch.zeros(1, dtype=torch.float32, device=dev)
     clocks = torch.zeros(2 * blocks, dtype=torch.int64, device=dev)
     out = {}
-    for label, rnd in (("random_bits", 1), ("constant_bits", 0)):
-        def launch():
-            rc = lib.mi355_probe_mfma(sink.data_ptr(), clocks.data_ptr(), blocks, iters, rnd,
-                                      torch.cuda.current_stream().cuda_stream)
-            assert rc == 0
-        ms = time_events(launch, 3, warmup=1)
-        flops = blocks * 8.0 * iters * 8 * 32768
-        c = clocks.view(blocks, 2).double()
-        out[label] = {"TFLOP/s": round(flops / (ms * 1e-3) / 1e12, 1),
-                      "core_clock_mhz": round(float((c[:, 0] / c[:, 1]).mean()) * 100.0, 0)}
+    # 16x16x32 is the shape of the row-tiled grouped GEMMs, 32x32x16 that of the weight gradients
+    for shape, name, iters in ((1, "16x16x32", 50000), (0, "32x32x16", 100000)):
+        out[name] = {}
+        for label, rnd in (("random_bits", 1), ("constant_bits", 0)):
+            def launch():
+                rc = lib.mi355_probe_mfma(sink.data_ptr(), clocks.data_ptr(), blocks, iters, rnd, shape,
+                                          torch.cuda.current_stream().cuda_stream)
+                assert rc == 0
+            ms = time_events(launch, 2, warmup=1)
+            flops = blocks * 8.0 * iters * 262144 * (shape + 1)
+            c = clocks.view(blocks, 2).double()
+            out[name][label] = {"TFLOP/s": round(flops / (ms * 1e-3) / 1e12, 1),
+                                "core_clock_mhz": round(float((c[:, 0] / c[:, 1]).mean()) * 100.0, 0)}
     return out
 
 
@@ -254,7 +257,8 @@ def main():
         # the same instruction with operands in registers: the rate the card holds under
         # its own power management, next to the data-sheet peak above
         roofline["sustained_mfma"] = probe
-        roofline["frac_of_sustained"] = round(ach / probe["random_bits"]["TFLOP/s"], 4)
+        shape = "32x32x16" if dominant.startswith("dw") else "16x16x32"
+        roofline["frac_of_sustained"] = round(ach / probe[shape]["random_bits"]["TFLOP/s"], 4)
 
     result = {
         "metric": "MoE layer fwd+bwd tokens/s (Qwen3-30B-A3B shape, 1 GPU)",
