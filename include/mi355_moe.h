@@ -155,7 +155,11 @@ int mi355_balance_loss_bwd(const float* scores_TE, const float* f_E,
  * Outputs (all caller-allocated, int32):
  *   counts_E      (E)     slots per expert, over all experts
  *   seg_offsets   (El+1)  first row of each local segment; [El] = total rows used
- *   seg_counts    (El)    real (unpadded) rows per local segment
+ *   seg_counts    (2*El)  [0,El): real (unpadded) rows per local segment;
+ *                 [El,2*El): the local expert indices ordered by descending row
+ *                 count, ties to the lower index -- the order in which the
+ *                 weight-gradient kernels below walk the experts, so that the
+ *                 longest contractions start first under skewed routing
  *   row_of_slot   (N)     row of slot t*K+k, or -1 when not local
  *   slot_of_row   (row_capacity) slot held by each row, -1 for padding / unused
  *   token_of_row  (row_capacity) token held by each row (slot / K), -1 for padding /
@@ -184,7 +188,8 @@ int mi355_permute_plan(const int64_t* ids_TK, int64_t T, int64_t K, int64_t E,
  * GroupedExperts.forward receives, llmtuner/models/common/moe/experts.py:152-204
  * (offsets_E = cumsum(counts), :204).  counts: (El) int32; negative counts are
  * treated as 0 and segments are clamped to the row_capacity rows that exist.
- * tile_capacity >= row_capacity/tile_m + El is always enough.
+ * seg_counts is (2*El) int32 as in mi355_permute_plan (counts, then the experts by
+ * descending count).  tile_capacity >= row_capacity/tile_m + El is always enough.
  */
 int mi355_segments_from_counts(const int32_t* counts, int64_t El, int64_t tile_m,
                                int64_t row_capacity, int32_t* seg_offsets, int32_t* seg_counts,

@@ -141,6 +141,8 @@ def test_permute_plan_is_the_stable_argsort(ops, T, K, E, align, local):
     seg_off = torch.cat([torch.zeros(1, dtype=torch.long), padded.cumsum(0)])
     assert torch.equal(plan.seg_offsets.cpu().long(), seg_off)
     assert torch.equal(plan.seg_counts.cpu().long(), lc)
+    # experts by descending count, ties to the lower index (what the weight-gradient walk reads)
+    assert plan.expert_order.cpu().tolist() == sorted(range(hi - lo), key=lambda j: (-int(lc[j]), j))
     total = int(seg_off[-1])
     # expected slot_of_row: each segment's slots then -1 padding
     exp = torch.full((plan.row_capacity,), -1, dtype=torch.long)
@@ -266,6 +268,7 @@ def _experts_case(ops, dtype, counts, D, Fd, std=0.1, seed=0):
     ref_in = [t.clone().requires_grad_() for t in (x, w1, w3, w2)]
     ref = R.grouped_experts(ref_in[0], torch.tensor(counts), *ref_in[1:])
     plan = ops.segments_from_counts(torch.tensor(counts, dtype=torch.int32, device=DEV), Rn)
+    assert plan.expert_order.cpu().tolist() == sorted(range(El), key=lambda j: (-counts[j], j))
     dx_, dw1_, dw3_, dw2_ = (t.to(DEV) for t in (x, w1, w3, w2))
     y, gate, up, h = ops.grouped_swiglu_fwd(dx_, dw1_, dw3_, dw2_, plan)
     tol = FP32_TOL if dtype == torch.float32 else BF16_TOL
@@ -300,6 +303,9 @@ def test_grouped_experts_bf16_generic_shapes(ops, counts, D, Fd):
     ((128, 128), 64, 64), ((5, 6, 4, 7), 128, 64), ((200, 0, 129, 1, 300), 256, 192),
     ((0, 0, 0), 64, 128), ((513, 77), 512, 320), ((1000,), 256, 768),
     ((200, 0, 129), 384, 768), ((131, 260), 768, 384),
+    # more experts than XCDs with a skewed, tie-laden histogram: the weight-gradient walk by
+    # descending count must still visit every expert's every tile exactly once
+    ((300, 0, 5, 700, 1, 64, 65, 0, 128, 129, 2, 5, 4, 250, 0, 90, 17, 33, 640), 384, 512),
 ])
 def test_grouped_experts_bf16_mfma(ops, counts, D, Fd):
     print(f"experts bf16 mfma {counts} D={D} F={Fd}", flush=True)

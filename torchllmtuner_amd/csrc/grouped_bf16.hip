@@ -475,7 +475,8 @@ struct WgradArgs {
   uint16_t* c;        // (El, M, N)
   const int32_t* b_src;  // row -> row of b to read (token gather), or null
   const int32_t* seg_offsets;
-  const int32_t* seg_counts;
+  const int32_t* seg_counts;  // (2 El): row counts, then the local experts by descending count
+  int El;
   int M, N;
   int m_tiles, n_tiles;
   int total;  // El * m_tiles * n_tiles
@@ -500,22 +501,47 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
   }
   const u32x4 zero = {0, 0, 0, 0};
 
-  // Persistent workgroups, same walk as the row-tiled kernels.  The K extent is one
-  // expert's rows (a handful of 64-row steps), so what surrounds the K loop matters: the
-  // first operands of the next tile are requested before the epilogue of the current one
-  // and land while it runs, segment bounds are looked up two tiles ahead, and with a
-  // gathered B operand the row indices of a K step are fetched one step before its data.
-  const int chunk = (p.total + 7) >> 3;
+  // Persistent workgroups.  A tile's cost is its expert's row count (the contraction
+  // length), which a skewed router spreads over two orders of magnitude, so tiles are not
+  // walked in expert order: experts are taken by descending row count (the plan's order,
+  // second half of seg_counts) and dealt to the eight XCDs a round at a time, and the CUs of an
+  // XCD deal that XCD's tiles round-robin among themselves -- the longest contractions
+  // start first and in parallel, and an expert's tiles still share one L2.  The K extent
+  // is short for a balanced router (a handful of 64-row steps), so what surrounds the K
+  // loop matters too: the first operands of the next tile are requested before the
+  // epilogue of the current one and land while it runs, segment bounds are looked up
+  // ahead, and with a gathered B operand the row indices of a K step are fetched one step
+  // before its data.
+  const int El = p.El;
+  const int xcd = blockIdx.x & 7;
+  const int32_t* order = p.seg_counts + El;
+  // Whole experts are dealt in rounds of eight, each round in the opposite direction of the
+  // one before (so no XCD always gets the larger expert of its round); the El % 8 smallest
+  // experts left over are cut into eight equal contiguous runs of tiles instead.
+  const int n_full = (El >> 3) * per_e;
+  const int pool = (El & 7) * per_e;
+  const int p0 = static_cast<int>(static_cast<int64_t>(pool) * xcd >> 3);
+  const int p1 = static_cast<int>(static_cast<int64_t>(pool) * (xcd + 1) >> 3);
+  const int n_x = n_full + (p1 - p0);  // tiles of this XCD
   const int stride = gridDim.x >> 3;
-  const int pid_base = (blockIdx.x & 7) * chunk;
   int within = blockIdx.x >> 3;
-  if (within >= chunk || pid_base + within >= p.total) return;
-  auto exists = [&](int w) { return w < chunk && pid_base + w < p.total; };
+  if (within >= n_x) return;
+  auto exists = [&](int w) { return w < n_x; };
+  // this XCD's w-th tile (w clamped to an existing tile) as rank * per_e + tile in expert
+  auto flat_of = [&](int w) -> int {
+    w = exists(w) ? w : within;
+    if (w >= n_full) return 8 * n_full + p0 + (w - n_full);
+    const int round = w / per_e;
+    return (round * 8 + ((round & 1) ? 7 - xcd : xcd)) * per_e + (w - round * per_e);
+  };
+  // (clamped: an order array the caller never filled must not turn into a wild address)
+  auto expert_at = [&](int flat) -> int { return min(max(order[flat / per_e], 0), El - 1); };
+  auto expert_of = [&](int w) -> int { return expert_at(flat_of(w)); };
+  auto tile_in_expert = [&](int w) -> int { return flat_of(w) % per_e; };
 
   // state of the tile whose operands are being fetched
-  int pid = pid_base + within;
-  int e = pid / per_e;
-  int m0 = ((pid % per_e) / p.n_tiles) * WBM, n0 = ((pid % per_e) % p.n_tiles) * WBN;
+  int e = expert_of(within);
+  int m0 = (tile_in_expert(within) / p.n_tiles) * WBM, n0 = (tile_in_expert(within) % p.n_tiles) * WBN;
   int seg0 = p.seg_offsets[e], cnt = p.seg_counts[e];
   const uint16_t* a_base;
   const uint16_t* b_base;
@@ -549,20 +575,18 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) bidx[i] = row_index(seg0, cnt, 1, i);
   }
-  // segment of the next tile (the one after it is looked up inside the loop)
-  int nseg0, ncnt;
-  {
-    const int ne = (pid_base + (exists(within + stride) ? within + stride : within)) / per_e;
-    nseg0 = p.seg_offsets[ne];
-    ncnt = p.seg_counts[ne];
-  }
+  // expert and segment of the next tile, expert of the one after it (its segment is
+  // looked up inside the loop, the expert after that too)
+  int ne = expert_of(within + stride);
+  int nseg0 = p.seg_offsets[ne], ncnt = p.seg_counts[ne];
+  int e2 = expert_of(within + 2 * stride);
 
   for (;;) {
     const bool more = exists(within + stride);
-    const int npid = pid_base + within + stride;
-    // two tiles ahead: segment bounds, used one tile later
-    const int e2 = (pid_base + (exists(within + 2 * stride) ? within + 2 * stride : within)) / per_e;
+    const int nw = within + stride;
+    // two tiles ahead: segment bounds, used one tile later; three ahead: the expert
     const int n2seg0 = p.seg_offsets[e2], n2cnt = p.seg_counts[e2];
+    const int e3 = expert_of(within + 3 * stride);
     // next tile: B rows of its first K step (its bounds were looked up a tile ago)
     int nidx[4];
     if (ncnt > 0) {
@@ -633,9 +657,10 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
 
     // switch the fetch state to the next tile and request its first K step
     if (more) {
-      e = npid / per_e;
-      m0 = ((npid % per_e) / p.n_tiles) * WBM;
-      n0 = ((npid % per_e) % p.n_tiles) * WBN;
+      e = ne;
+      const int nt = tile_in_expert(nw);
+      m0 = (nt / p.n_tiles) * WBM;
+      n0 = (nt % p.n_tiles) * WBN;
       seg0 = nseg0;
       cnt = ncnt;
       set_bases();
@@ -673,6 +698,8 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
     phase_barrier();
     if (!more) break;
     within += stride;
+    ne = e2;
+    e2 = e3;
     nseg0 = n2seg0;
     ncnt = n2cnt;
   }
@@ -802,7 +829,7 @@ int bf16_grouped_bwd(const void* dy, const void* rows, const int32_t* token_of_r
   auto wgrad = [&](const void* A, const void* B, const int32_t* b_src, void* C, int64_t M, int64_t N, const char* what) {
     WgradArgs w{};
     w.a = (const uint16_t*)A; w.b = (const uint16_t*)B; w.c = (uint16_t*)C; w.b_src = b_src;
-    w.seg_offsets = seg_offsets; w.seg_counts = seg_counts; w.M = (int)M; w.N = (int)N;
+    w.seg_offsets = seg_offsets; w.seg_counts = seg_counts; w.El = (int)El; w.M = (int)M; w.N = (int)N;
     w.m_tiles = (int)((M + WBM - 1) / WBM); w.n_tiles = (int)((N + WBN - 1) / WBN);
     w.total = (int)(El * w.m_tiles * w.n_tiles);
     const dim3 grid(std::min(round8(w.total), resident_blocks()));

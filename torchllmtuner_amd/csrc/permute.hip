@@ -122,6 +122,17 @@ __global__ __launch_bounds__(1024) void plan_scan_kernel(
     *num_tiles = toff < tile_capacity ? toff : tile_capacity;
   }
   __syncthreads();
+  // local experts by descending row count (ties to the lower index): the order in which the
+  // weight-gradient kernels start their tiles, longest contraction first
+  for (int j = tid; j < El; j += blockDim.x) {
+    const int c = cnt_sh[lo + j];
+    int rank = 0;
+    for (int o = 0; o < El; ++o) {
+      const int co = cnt_sh[lo + o];
+      rank += (co > c || (co == c && o < j)) ? 1 : 0;
+    }
+    seg_counts[El + rank] = j;
+  }
   for (int j = tid; j <= El; j += blockDim.x) seg_offsets[j] = seg_off_sh[j];
   for (int j = tid; j < El; j += blockDim.x) {
     const int c = cnt_sh[lo + j];
@@ -164,6 +175,17 @@ __global__ __launch_bounds__(256) void segments_from_counts_kernel(
     *num_tiles = toff < tile_capacity ? toff : tile_capacity;
   }
   __syncthreads();
+  // local experts by descending row count (ties to the lower index): the order in which the
+  // weight-gradient kernels start their tiles, longest contraction first
+  for (int j = tid; j < El; j += blockDim.x) {
+    const int c = cnt_sh[j];
+    int rank = 0;
+    for (int o = 0; o < El; ++o) {
+      const int co = cnt_sh[o];
+      rank += (co > c || (co == c && o < j)) ? 1 : 0;
+    }
+    seg_counts[El + rank] = j;
+  }
   for (int j = tid; j <= El; j += blockDim.x) seg_offsets[j] = seg_off_sh[j];
   for (int j = tid; j < El; j += blockDim.x) {
     const int c = cnt_sh[j];

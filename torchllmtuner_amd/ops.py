@@ -196,6 +196,9 @@ class PermutePlan:
     tile_expert: torch.Tensor
     tile_row0: torch.Tensor
     num_tiles: torch.Tensor
+    # local experts by descending row count; lives right behind seg_counts in memory, where
+    # the weight-gradient kernels look for it
+    expert_order: torch.Tensor | None = None
 
     @property
     def num_local_experts(self) -> int:
@@ -224,11 +227,12 @@ def permute_plan(ids_TK, num_experts, local_lo=0, local_hi=None, align=1) -> Per
     lib = _lib.load()
     i32 = dict(dtype=torch.int32, device=dev)
     # one allocation for the small arrays, one for the per-slot / per-row ones
-    small = torch.empty(E + (El + 1) + El + 2 * tile_cap + 1, **i32)
+    small = torch.empty(E + (El + 1) + 2 * El + 2 * tile_cap + 1, **i32)
     o = 0
     counts_E = small[o:o + E]; o += E
     seg_offsets = small[o:o + El + 1]; o += El + 1
-    seg_counts = small[o:o + El]; o += El
+    # the library writes 2*El ints here: the counts, then the experts by descending count
+    seg_counts = small[o:o + El]; expert_order = small[o + El:o + 2 * El]; o += 2 * El
     tile_expert = small[o:o + tile_cap]; o += tile_cap
     tile_row0 = small[o:o + tile_cap]; o += tile_cap
     num_tiles = small[o:o + 1]
@@ -244,7 +248,8 @@ def permute_plan(ids_TK, num_experts, local_lo=0, local_hi=None, align=1) -> Per
         )
     _lib.check(rc, "permute_plan")
     return PermutePlan(T, K, E, lo, hi, align, tm, row_cap, tile_cap, counts_E, seg_offsets,
-                       seg_counts, row_of_slot, slot_of_row, token_of_row, tile_expert, tile_row0, num_tiles)
+                       seg_counts, row_of_slot, slot_of_row, token_of_row, tile_expert, tile_row0, num_tiles,
+                       expert_order)
 
 
 def segments_from_counts(counts_e, total_rows: int) -> PermutePlan:
@@ -255,10 +260,10 @@ def segments_from_counts(counts_e, total_rows: int) -> PermutePlan:
     tm = tile_m()
     tile_cap = total_rows // tm + El + 1
     i32 = dict(dtype=torch.int32, device=dev)
-    small = torch.empty((El + 1) + El + 2 * tile_cap + 1, **i32)
+    small = torch.empty((El + 1) + 2 * El + 2 * tile_cap + 1, **i32)
     o = 0
     seg_offsets = small[o:o + El + 1]; o += El + 1
-    seg_counts = small[o:o + El]; o += El
+    seg_counts = small[o:o + El]; expert_order = small[o + El:o + 2 * El]; o += 2 * El
     tile_expert = small[o:o + tile_cap]; o += tile_cap
     tile_row0 = small[o:o + tile_cap]; o += tile_cap
     num_tiles = small[o:o + 1]
@@ -269,7 +274,7 @@ def segments_from_counts(counts_e, total_rows: int) -> PermutePlan:
         )
     _lib.check(rc, "segments_from_counts")
     return PermutePlan(0, 1, El, 0, El, 1, tm, total_rows, tile_cap, None, seg_offsets, seg_counts,
-                       None, None, None, tile_expert, tile_row0, num_tiles)
+                       None, None, None, tile_expert, tile_row0, num_tiles, expert_order)
 
 
 # ------------------------------------------------------------------ row movers
