@@ -260,6 +260,17 @@ def main():
         shape = "32x32x16" if dominant.startswith("dw") else "16x16x32"
         roofline["frac_of_sustained"] = round(ach / probe[shape]["random_bits"]["TFLOP/s"], 4)
 
+    if not args.no_probe:
+        # The vendor library's dense GEMM with the dominant kernel's flops (all rows against
+        # ONE expert's gate and up weights, random values, no SwiGLU, no routing): what a
+        # tuned kernel holds on this card at this size, next to the data-sheet peak.
+        a = torch.randn(R_rows, D, device=dev).bfloat16()
+        b = torch.randn(2 * F, D, device=dev).bfloat16()
+        ms = time_events(lambda: torch.mm(a, b.t()), 10, warmup=3)
+        roofline["vendor_dense_gemm"] = {"shape_mnk": [R_rows, 2 * F, D], "ms": round(ms, 4),
+                                         "TFLOP/s": round(2.0 * R_rows * 2 * F * D / (ms * 1e-3) / 1e12, 1)}
+        del a, b
+
     result = {
         "metric": "MoE layer fwd+bwd tokens/s (Qwen3-30B-A3B shape, 1 GPU)",
         "value": round(tokens_per_s, 1),
