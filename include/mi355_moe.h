@@ -101,6 +101,47 @@ int mi355_router_select_fwd(const float* logits_TE, const float* expert_bias,
                             int num_limited, int select_mode, void* stream);
 
 /*
+ * The same selection for a quantile-balanced router in training
+ * (QuantileBalancedTopKRouter._select_experts, routing.py:399-430: one biased
+ * top-(K+1), sorted): plain top-k over scores + expert_bias, and additionally
+ * cutoff_T[t] = the (K+1)-th largest biased score of token t, the value the required
+ * biases of mi355_quantile_observe are measured against.  Needs K < E.
+ */
+int mi355_router_select_cutoff_fwd(const float* logits_TE, const float* expert_bias,
+                                   float* weights_TK, int64_t* ids_TK, float* scores_TE,
+                                   float* cutoff_T, int64_t T, int64_t E, int64_t K,
+                                   int score_func, int route_norm, float route_scale,
+                                   void* stream);
+
+/*
+ * Required-bias histogram of quantile-balanced routing, _observe_quantile_histogram,
+ * routing.py:433-461: for every token t that is not padding and every expert e,
+ *   bin = clamp(floor((cutoff_T[t] - scores_TE[t][e] - (min(bias) - 1)) / width), 0, B-1),
+ *   width = (max(bias) - min(bias) + 2) / B,   histogram_EB[e][bin] += 1.
+ * histogram_EB: (E,B) int64, accumulated into (the caller zeroes it once per
+ * optimizer step).  padding_mask_T: (T) bytes, non-zero = padding, or NULL.
+ * The fp32 operations are the reference's in its order; integer atomics make the
+ * result independent of scheduling.
+ */
+int mi355_quantile_observe(const float* scores_TE, const float* cutoff_T,
+                           const float* expert_bias_E, const uint8_t* padding_mask_T,
+                           int64_t* histogram_EB, int64_t T, int64_t E, int64_t B,
+                           void* stream);
+
+/*
+ * Next mean-centred expert bias from the histogram,
+ * QuantileBalancer.estimate_expert_bias, routing.py:557-610: per expert the K/E
+ * quantile of its required-bias distribution (target rank ceil(count*K/E), linear
+ * interpolation inside the crossing bin with an integral numerator), experts without
+ * observations held at their current position, result minus its mean, times the bin
+ * width.  An all-zero histogram returns expert_bias_E unchanged, bit for bit.
+ * next_bias_E may not alias expert_bias_E.
+ */
+int mi355_quantile_estimate(const int64_t* histogram_EB, const float* expert_bias_E,
+                            float* next_bias_E, int64_t E, int64_t K, int64_t B,
+                            void* stream);
+
+/*
  * dlogits_TE from dweights_TK (and, optionally, a dense gradient dscores_TE on the
  * full score map, e.g. from an auxiliary loss; NULL = none): the backward of the
  * gather / norm / scale / score chain that autograd derives for routing.py:270-315.

@@ -300,6 +300,65 @@ def balance_loss(scores_TE, routing_map_TE, padding_mask_T=None):
     return (f_E * p_E).sum()
 
 
+def select_top_k_plus_one(scores_TE, expert_bias_E, top_k):
+    """Training-time selection of the quantile-balanced router
+    (llmtuner/models/common/moe/routing.py:411-430): one sorted top-(K+1) over the biased
+    scores; the first K ids route, the (K+1)-th biased score is the cutoff.  Ties go to the
+    lower expert id (stable descending sort; ``torch.topk`` leaves them unspecified).
+    Returns ``(ids_TK int64, cutoff_T1 fp32)``."""
+    biased_TE = scores_TE + expert_bias_E
+    order = torch.argsort(biased_TE, dim=-1, descending=True, stable=True)
+    cutoff_T1 = biased_TE.gather(-1, order[:, top_k:top_k + 1])
+    return order[:, :top_k].contiguous(), cutoff_T1
+
+
+def quantile_observe(histogram_EB, scores_TE, cutoff_T1, expert_bias_E, padding_mask_T=None):
+    """``_observe_quantile_histogram`` (routing.py:433-461), in place on the int64
+    histogram: required bias ``cutoff - score`` of every valid (token, expert) pair, binned
+    uniformly over ``[min(bias) - 1, max(bias) + 1]``; fp32 operations in the reference's
+    order, counted pair by pair."""
+    if padding_mask_T is not None:
+        keep = ~padding_mask_T
+        scores_TE, cutoff_T1 = scores_TE[keep], cutoff_T1[keep]
+    num_bins = histogram_EB.shape[1]
+    lower = expert_bias_E.min() - 1.0
+    width = (expert_bias_E.max() - expert_bias_E.min() + 2.0) / num_bins
+    bins_TE = torch.floor((cutoff_T1 - scores_TE - lower) / width).to(torch.int64).clamp(0, num_bins - 1)
+    for e in range(histogram_EB.shape[0]):
+        histogram_EB[e] += torch.bincount(bins_TE[:, e], minlength=num_bins)
+
+
+def quantile_estimate(histogram_EB, expert_bias_E, top_k):
+    """``QuantileBalancer.estimate_expert_bias`` (routing.py:557-610): the ``K/E`` quantile
+    of each expert's histogram (target rank ``ceil(count*K/E)``; position = crossing bin +
+    ``(count*K - before*E) / E / in_bin``, the numerator integral), experts without
+    observations held at their current position, then mean-centred and scaled by the bin
+    width.  No observation at all returns a copy of the bias."""
+    E, B = histogram_EB.shape
+    counts_E = histogram_EB.sum(dim=-1)
+    if not bool(counts_E.any()):
+        return expert_bias_E.clone()
+    width = (expert_bias_E.max() - expert_bias_E.min() + 2.0) / B
+    pos_E = torch.empty(E, dtype=torch.float32)
+    for e in range(E):
+        count = int(counts_E[e])
+        if count == 0:
+            pos_E[e] = (expert_bias_E[e] - (expert_bias_E.min() - 1.0)) / width
+            continue
+        numerator = count * top_k
+        rank = -(-numerator // E)
+        running = 0
+        for b in range(B):
+            in_bin = int(histogram_EB[e, b])
+            if running + in_bin >= rank:
+                break
+            running += in_bin
+        residual = torch.tensor(numerator - running * E, dtype=torch.int64)
+        fraction = residual.float() / E / torch.tensor(float(in_bin)).clamp(min=1.0)
+        pos_E[e] = torch.tensor(float(b)) + fraction
+    return ((pos_E - pos_E.mean()) * width).to(expert_bias_E.dtype)
+
+
 def shared_expert(x_TD, gate_w_FD, up_w_FD, down_w_DF):
     """The HF dense MLP reused as the shared expert (block_conversion.py:278-291)."""
     return F.linear(F.silu(F.linear(x_TD, gate_w_FD)) * F.linear(x_TD, up_w_FD), down_w_DF)

@@ -433,3 +433,89 @@ def test_balance_loss_matches_the_paper_formula_and_invariants():
     fE = counts / counts.sum() * E
     want = (fE[None, :] - (s / S * fE).sum(-1, keepdim=True)) / S
     torch.testing.assert_close(sg.grad, want, rtol=1e-5, atol=1e-6)
+
+
+# ---------------------------------------------------------------- quantile-balanced routing
+def test_quantile_worked_example_bins_and_estimate():
+    """tests/unit_tests/cpu/models/test_moe_routing.py:233-257: E=4, K=2, 10 bins, zero bias,
+    every token scored [0.92, 0.68, 0.31, 0.07] -> cutoff 0.31, required biases in bins
+    1, 3, 5, 6, next bias [-0.55, -0.15, 0.25, 0.45]."""
+    scores = torch.tensor([0.92, 0.68, 0.31, 0.07]).expand(4, -1)
+    bias = torch.zeros(4)
+    ids, cutoff = R.select_top_k_plus_one(scores, bias, 2)
+    assert torch.equal(ids, torch.tensor([[0, 1]] * 4))
+    assert torch.equal(cutoff, torch.full((4, 1), 0.31))
+    hist = torch.zeros(4, 10, dtype=torch.int64)
+    R.quantile_observe(hist, scores, cutoff, bias)
+    assert hist.sum(dim=-1).tolist() == [4, 4, 4, 4]
+    assert hist.nonzero().tolist() == [[0, 1], [1, 3], [2, 5], [3, 6]]
+    torch.testing.assert_close(R.quantile_estimate(hist, bias, 2), torch.tensor([-0.55, -0.15, 0.25, 0.45]))
+
+
+def test_quantile_histogram_counts_past_int32_and_fractional_large_counts():
+    # test_moe_routing.py:357-367
+    hist = torch.zeros(2, 4, dtype=torch.int64)
+    hist[:, 2] = torch.iinfo(torch.int32).max
+    R.quantile_observe(hist, torch.full((1, 2), 0.5), torch.full((1, 1), 0.5), torch.zeros(2))
+    assert hist[:, 2].tolist() == [2147483648, 2147483648]
+    # test_moe_routing.py:583-592: float32 cannot hold the half-token target, the integral
+    # numerator can
+    hist = torch.tensor([[8388609, 1, 0, 8388609], [8388609, 0, 1, 8388608]], dtype=torch.int64)
+    got = R.quantile_estimate(hist, torch.zeros(2), 1)
+    assert torch.equal(got, torch.tensor([0.125, -0.125]))
+
+
+def test_quantile_empty_window_returns_the_bias_bit_for_bit():
+    # test_moe_routing.py:430-441
+    original = torch.tensor([-0.31, -0.12, 0.17, 0.26])
+    current = original.clone()
+    for _ in range(20):
+        current = R.quantile_estimate(torch.zeros(4, 32, dtype=torch.int64), current, 2)
+    assert torch.equal(current, original)
+
+
+def test_quantile_estimate_is_mean_centred_and_pushes_toward_balance():
+    # test_moe_routing.py:260-298
+    g = torch.Generator().manual_seed(0)
+    scores = torch.sigmoid(torch.randn(16, 4, generator=g))
+    bias = torch.zeros(4)
+    _, cutoff = R.select_top_k_plus_one(scores, bias, 2)
+    hist = torch.zeros(4, 32, dtype=torch.int64)
+    R.quantile_observe(hist, scores, cutoff, bias)
+    assert abs(float(R.quantile_estimate(hist, bias, 2).sum())) < 1e-6
+    # expert 0 wins every token: it must lose bias, an idle one must gain
+    logits = torch.zeros(32, 4)
+    logits[:, 0] = 4.0 * torch.randn(32, generator=g).abs() + 1.0
+    logits[:, 1:] = 0.01 * torch.randn(32, 3, generator=g)
+    scores = torch.sigmoid(logits)
+    ids, cutoff = R.select_top_k_plus_one(scores, bias, 2)
+    assert (ids[:, 0] == 0).all()
+    hist = torch.zeros(4, 100, dtype=torch.int64)
+    R.quantile_observe(hist, scores, cutoff, bias)
+    nxt = R.quantile_estimate(hist, bias, 2)
+    assert float(nxt[0]) < 0 and float(nxt[1:].max()) > 0
+
+
+def test_quantile_observe_filters_padding_and_matches_pairwise_brute_force():
+    g = torch.Generator().manual_seed(5)
+    T, E, B, K = 37, 6, 17, 2
+    scores = torch.sigmoid(torch.randn(T, E, generator=g))
+    bias = torch.rand(E, generator=g) * 0.4 - 0.2
+    pad = torch.rand(T, generator=g) < 0.3
+    _, cutoff = R.select_top_k_plus_one(scores, bias, K)
+    hist = torch.zeros(E, B, dtype=torch.int64)
+    R.quantile_observe(hist, scores, cutoff, bias, padding_mask_T=pad)
+    assert int(hist.sum()) == int((~pad).sum()) * E  # test_moe_routing.py:576
+    lower = float(bias.min()) - 1.0
+    width = (float(bias.max()) - float(bias.min()) + 2.0) / B
+    want = torch.zeros_like(hist)
+    for t in range(T):
+        if pad[t]:
+            continue
+        for e in range(E):
+            req = float(cutoff[t, 0]) - float(scores[t, e])
+            want[e, min(max(int((req - lower) // width), 0), B - 1)] += 1
+    # the double-precision brute force may put a pair that sits on a bin edge next door
+    assert int((hist - want).abs().sum()) <= 2
+    # the cutoff is the (K+1)-th largest biased score
+    assert torch.equal(cutoff[:, 0], (scores + bias).sort(dim=-1, descending=True).values[:, K])

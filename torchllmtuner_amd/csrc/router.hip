@@ -71,8 +71,8 @@ template <int VPL>
 __global__ __launch_bounds__(256) void select_fwd_kernel(
     const float* __restrict__ logits, const float* __restrict__ expert_bias,
     float* __restrict__ weights, int64_t* __restrict__ ids, float* __restrict__ scores_out,
-    int T, int E, int K, int score_func, int route_norm, float route_scale, int num_groups,
-    int num_limited, int mode) {
+    float* __restrict__ cutoff_out, int T, int E, int K, int score_func, int route_norm,
+    float route_scale, int num_groups, int num_limited, int mode) {
   const int lane = threadIdx.x & 63;
   const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= T) return;
@@ -158,6 +158,18 @@ __global__ __launch_bounds__(256) void select_fwd_kernel(
       }
       sv = __shfl(sv, owner, kWave);
       if (lane == k) { my_w = sv; my_id = bi; }
+    }
+    if (cutoff_out) {
+      // the best choice score left after the K winners: the (K+1)-th of a sorted top-(K+1)
+      float bv = -INFINITY;
+      int bi = 0x7fffffff;
+#pragma unroll
+      for (int j = 0; j < VPL; ++j) {
+        if ((taken >> j) & 1u) continue;
+        if (bi == 0x7fffffff || c[j] > bv) { bv = c[j]; bi = lane + j * kWave; }
+      }
+      wave_argmax(bv, bi);
+      if (lane == 0) cutoff_out[t] = bv;
     }
   } else {
     // fixed: (t + k) % E ; balanced: (t*K + k) % E ; lane k owns slot k (K <= 64)
@@ -394,10 +406,30 @@ extern "C" int mi355_router_select_fwd(const float* logits, const float* expert_
   MI355_REQUIRE(logits && weights && ids, "router_select_fwd: null pointer");
   const dim3 grid((unsigned)((T + 3) / 4));
   DISPATCH_VPL(E, hipLaunchKernelGGL(select_fwd_kernel<VPL>, grid, dim3(256), 0, as_stream(stream),
-                                     logits, expert_bias, weights, ids, scores_TE, (int)T, (int)E,
-                                     (int)K, score_func, route_norm, route_scale, num_groups,
-                                     num_limited, select_mode));
+                                     logits, expert_bias, weights, ids, scores_TE,
+                                     static_cast<float*>(nullptr), (int)T, (int)E, (int)K, score_func,
+                                     route_norm, route_scale, num_groups, num_limited, select_mode));
   return check_launch("router_select_fwd");
+}
+
+extern "C" int mi355_router_select_cutoff_fwd(const float* logits, const float* expert_bias,
+                                              float* weights, int64_t* ids, float* scores_TE,
+                                              float* cutoff_T, int64_t T, int64_t E, int64_t K,
+                                              int score_func, int route_norm, float route_scale,
+                                              void* stream) {
+  if (int rc = check_router_args(T, E, K)) return rc;
+  MI355_REQUIRE(score_func >= 0 && score_func <= 2, "router_select_cutoff_fwd: unknown score_func %d", score_func);
+  MI355_REQUIRE(K <= 64, "router_select_cutoff_fwd: top_k > 64 unsupported");
+  MI355_REQUIRE(K < E, "router_select_cutoff_fwd: top_k (%lld) must leave a (K+1)-th expert of %lld",
+                (long long)K, (long long)E);
+  if (T == 0) return MI355_OK;
+  MI355_REQUIRE(logits && weights && ids && cutoff_T, "router_select_cutoff_fwd: null pointer");
+  const dim3 grid((unsigned)((T + 3) / 4));
+  DISPATCH_VPL(E, hipLaunchKernelGGL(select_fwd_kernel<VPL>, grid, dim3(256), 0, as_stream(stream),
+                                     logits, expert_bias, weights, ids, scores_TE, cutoff_T, (int)T,
+                                     (int)E, (int)K, score_func, route_norm, route_scale, 0, 0,
+                                     MI355_SELECT_TOPK));
+  return check_launch("router_select_cutoff_fwd");
 }
 
 extern "C" int mi355_router_select_bwd(const float* logits, const int64_t* ids,

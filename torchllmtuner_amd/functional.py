@@ -82,6 +82,38 @@ class RouteSelectFunction(torch.autograd.Function):
         return (dlogits,) + (None,) * 9
 
 
+class RouteSelectCutoffFunction(torch.autograd.Function):
+    """The same selection for a quantile-balanced router in training: also returns the
+    dense score map and the (K+1)-th biased score of every token (not differentiable;
+    it only feeds the required-bias histogram).
+
+    Returns ``(weights_TK, ids_TK, scores_TE, cutoff_T)``.
+    """
+
+    @staticmethod
+    def forward(ctx, logits_TE, expert_bias_E, top_k, score_func, route_norm, route_scale):
+        weights, ids, scores, cutoff = ops.router_select_cutoff_fwd(
+            logits_TE, expert_bias_E, top_k, score_func, route_norm, route_scale
+        )
+        ctx.save_for_backward(logits_TE, ids)
+        ctx.cfg = (score_func, route_norm, route_scale)
+        ctx.set_materialize_grads(False)  # no dense zero gradient for an unused score map
+        ctx.mark_non_differentiable(ids, cutoff)
+        return weights, ids, scores, cutoff
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, dweights, _dids, dscores, _dcutoff):
+        logits, ids = ctx.saved_tensors
+        score_func, route_norm, route_scale = ctx.cfg
+        dlogits = None
+        if ctx.needs_input_grad[0]:
+            dlogits = ops.router_select_bwd(
+                logits, ids, dweights, dscores, score_func, route_norm, route_scale, ops.SELECT_TOPK
+            )
+        return (dlogits,) + (None,) * 5
+
+
 class PermuteRowsFunction(torch.autograd.Function):
     """rows[r] = x[token of row r]; backward sums the K row gradients per token."""
 
@@ -174,6 +206,10 @@ def route_select(logits_TE, expert_bias_E, top_k, score_func, route_norm, route_
         logits_TE, expert_bias_E, top_k, score_func, route_norm, route_scale,
         num_groups or 0, num_limited or 0, mode, want_scores,
     )
+
+
+def route_select_cutoff(logits_TE, expert_bias_E, top_k, score_func, route_norm, route_scale):
+    return RouteSelectCutoffFunction.apply(logits_TE, expert_bias_E, top_k, score_func, route_norm, route_scale)
 
 
 def permute_rows(x_TD, plan):

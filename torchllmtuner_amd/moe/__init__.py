@@ -2,6 +2,13 @@
 
 from .activation import SwiGLU
 from .auxiliary_loss import AuxLoss, MicrobatchWiseLoadBalanceLoss
+from .bias_update import (
+    collect_moe_layers,
+    register_moe_balancing_hook,
+    reset_routing_statistics,
+    update_expert_bias,
+    update_quantile_expert_bias,
+)
 from .convert import (
     hf_expert_state_to_native,
     moe_from_packed_experts,
@@ -11,7 +18,7 @@ from .convert import (
 from .experts import DenseSwiGLU, DispatchObservation, ExpertErrorCapture, GroupedExperts, RoutedExperts
 from .layer import MoE
 from .linear import RouterGateLinear
-from .routing import TokenChoiceTopKRouter
+from .routing import QuantileBalancedTopKRouter, QuantileBalancer, TokenChoiceTopKRouter
 from .token_dispatch import (
     LocalDispatchMetadata,
     LocalShareTokenDispatcher,
@@ -31,12 +38,19 @@ __all__ = [
     "MicrobatchWiseLoadBalanceLoss",
     "MoE",
     "PaddedTokenDispatcher",
+    "QuantileBalancedTopKRouter",
+    "QuantileBalancer",
     "RoutedExperts",
     "RouterGateLinear",
     "SwiGLU",
     "TokenChoiceTopKRouter",
+    "collect_moe_layers",
     "hf_expert_state_to_native",
     "moe_from_packed_experts",
     "native_ep_expert_key",
     "native_expert_state_to_hf",
+    "register_moe_balancing_hook",
+    "reset_routing_statistics",
+    "update_expert_bias",
+    "update_quantile_expert_bias",
 ]

@@ -20,7 +20,7 @@ import torch.nn as nn
 
 from .auxiliary_loss import in_checkpoint_recompute
 from .experts import RoutedExperts
-from .routing import TokenChoiceTopKRouter
+from .routing import QuantileBalancedTopKRouter, TokenChoiceTopKRouter
 
 __all__ = ["MoE", "in_checkpoint_recompute"]
 
@@ -57,6 +57,13 @@ class MoE(nn.Module):
             raise ValueError(
                 f"MoE dispatcher.top_k must match router.top_k; got {dispatcher.top_k} and {router.top_k}"
             )
+        quantile_balanced = isinstance(router, QuantileBalancedTopKRouter)
+        if quantile_balanced and load_balance_coeff is not None:
+            raise ValueError(
+                "A QuantileBalancedTopKRouter is balanced by the quantile "
+                "update, so load_balance_coeff must be None -- the sign-based "
+                "and quantile updates cannot both own expert_bias_E."
+            )
         if load_balance_coeff is not None and (
             not isinstance(load_balance_coeff, Real)
             or isinstance(load_balance_coeff, bool)
@@ -68,7 +75,8 @@ class MoE(nn.Module):
         self.router = router
         self.shared_experts = shared_experts
         self.load_balance_coeff = load_balance_coeff
-        if load_balance_coeff is not None:
+        # both balancing schemes persist the balance they reached (layer.py:169-177)
+        if load_balance_coeff is not None or quantile_balanced:
             self.register_buffer(
                 "expert_bias_E", torch.zeros(num_experts, dtype=torch.float32), persistent=True
             )
@@ -134,7 +142,9 @@ class MoE(nn.Module):
                 tokens, self.expert_bias_E, padding_mask_T=padding_mask
             )
         else:
-            topk_scores_TK, topk_expert_ids_TK = router.route(tokens, self.expert_bias_E)
+            topk_scores_TK, topk_expert_ids_TK = router.route(
+                tokens, self.expert_bias_E, padding_mask_T=padding_mask
+            )
 
         plan = self.routed_experts.token_dispatcher.plan(topk_expert_ids_TK)
         out_TD = self.routed_experts.forward_planned(tokens, topk_scores_TK, plan)

@@ -22,9 +22,10 @@ import torch.nn as nn
 
 from .. import functional as Fn
 from .. import ops
+from .auxiliary_loss import in_checkpoint_recompute
 from .linear import RouterGateLinear
 
-__all__ = ["TokenChoiceTopKRouter"]
+__all__ = ["QuantileBalancedTopKRouter", "QuantileBalancer", "TokenChoiceTopKRouter"]
 
 
 class TokenChoiceTopKRouter(nn.Module):
@@ -114,7 +115,8 @@ class TokenChoiceTopKRouter(nn.Module):
             return ops.SELECT_BALANCED
         return ops.SELECT_TOPK
 
-    def _select(self, logits_TE, expert_bias_E, want_scores):
+    def _select(self, logits_TE, expert_bias_E, want_scores, padding_mask_T=None):
+        # padding_mask_T is for subclasses that keep statistics (the quantile router)
         return Fn.route_select(
             logits_TE,
             expert_bias_E,
@@ -128,8 +130,10 @@ class TokenChoiceTopKRouter(nn.Module):
             want_scores,
         )
 
-    def route(self, x_TD: torch.Tensor, expert_bias_E: torch.Tensor | None = None):
-        """Scores and ids only: ``(topk_scores_TK fp32, topk_expert_ids_TK int64)``."""
+    def route(self, x_TD: torch.Tensor, expert_bias_E: torch.Tensor | None = None, *,
+              padding_mask_T: torch.Tensor | None = None):
+        """Scores and ids only: ``(topk_scores_TK fp32, topk_expert_ids_TK int64)``.
+        ``padding_mask_T`` only matters to routers that keep statistics."""
         logits_TE = self.gate(x_TD)
         scores_TK, ids_TK, _ = self._select(logits_TE, expert_bias_E, False)
         return scores_TK, ids_TK
@@ -153,7 +157,7 @@ class TokenChoiceTopKRouter(nn.Module):
         logits_TE = self.gate(x_TD)
         want_scores = self.training and self.aux_loss is not None
         topk_scores_TK, topk_expert_ids_TK, scores_TE = self._select(
-            logits_TE, expert_bias_E, want_scores
+            logits_TE, expert_bias_E, want_scores, padding_mask_T
         )
         # One-hot map of each token's chosen experts; (T, E) bool is index glue, not
         # arithmetic, and is built with a scatter like the reference's.
@@ -171,3 +175,116 @@ class TokenChoiceTopKRouter(nn.Module):
                 scores_TE, masked_map, carrier=topk_scores_TK, padding_mask_T=padding_mask_T
             )
         return topk_scores_TK, topk_expert_ids_TK, routing_map_TE
+
+
+class QuantileBalancer(nn.Module):
+    """Required-bias histogram of quantile-balanced routing and the bias read back from it
+    (llmtuner/models/common/moe/routing.py:491-610).
+
+    For sigmoid scores in [0, 1] the bias an expert needs to win a token lies between the
+    smallest current bias minus one and the largest plus one; every training micro-batch
+    adds ``cutoff - score`` of each (token, expert) pair to ``num_bins`` uniform bins over
+    that interval (one device kernel, int64 counters), and ``estimate_expert_bias`` reads
+    the ``top_k / num_experts`` quantile of every expert back out (one device kernel).
+    The histogram is scratch state: it follows device moves and never lands in a checkpoint.
+    """
+
+    def __init__(self, num_experts: int, top_k: int, num_bins: int) -> None:
+        super().__init__()
+        for name, value in (("num_experts", num_experts), ("top_k", top_k), ("num_bins", num_bins)):
+            if not isinstance(value, int) or isinstance(value, bool) or value < 1:
+                raise ValueError(f"{name} must be positive integer, got {value!r}")
+        if not 0 < top_k < num_experts:
+            raise ValueError(f"top_k ({top_k}) must be between zero and num_experts ({num_experts})")
+        self.num_experts = num_experts
+        self.top_k = top_k
+        self.num_bins = num_bins
+        self.register_buffer(
+            "required_bias_histogram_EB",
+            torch.zeros(num_experts, num_bins, dtype=torch.int64),
+            persistent=False,
+        )
+
+    @torch.no_grad()
+    def observe(self, scores_TE, cutoff_T1, expert_bias_E, *, padding_mask_T=None) -> None:
+        """Accumulate one micro-batch; padding tokens and checkpoint replays are skipped."""
+        if not self.training or in_checkpoint_recompute.get():
+            return
+        ops.quantile_observe(
+            self.required_bias_histogram_EB, scores_TE, cutoff_T1, expert_bias_E, padding_mask_T
+        )
+
+    @torch.no_grad()
+    def estimate_expert_bias(self, histogram_EB, expert_bias_E):
+        """The next mean-centred bias; an empty histogram returns a copy of the current one."""
+        if histogram_EB.shape != (self.num_experts, self.num_bins):
+            raise ValueError(
+                f"histogram_EB must have shape {(self.num_experts, self.num_bins)}, "
+                f"got {tuple(histogram_EB.shape)}"
+            )
+        return ops.quantile_estimate(histogram_EB, expert_bias_E, self.top_k)
+
+
+class QuantileBalancedTopKRouter(TokenChoiceTopKRouter):
+    """Top-k router balanced by a histogram-estimated quantile bias
+    (llmtuner/models/common/moe/routing.py:348-430).
+
+    A training forward takes one biased top-(K+1): the first K experts route the token,
+    the (K+1)-th biased score is the cutoff the required biases are measured against.
+    Sigmoid scores only, no group-limited routing, no debug routings -- as in the
+    reference, whose constructor takes none of those arguments.  Eval routes with the
+    plain biased top-k and observes nothing.
+    """
+
+    def __init__(
+        self,
+        num_experts: int,
+        dim: int,
+        top_k: int = 1,
+        *,
+        num_bins: int = 1000,
+        route_norm: bool = False,
+        route_scale: float = 1.0,
+        aux_loss=None,
+    ) -> None:
+        super().__init__(
+            num_experts=num_experts, dim=dim, top_k=top_k, score_func="sigmoid",
+            route_norm=route_norm, route_scale=route_scale, aux_loss=aux_loss,
+        )
+        self.quantile_balancer = QuantileBalancer(num_experts=num_experts, top_k=top_k, num_bins=num_bins)
+
+    def _require_bias(self, expert_bias_E):
+        if expert_bias_E is None:
+            raise ValueError(
+                "Quantile-balanced routing requires an expert bias; the MoE "
+                "owning this router must register expert_bias_E."
+            )
+
+    def _select_observing(self, logits_TE, expert_bias_E, padding_mask_T):
+        """Biased top-(K+1) in one kernel, histogram accumulation in a second."""
+        scores_TK, ids_TK, scores_TE, cutoff_T = Fn.route_select_cutoff(
+            logits_TE, expert_bias_E, self.top_k, self.score_func, self.route_norm, float(self.route_scale)
+        )
+        self.quantile_balancer.observe(
+            scores_TE.detach(), cutoff_T, expert_bias_E, padding_mask_T=padding_mask_T
+        )
+        return scores_TK, ids_TK, scores_TE
+
+    def forward(self, x_TD, expert_bias_E=None, *, padding_mask_T=None):
+        self._require_bias(expert_bias_E)
+        return super().forward(x_TD, expert_bias_E, padding_mask_T=padding_mask_T)
+
+    def route(self, x_TD, expert_bias_E=None, *, padding_mask_T=None):
+        self._require_bias(expert_bias_E)
+        if not self.training:
+            return super().route(x_TD, expert_bias_E)
+        if padding_mask_T is not None:
+            padding_mask_T = padding_mask_T.reshape(-1)
+        scores_TK, ids_TK, _ = self._select_observing(self.gate(x_TD), expert_bias_E, padding_mask_T)
+        return scores_TK, ids_TK
+
+    def _select(self, logits_TE, expert_bias_E, want_scores, padding_mask_T=None):
+        self._require_bias(expert_bias_E)
+        if not self.training:
+            return super()._select(logits_TE, expert_bias_E, want_scores)
+        return self._select_observing(logits_TE, expert_bias_E, padding_mask_T)

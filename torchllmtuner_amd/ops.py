@@ -119,6 +119,70 @@ def router_select_fwd(logits_TE, expert_bias_E, top_k, score_func, route_norm, r
     return weights, ids, scores
 
 
+def router_select_cutoff_fwd(logits_TE, expert_bias_E, top_k, score_func, route_norm, route_scale):
+    """Biased top-k plus the (K+1)-th biased score of every token: returns
+    ``(weights_TK, ids_TK, scores_TE, cutoff_T)``."""
+    dev = _dev(logits_TE, expert_bias_E)
+    if logits_TE.dtype != torch.float32:
+        raise TypeError("router logits must be float32")
+    logits_TE = _c(logits_TE)
+    T, E = logits_TE.shape
+    bias = None if expert_bias_E is None else _c(expert_bias_E.float())
+    weights = torch.empty(T, top_k, dtype=torch.float32, device=dev)
+    ids = torch.empty(T, top_k, dtype=torch.int64, device=dev)
+    scores = torch.empty(T, E, dtype=torch.float32, device=dev)
+    cutoff = torch.empty(T, dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_router_select_cutoff_fwd(
+            _p(logits_TE), _p(bias), _p(weights), _p(ids), _p(scores), _p(cutoff), T, E, top_k,
+            SCORE_FUNCS[score_func], int(route_norm), float(route_scale), _stream(dev),
+        )
+    _lib.check(rc, "router_select_cutoff_fwd")
+    return weights, ids, scores, cutoff
+
+
+def quantile_observe(histogram_EB, scores_TE, cutoff_T, expert_bias_E, padding_mask_T=None):
+    """Accumulates the required-bias histogram in place (int64 ``(E, B)``)."""
+    dev = _dev(histogram_EB, scores_TE, cutoff_T, expert_bias_E, padding_mask_T)
+    if histogram_EB.dtype != torch.int64 or not histogram_EB.is_contiguous():
+        raise TypeError("histogram_EB must be a contiguous int64 tensor")
+    scores_TE = _c(scores_TE.float())
+    T, E = scores_TE.shape
+    if histogram_EB.shape[0] != E or cutoff_T.numel() != T or expert_bias_E.numel() != E:
+        raise ValueError(
+            f"quantile_observe: histogram {tuple(histogram_EB.shape)}, scores {(T, E)}, "
+            f"cutoff {tuple(cutoff_T.shape)} and bias {tuple(expert_bias_E.shape)} do not agree"
+        )
+    cutoff_T = _c(cutoff_T.float().reshape(-1))
+    bias = _c(expert_bias_E.float())
+    pad = None
+    if padding_mask_T is not None:
+        if padding_mask_T.dtype != torch.bool or padding_mask_T.numel() != T:
+            raise ValueError("padding_mask_T must be a bool tensor with one entry per token")
+        pad = _c(padding_mask_T.reshape(-1)).view(torch.uint8)
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_quantile_observe(
+            _p(scores_TE), _p(cutoff_T), _p(bias), _p(pad), _p(histogram_EB), T, E,
+            histogram_EB.shape[1], _stream(dev),
+        )
+    _lib.check(rc, "quantile_observe")
+
+
+def quantile_estimate(histogram_EB, expert_bias_E, top_k):
+    """The next mean-centred expert bias (new tensor, dtype of ``expert_bias_E``)."""
+    dev = _dev(histogram_EB, expert_bias_E)
+    if histogram_EB.dtype != torch.int64:
+        raise TypeError("histogram_EB must be int64")
+    histogram_EB = _c(histogram_EB)
+    E, B = histogram_EB.shape
+    bias = _c(expert_bias_E.float())
+    out = torch.empty(E, dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_quantile_estimate(_p(histogram_EB), _p(bias), _p(out), E, top_k, B, _stream(dev))
+    _lib.check(rc, "quantile_estimate")
+    return out.to(expert_bias_E.dtype)
+
+
 def router_select_bwd(logits_TE, ids_TK, dweights_TK, dscores_TE, score_func, route_norm,
                       route_scale, mode=SELECT_TOPK):
     dev = _dev(logits_TE, ids_TK, dweights_TK, dscores_TE)
