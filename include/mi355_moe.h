@@ -135,11 +135,11 @@ int mi355_quantile_observe(const float* scores_TE, const float* cutoff_T,
  * interpolation inside the crossing bin with an integral numerator), experts without
  * observations held at their current position, result minus its mean, times the bin
  * width.  An all-zero histogram returns expert_bias_E unchanged, bit for bit.
- * next_bias_E may not alias expert_bias_E.
+ * next_bias_E may not alias expert_bias_E.  workspace: 8*E bytes.
  */
 int mi355_quantile_estimate(const int64_t* histogram_EB, const float* expert_bias_E,
-                            float* next_bias_E, int64_t E, int64_t K, int64_t B,
-                            void* stream);
+                            float* next_bias_E, void* workspace, int64_t E, int64_t K,
+                            int64_t B, void* stream);
 
 /*
  * dlogits_TE from dweights_TK (and, optionally, a dense gradient dscores_TE on the

@@ -115,6 +115,6 @@ def test_quantile_entry_points_validate_shapes_without_a_gpu():
     lib = _lib.load()
     assert lib.mi355_quantile_observe(None, None, None, None, None, 4, 0, 10, None) != 0
     assert b"quantile_observe" in lib.mi355_moe_last_error()
-    assert lib.mi355_quantile_estimate(None, None, None, 4, 4, 10, None) != 0  # K must be < E
+    assert lib.mi355_quantile_estimate(None, None, None, None, 4, 4, 10, None) != 0  # K must be < E
     assert lib.mi355_router_select_cutoff_fwd(None, None, None, None, None, None, 4, 8, 8, 0, 0, 1.0, None) != 0
     assert b"(K+1)-th" in lib.mi355_moe_last_error()

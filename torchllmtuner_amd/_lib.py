@@ -34,7 +34,7 @@ SIGNATURES = {
     "mi355_router_select_fwd": (I, [P, P, P, P, P, L, L, L, I, I, F, I, I, I, P]),
     "mi355_router_select_cutoff_fwd": (I, [P, P, P, P, P, P, L, L, L, I, I, F, P]),
     "mi355_quantile_observe": (I, [P, P, P, P, P, L, L, L, P]),
-    "mi355_quantile_estimate": (I, [P, P, P, L, L, L, P]),
+    "mi355_quantile_estimate": (I, [P, P, P, P, L, L, L, P]),
     "mi355_router_select_bwd": (I, [P, P, P, P, P, L, L, L, I, I, F, I, P]),
     "mi355_permute_plan_workspace_bytes": (L, [L, L, L]),
     "mi355_permute_plan": (I, [P, L, L, L, L, L, L, L, P, P, P, P, P, P, L, P, P, P, L, P, P]),

@@ -65,27 +65,65 @@ __global__ __launch_bounds__(256) void quantile_observe_kernel(
   }
 }
 
+// The same histogram through LDS: a workgroup owns `eg` neighbouring experts and a run of
+// tokens, counts their pairs in 32-bit LDS bins (a call adds fewer than 2^31 pairs to a
+// bin) and then adds its non-empty bins to the 64-bit histogram.  The required biases of
+// one expert cluster in a few dozen bins, so this replaces most of the global atomics,
+// which queue up on those few addresses, by LDS ones.
+__global__ __launch_bounds__(256) void quantile_observe_lds_kernel(
+    const float* __restrict__ scores, const float* __restrict__ cutoff, const float* __restrict__ bias,
+    const uint8_t* __restrict__ padding, unsigned long long* __restrict__ hist, int T, int E, int B,
+    int eg, int tokens_per_block) {
+#pragma clang fp contract(off)
+  extern __shared__ unsigned bins[];  // [eg][B]
+  __shared__ float red[512];
+  float mn, mx;
+  bias_range(bias, E, red, mn, mx);
+  const float lower = mn - 1.0f;
+  const float width = ((mx - mn) + 2.0f) / static_cast<float>(B);
+  const float top = static_cast<float>(B - 1);
+  const int e0 = blockIdx.x * eg;
+  const int ne = min(eg, E - e0);
+  const int t0 = blockIdx.y * tokens_per_block;
+  const int nt = min(tokens_per_block, T - t0);
+  for (int i = threadIdx.x; i < eg * B; i += 256) bins[i] = 0u;
+  __syncthreads();
+  for (int i = threadIdx.x; i < nt * eg; i += 256) {
+    const int t = t0 + i / eg, j = i % eg;
+    if (j >= ne || (padding && padding[t])) continue;
+    const float required = cutoff[t] - scores[static_cast<int64_t>(t) * E + e0 + j];
+    float q = floorf((required - lower) / width);
+    q = fminf(fmaxf(q, 0.0f), top);
+    atomicAdd(bins + j * B + static_cast<int>(q), 1u);
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < ne * B; i += 256) {
+    const unsigned c = bins[i];
+    if (c) atomicAdd(hist + static_cast<int64_t>(e0) * B + i, static_cast<unsigned long long>(c));
+  }
+}
+
 __device__ __forceinline__ long long wave_sum_i64(long long v) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
   return v;
 }
 
-__global__ __launch_bounds__(256) void quantile_estimate_kernel(const long long* __restrict__ hist,
+// Quantile position of every expert (in bins): one wavefront per expert.  pos_E[E] holds
+// the positions, observed_E[e] whether expert e saw anything.
+__global__ __launch_bounds__(256) void quantile_position_kernel(const long long* __restrict__ hist,
                                                                 const float* __restrict__ bias,
-                                                                float* __restrict__ out, int E, int K, int B) {
+                                                                float* __restrict__ pos, int* __restrict__ observed_E,
+                                                                int E, int K, int B) {
 #pragma clang fp contract(off)
-  extern __shared__ float pos[];  // [E]
   __shared__ float red[512];
-  __shared__ int observed;        // some expert has a non-empty histogram
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  if (threadIdx.x == 0) observed = 0;
   float mn, mx;
-  bias_range(bias, E, red, mn, mx);  // its barriers also publish `observed = 0`
+  bias_range(bias, E, red, mn, mx);
   const float width = ((mx - mn) + 2.0f) / static_cast<float>(B);
   const float lower = mn - 1.0f;
 
-  for (int e = wave; e < E; e += 4) {
+  for (int e = blockIdx.x * 4 + wave; e < E; e += gridDim.x * 4) {
     const long long* row = hist + static_cast<int64_t>(e) * B;
     long long cnt = 0;
     for (int b = lane; b < B; b += 64) cnt += row[b];
@@ -127,9 +165,26 @@ __global__ __launch_bounds__(256) void quantile_estimate_kernel(const long long*
       // an expert that saw nothing keeps its place
       if (cnt == 0) p = (bias[e] - lower) / width;
       pos[e] = p;
-      if (cnt != 0) observed = 1;
+      observed_E[e] = cnt != 0;
     }
   }
+}
+
+// Mean-centring of the positions, in one workgroup and a fixed summation order.
+__global__ __launch_bounds__(256) void quantile_centre_kernel(const float* __restrict__ pos,
+                                                              const int* __restrict__ observed_E,
+                                                              const float* __restrict__ bias,
+                                                              float* __restrict__ out, int E, int B) {
+#pragma clang fp contract(off)
+  __shared__ float red[512];
+  __shared__ int observed;  // some expert has a non-empty histogram
+  if (threadIdx.x == 0) observed = 0;
+  float mn, mx;
+  bias_range(bias, E, red, mn, mx);  // its barriers also publish `observed = 0`
+  const float width = ((mx - mn) + 2.0f) / static_cast<float>(B);
+  int any = 0;
+  for (int e = threadIdx.x; e < E; e += 256) any |= observed_E[e];
+  if (any) observed = 1;
   __syncthreads();
   if (!observed) {  // no valid token at all: the bias comes back bit for bit
     for (int e = threadIdx.x; e < E; e += 256) out[e] = bias[e];
@@ -160,23 +215,39 @@ extern "C" int mi355_quantile_observe(const float* scores_TE, const float* cutof
                 "quantile_observe: bad shape T=%lld E=%lld B=%lld", (long long)T, (long long)E, (long long)B);
   if (T == 0) return MI355_OK;
   MI355_REQUIRE(scores_TE && cutoff_T && expert_bias_E && histogram_EB, "quantile_observe: null pointer");
+  unsigned long long* hist = reinterpret_cast<unsigned long long*>(histogram_EB);
+  // experts per workgroup: what 32 KiB of LDS bins hold, at most 4 (more workgroups)
+  const int64_t eg = std::min<int64_t>(std::min<int64_t>(4, E), (32 * 1024) / (B * 4));
+  if (eg >= 1 && T >= 256) {
+    const int64_t groups = (E + eg - 1) / eg;
+    // about 256 workgroups, each with at least 256 tokens so that the LDS bins pay off
+    const int64_t chunks = std::max<int64_t>(1, std::min<int64_t>(T / 256, (256 + groups - 1) / groups));
+    const int64_t per = (T + chunks - 1) / chunks;
+    hipLaunchKernelGGL(quantile_observe_lds_kernel, dim3((unsigned)groups, (unsigned)((T + per - 1) / per)),
+                       dim3(256), (size_t)(eg * B * 4), as_stream(stream), scores_TE, cutoff_T, expert_bias_E,
+                       padding_mask_T, hist, (int)T, (int)E, (int)B, (int)eg, (int)per);
+    return check_launch("quantile_observe");
+  }
   const int64_t total = T * E;
   const unsigned blocks = (unsigned)std::min<int64_t>((total + 255) / 256, 4096);
   hipLaunchKernelGGL(quantile_observe_kernel, dim3(blocks), dim3(256), 0, as_stream(stream), scores_TE,
-                     cutoff_T, expert_bias_E, padding_mask_T,
-                     reinterpret_cast<unsigned long long*>(histogram_EB), (int)T, (int)E, (int)B);
+                     cutoff_T, expert_bias_E, padding_mask_T, hist, (int)T, (int)E, (int)B);
   return check_launch("quantile_observe");
 }
 
 extern "C" int mi355_quantile_estimate(const int64_t* histogram_EB, const float* expert_bias_E,
-                                       float* next_bias_E, int64_t E, int64_t K, int64_t B,
-                                       void* stream) {
+                                       float* next_bias_E, void* workspace, int64_t E, int64_t K,
+                                       int64_t B, void* stream) {
   MI355_REQUIRE(E >= 1 && E <= 8192 && B >= 1 && B < (1 << 24) && K >= 1 && K < E,
                 "quantile_estimate: bad shape E=%lld K=%lld B=%lld (0 < K < E <= 8192)", (long long)E,
                 (long long)K, (long long)B);
-  MI355_REQUIRE(histogram_EB && expert_bias_E && next_bias_E, "quantile_estimate: null pointer");
-  hipLaunchKernelGGL(quantile_estimate_kernel, dim3(1), dim3(256), (size_t)E * sizeof(float),
-                     as_stream(stream), reinterpret_cast<const long long*>(histogram_EB), expert_bias_E,
-                     next_bias_E, (int)E, (int)K, (int)B);
+  MI355_REQUIRE(histogram_EB && expert_bias_E && next_bias_E && workspace, "quantile_estimate: null pointer");
+  float* pos = static_cast<float*>(workspace);
+  int* observed = reinterpret_cast<int*>(pos + E);
+  hipLaunchKernelGGL(quantile_position_kernel, dim3((unsigned)((E + 3) / 4)), dim3(256), 0, as_stream(stream),
+                     reinterpret_cast<const long long*>(histogram_EB), expert_bias_E, pos, observed, (int)E,
+                     (int)K, (int)B);
+  hipLaunchKernelGGL(quantile_centre_kernel, dim3(1), dim3(256), 0, as_stream(stream), pos, observed,
+                     expert_bias_E, next_bias_E, (int)E, (int)B);
   return check_launch("quantile_estimate");
 }

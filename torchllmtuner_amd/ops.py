@@ -177,8 +177,11 @@ def quantile_estimate(histogram_EB, expert_bias_E, top_k):
     E, B = histogram_EB.shape
     bias = _c(expert_bias_E.float())
     out = torch.empty(E, dtype=torch.float32, device=dev)
+    ws = torch.empty(2 * E, dtype=torch.float32, device=dev)
     with torch.cuda.device(dev):
-        rc = _lib.load().mi355_quantile_estimate(_p(histogram_EB), _p(bias), _p(out), E, top_k, B, _stream(dev))
+        rc = _lib.load().mi355_quantile_estimate(
+            _p(histogram_EB), _p(bias), _p(out), _p(ws), E, top_k, B, _stream(dev)
+        )
     _lib.check(rc, "quantile_estimate")
     return out.to(expert_bias_E.dtype)
 
