@@ -360,6 +360,30 @@ int mi355_grouped_swiglu_stage(int stage, const void* dy, const void* rows,
                                void* dw1, void* dw3, void* dw2, int64_t El, int64_t D,
                                int64_t F, int64_t row_capacity, void* stream);
 
+/*
+ * RMS normalisation over the last axis, the `rms_norm` entry of the reference's kernel
+ * registry (llmtuner/kernel/ops/rms_norm.py:10-31; reference math
+ * llmtuner/kernel/cpu/basic.py:17-25 = torch.nn.functional.rms_norm): the norm the decoder
+ * layer applies right before the MoE block (models/qwen/qwen3/model.py:452).
+ *   r[t] = 1/sqrt(mean_d x[t][d]^2 + epsilon);   y[t][d] = (x[t][d] * r[t]) * weight[d]
+ * computed in fp32 and rounded once to `dtype` (fp32 or bf16; x, weight and y share it).
+ * rstd: optional (rows) fp32 output of r, the only thing the backward keeps.
+ */
+int mi355_rms_norm_fwd(const void* x, const void* weight, int dtype, void* y, float* rstd,
+                       int64_t rows, int64_t D, float epsilon, void* stream);
+
+/*
+ * Backward of the above (autograd-derived in the reference), g = dy * weight, xh = x * r:
+ *   dx[t][d] = r[t] * (g[t][d] - xh[t][d] * mean_d(g[t][.] * xh[t][.]))
+ *   dweight[d] = sum_t dy[t][d] * xh[t][d]      (fixed summation order, no atomics)
+ * dx or dweight may be NULL to skip it.  workspace (for dweight):
+ * mi355_rms_norm_bwd_workspace_bytes(rows, D) bytes.
+ */
+int64_t mi355_rms_norm_bwd_workspace_bytes(int64_t rows, int64_t D);
+int mi355_rms_norm_bwd(const void* dy, const void* x, const void* weight, const float* rstd,
+                       int dtype, void* dx, void* dweight, void* workspace, int64_t rows,
+                       int64_t D, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

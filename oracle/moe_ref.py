@@ -359,6 +359,18 @@ def quantile_estimate(histogram_EB, expert_bias_E, top_k):
     return ((pos_E - pos_E.mean()) * width).to(expert_bias_E.dtype)
 
 
+def rms_norm(hidden_states, weight, epsilon):
+    """The reference's CPU backend of ``rms_norm`` (llmtuner/kernel/cpu/basic.py:17-25) is
+    ``torch.nn.functional.rms_norm`` over the last axis; written out: fp32 (or wider)
+    arithmetic ``(x * rsqrt(mean(x^2) + eps)) * w`` and one rounding to the input dtype at the
+    end (checked bit for bit against the library routine in the tests, and against the
+    reference's own formula, tests/unit_tests/cpu/kernel/test_kernel_contracts.py:100-105)."""
+    wide = torch.promote_types(hidden_states.dtype, torch.float32)
+    x = hidden_states.to(wide)
+    r = torch.rsqrt(x.pow(2).mean(dim=-1, keepdim=True) + epsilon)
+    return ((x * r) * weight.to(wide)).to(hidden_states.dtype)
+
+
 def shared_expert(x_TD, gate_w_FD, up_w_FD, down_w_DF):
     """The HF dense MLP reused as the shared expert (block_conversion.py:278-291)."""
     return F.linear(F.silu(F.linear(x_TD, gate_w_FD)) * F.linear(x_TD, up_w_FD), down_w_DF)

@@ -139,3 +139,85 @@ def test_empty_permutation_retains_autograd_and_negative_ids_raise():
     assert result.shape == (0, 4) and result.requires_grad
     with pytest.raises(ValueError, match="non-negative"):
         moe_token_permute(torch.ones(2, 4, device=DEV), torch.tensor([[0], [-1]], device=DEV))
+
+
+# ------------------------------------------------------------------ rms_norm
+def test_rms_norm_is_registered_for_the_gpu_only_and_validates_metadata():
+    from torchllmtuner_amd.kernel_registry import rms_norm, rms_norm_mi355
+
+    assert get_kernel("rms_norm", "cuda") is rms_norm_mi355
+    assert set(registry._KERNEL_REGISTRY["rms_norm"]) == {"cuda"}
+    with pytest.raises(KeyError, match="not available"):
+        rms_norm(torch.ones(2, 4), torch.ones(4), 1e-6)
+    with pytest.raises(NotImplementedError, match="only implementation"):
+        rms_norm(torch.ones(2, 4), torch.ones(4), 1e-6, use_eager=True)
+    # tests/unit_tests/cpu/kernel/test_kernel_contracts.py:108-111 and validation.py:110-120
+    for epsilon in (-1.0, float("nan"), float("inf")):
+        with pytest.raises(ValueError, match="epsilon"):
+            rms_norm_mi355(torch.ones(2, 4), torch.ones(4), epsilon)
+    with pytest.raises(ValueError, match="1-D weight"):
+        rms_norm_mi355(torch.ones(2, 4), torch.ones(1, 4), 1e-6)
+    with pytest.raises(ValueError, match="must match"):
+        rms_norm_mi355(torch.ones(2, 4), torch.ones(5), 1e-6)
+    with pytest.raises(RuntimeError, match="HIP device"):
+        rms_norm_mi355(torch.ones(2, 4), torch.ones(4), 1e-6)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(2, 3, 8), (300, 2048), (5, 100), (7, 1), (7, 2), (0, 64), (4, 2, 7168), (33, 4100)])
+def test_rms_norm_matches_the_oracle_forward_and_backward(dtype, shape):
+    from oracle import moe_ref as R
+    from tests.helpers import rel_l2, rel_max
+    from torchllmtuner_amd.kernel_registry import rms_norm
+
+    print(f"rms_norm {dtype} {shape}", flush=True)
+    g = torch.Generator().manual_seed(sum(shape))
+    x = (torch.randn(*shape, generator=g) * 2).to(dtype)
+    w = (1 + 0.3 * torch.randn(shape[-1], generator=g)).to(dtype)
+    dy = torch.randn(*shape, generator=g).to(dtype)
+    xr, wr = x.clone().requires_grad_(), w.clone().requires_grad_()
+    want = R.rms_norm(xr, wr, 1e-5)
+    want.backward(dy)
+    xd, wd = x.to(DEV).requires_grad_(), w.to(DEV).requires_grad_()
+    got = rms_norm(xd, wd, 1e-5)
+    got.backward(dy.to(DEV))
+    assert got.shape == want.shape and got.dtype == dtype
+    if x.numel() == 0:
+        assert xd.grad.shape == x.shape and float(wd.grad.abs().sum()) == 0.0
+        return
+    metric, tol = (rel_max, 1e-5) if dtype == torch.float32 else (rel_l2, 2e-2)
+    assert metric(got, want) < tol
+    assert metric(wd.grad, wr.grad) < tol
+    if shape[-1] == 1:
+        # dx of a one-element row is the difference of two equal terms (eps apart): compare it
+        # on the scale of those terms, which is the scale both sides round at
+        scale = float((dy.float() * w.float()).abs().max() / x.float().abs().min())
+        assert float((xd.grad.cpu().float() - xr.grad.float()).abs().max()) < 1e-5 * max(scale, 1.0)
+    else:
+        assert metric(xd.grad, xr.grad) < tol
+    if dtype == torch.bfloat16:
+        # one rounding at the end: at most one bf16 ulp from the library routine
+        ulp = want.detach().float().abs() * 2.0 ** -7 + 1e-30
+        assert bool(((got.detach().cpu().float() - want.detach().float()).abs() <= ulp).all())
+
+
+@pytest.mark.gpu
+def test_rms_norm_formula_in_front_of_the_block():
+    """The decoder layer's `mlp(norm(hidden))` (models/qwen/qwen3/model.py:452) with both halves
+    on the device kernels: gradients flow through the block into the norm."""
+    import torchllmtuner_amd as amd
+    from torchllmtuner_amd.kernel_registry import rms_norm
+
+    E, K, D, Fd = 8, 2, 64, 96
+    block = amd.MoE(E, amd.RoutedExperts(amd.GroupedExperts(D, Fd, E), amd.LocalTokenDispatcher(E, K)),
+                    amd.TokenChoiceTopKRouter(E, D, K, score_func="softmax", route_norm=True),
+                    load_balance_coeff=None).to(DEV)
+    for p in block.parameters():
+        torch.nn.init.normal_(p, std=0.1)
+    hidden = torch.randn(2, 16, D, device=DEV, requires_grad=True)
+    weight = torch.ones(D, device=DEV, requires_grad=True)
+    out = hidden + block(rms_norm(hidden, weight, 1e-6))
+    out.square().sum().backward()
+    assert hidden.grad.shape == hidden.shape and torch.isfinite(hidden.grad).all()
+    assert weight.grad.shape == (D,) and float(weight.grad.abs().sum()) > 0

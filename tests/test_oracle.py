@@ -519,3 +519,19 @@ def test_quantile_observe_filters_padding_and_matches_pairwise_brute_force():
     assert int((hist - want).abs().sum()) <= 2
     # the cutoff is the (K+1)-th largest biased score
     assert torch.equal(cutoff[:, 0], (scores + bias).sort(dim=-1, descending=True).values[:, K])
+
+
+# ---------------------------------------------------------------- rms_norm (kernel registry)
+def test_rms_norm_matches_the_reference_formula_gradients_and_the_library_routine():
+    # tests/unit_tests/cpu/kernel/test_kernel_contracts.py:100-105
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(2, 3, 8, dtype=torch.float64, generator=g).requires_grad_()
+    w = torch.randn(8, dtype=torch.float64, generator=g).requires_grad_()
+    expected = x * torch.rsqrt(x.square().mean(-1, keepdim=True) + 1e-5) * w
+    torch.testing.assert_close(R.rms_norm(x, w, 1e-5), expected)
+    assert torch.autograd.gradcheck(lambda a, b: R.rms_norm(a, b, 1e-5), (x, w))
+    # the reference's CPU backend is torch's own routine: equal bit for bit, rounding included
+    for dtype in (torch.float32, torch.bfloat16):
+        xs = (torch.randn(64, 256, generator=g) * 3).to(dtype)
+        ws = torch.randn(256, generator=g).to(dtype)
+        assert torch.equal(R.rms_norm(xs, ws, 1e-5), F.rms_norm(xs, (256,), ws, 1e-5))

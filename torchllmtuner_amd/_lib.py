@@ -36,6 +36,9 @@ SIGNATURES = {
     "mi355_quantile_observe": (I, [P, P, P, P, P, L, L, L, P]),
     "mi355_quantile_estimate": (I, [P, P, P, P, L, L, L, P]),
     "mi355_router_select_bwd": (I, [P, P, P, P, P, L, L, L, I, I, F, I, P]),
+    "mi355_rms_norm_fwd": (I, [P, P, I, P, P, L, L, F, P]),
+    "mi355_rms_norm_bwd_workspace_bytes": (L, [L, L]),
+    "mi355_rms_norm_bwd": (I, [P, P, P, P, I, P, P, P, L, L, P]),
     "mi355_permute_plan_workspace_bytes": (L, [L, L, L]),
     "mi355_permute_plan": (I, [P, L, L, L, L, L, L, L, P, P, P, P, P, P, L, P, P, P, L, P, P]),
     "mi355_segments_from_counts": (I, [P, L, L, L, P, P, P, P, P, L, P]),

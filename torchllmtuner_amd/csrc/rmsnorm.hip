@@ -1,0 +1,263 @@
+// RMS normalisation over the last axis and its backward: the `rms_norm` entry of the
+// reference's kernel registry (llmtuner/kernel/ops/rms_norm.py:10-31; reference math
+// llmtuner/kernel/cpu/basic.py:17-25 = torch.nn.functional.rms_norm).
+//
+//   r_t = rsqrt(mean_d x[t][d]^2 + eps)      y[t][d] = round((x[t][d] * r_t) * w[d])
+//
+// with everything in fp32 and ONE rounding to the storage type at the end, which is what
+// torch's CPU routine does for bf16 inputs.  Backward, with g = dy * w and xh = x * r:
+//   dx[t][d] = r_t * (g[t][d] - xh[t][d] * mean_d(g[t][.] * xh[t][.]))
+//   dw[d]    = sum_t dy[t][d] * xh[t][d]
+// HBM-bound: one wavefront per row for y and dx (16-byte lanes, the second pass over the
+// row comes from cache); dw as per-workgroup column sums over a run of rows, combined by a
+// second kernel in a fixed order (no atomics, deterministic).
+#include <algorithm>
+#include <initializer_list>
+
+#include "common.h"
+
+namespace mi355 {
+namespace {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// N consecutive elements as floats; N = 16 bytes' worth uses one 16-byte access
+template <typename T, int N>
+struct Pack;
+template <>
+struct Pack<float, 1> {
+  static __device__ __forceinline__ void load(const float* p, float (&v)[1]) { v[0] = *p; }
+  static __device__ __forceinline__ void store(float* p, const float (&v)[1]) { *p = v[0]; }
+};
+template <>
+struct Pack<float, 4> {
+  static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
+    const float4 q = *reinterpret_cast<const float4*>(p);
+    v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+  }
+  static __device__ __forceinline__ void store(float* p, const float (&v)[4]) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  }
+};
+template <>
+struct Pack<uint16_t, 1> {
+  static __device__ __forceinline__ void load(const uint16_t* p, float (&v)[1]) { v[0] = bf16_to_f32(*p); }
+  static __device__ __forceinline__ void store(uint16_t* p, const float (&v)[1]) { *p = f32_to_bf16(v[0]); }
+};
+template <>
+struct Pack<uint16_t, 8> {
+  static __device__ __forceinline__ void load(const uint16_t* p, float (&v)[8]) {
+    const u32x4 q = *reinterpret_cast<const u32x4*>(p);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      v[2 * j] = __uint_as_float(q[j] << 16);
+      v[2 * j + 1] = __uint_as_float(q[j] & 0xffff0000u);
+    }
+  }
+  static __device__ __forceinline__ void store(uint16_t* p, const float (&v)[8]) {
+    u32x4 q;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) q[j] = pack_bf16x2(v[2 * j], v[2 * j + 1]);
+    *reinterpret_cast<u32x4*>(p) = q;
+  }
+};
+template <typename T>
+constexpr int kVec = 16 / sizeof(T);
+
+template <typename T, int N>
+__device__ __forceinline__ float row_sumsq(const T* xr, int D, int lane) {
+  float ss = 0.0f;
+  for (int i = lane * N; i < D; i += kWave * N) {
+    float v[N];
+    Pack<T, N>::load(xr + i, v);
+#pragma unroll
+    for (int j = 0; j < N; ++j) ss += v[j] * v[j];
+  }
+  return ss;
+}
+
+template <typename T, int N>
+__device__ __forceinline__ void row_scale(const T* xr, const T* w, T* yr, float r, int D, int lane) {
+  for (int i = lane * N; i < D; i += kWave * N) {
+    float v[N], g[N], o[N];
+    Pack<T, N>::load(xr + i, v);
+    Pack<T, N>::load(w + i, g);
+#pragma unroll
+    for (int j = 0; j < N; ++j) o[j] = (v[j] * r) * g[j];
+    Pack<T, N>::store(yr + i, o);
+  }
+}
+
+// vec: rows start on 16-byte boundaries (D a multiple of 16 bytes' worth, aligned bases)
+template <typename T>
+__global__ __launch_bounds__(256) void rms_fwd_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                      T* __restrict__ y, float* __restrict__ rstd, int rows,
+                                                      int D, float eps, int vec) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const T* xr = x + static_cast<int64_t>(row) * D;
+  T* yr = y + static_cast<int64_t>(row) * D;
+  const float ss = wave_sum(vec ? row_sumsq<T, kVec<T>>(xr, D, lane) : row_sumsq<T, 1>(xr, D, lane));
+  const float r = 1.0f / sqrtf(ss / static_cast<float>(D) + eps);
+  if (vec) row_scale<T, kVec<T>>(xr, w, yr, r, D, lane); else row_scale<T, 1>(xr, w, yr, r, D, lane);
+  if (lane == 0 && rstd) rstd[row] = r;
+}
+
+template <typename T, int N>
+__device__ __forceinline__ float row_dot(const T* dyr, const T* xr, const T* w, float r, int D, int lane) {
+  float dot = 0.0f;
+  for (int i = lane * N; i < D; i += kWave * N) {
+    float a[N], b[N], g[N];
+    Pack<T, N>::load(dyr + i, a);
+    Pack<T, N>::load(xr + i, b);
+    Pack<T, N>::load(w + i, g);
+#pragma unroll
+    for (int j = 0; j < N; ++j) dot += (a[j] * g[j]) * (b[j] * r);
+  }
+  return dot;
+}
+
+template <typename T, int N>
+__device__ __forceinline__ void row_dx(const T* dyr, const T* xr, const T* w, T* dxr, float r, float c, int D,
+                                       int lane) {
+  for (int i = lane * N; i < D; i += kWave * N) {
+    float a[N], b[N], g[N], o[N];
+    Pack<T, N>::load(dyr + i, a);
+    Pack<T, N>::load(xr + i, b);
+    Pack<T, N>::load(w + i, g);
+#pragma unroll
+    for (int j = 0; j < N; ++j) o[j] = r * (a[j] * g[j] - (b[j] * r) * c);
+    Pack<T, N>::store(dxr + i, o);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void rms_dx_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+                                                     const T* __restrict__ w, const float* __restrict__ rstd,
+                                                     T* __restrict__ dx, int rows, int D, int vec) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int64_t o = static_cast<int64_t>(row) * D;
+  const float r = rstd[row];
+  const float dot = vec ? row_dot<T, kVec<T>>(dy + o, x + o, w, r, D, lane) : row_dot<T, 1>(dy + o, x + o, w, r, D, lane);
+  const float c = wave_sum(dot) / static_cast<float>(D);
+  if (vec) row_dx<T, kVec<T>>(dy + o, x + o, w, dx + o, r, c, D, lane);
+  else row_dx<T, 1>(dy + o, x + o, w, dx + o, r, c, D, lane);
+}
+
+// rows per workgroup of the column sums: 64, more once that would exceed 4096 workgroups
+__host__ __device__ inline int64_t dw_rows_per_chunk(int64_t rows) {
+  const int64_t per = (rows + 4095) / 4096;
+  return per < 64 ? 64 : per;
+}
+
+// partial[chunk][d] = sum over the chunk's rows of dy * x * r
+template <typename T>
+__global__ __launch_bounds__(256) void rms_dw_partial_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+                                                             const float* __restrict__ rstd,
+                                                             float* __restrict__ partial, int rows, int D,
+                                                             int per) {
+  const int d = blockIdx.x * 256 + threadIdx.x;
+  const int r0 = blockIdx.y * per;
+  const int r1 = min(r0 + per, rows);
+  if (d >= D) return;
+  float acc = 0.0f;
+  for (int row = r0; row < r1; ++row) {
+    const int64_t o = static_cast<int64_t>(row) * D + d;
+    float a[1], b[1];
+    Pack<T, 1>::load(dy + o, a);
+    Pack<T, 1>::load(x + o, b);
+    acc += a[0] * (b[0] * rstd[row]);
+  }
+  partial[static_cast<int64_t>(blockIdx.y) * D + d] = acc;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void rms_dw_final_kernel(const float* __restrict__ partial, T* __restrict__ dw,
+                                                           int chunks, int D) {
+  const int d = blockIdx.x * 256 + threadIdx.x;
+  if (d >= D) return;
+  float acc = 0.0f;
+  for (int c = 0; c < chunks; ++c) acc += partial[static_cast<int64_t>(c) * D + d];
+  const float out[1] = {acc};
+  Pack<T, 1>::store(dw + d, out);
+}
+
+int rows_are_16_byte_aligned(int64_t D, int dtype, std::initializer_list<const void*> ptrs) {
+  const int64_t per16 = dtype == MI355_F32 ? 4 : 8;
+  if (D % per16 != 0) return 0;
+  for (const void* p : ptrs)
+    if (reinterpret_cast<uintptr_t>(p) % 16 != 0) return 0;
+  return 1;
+}
+
+int check_shape(const char* what, int64_t rows, int64_t D, int dtype) {
+  MI355_REQUIRE(dtype == MI355_F32 || dtype == MI355_BF16, "%s: dtype %d is neither fp32 nor bf16", what, dtype);
+  MI355_REQUIRE(rows >= 0 && rows < (1ll << 31) && D >= 1 && D < (1ll << 31), "%s: bad shape rows=%lld D=%lld", what,
+                (long long)rows, (long long)D);
+  return MI355_OK;
+}
+
+}  // namespace
+}  // namespace mi355
+
+using namespace mi355;
+
+extern "C" int mi355_rms_norm_fwd(const void* x, const void* weight, int dtype, void* y, float* rstd,
+                                  int64_t rows, int64_t D, float epsilon, void* stream) {
+  if (int rc = check_shape("rms_norm_fwd", rows, D, dtype)) return rc;
+  MI355_REQUIRE(epsilon >= 0.0f && epsilon < INFINITY, "rms_norm_fwd: epsilon must be finite and nonnegative");
+  if (rows == 0) return MI355_OK;
+  MI355_REQUIRE(x && weight && y, "rms_norm_fwd: null pointer");
+  const dim3 grid((unsigned)((rows + 3) / 4));
+  const int vec = rows_are_16_byte_aligned(D, dtype, {x, weight, y});
+  if (dtype == MI355_F32)
+    hipLaunchKernelGGL(rms_fwd_kernel<float>, grid, dim3(256), 0, as_stream(stream), static_cast<const float*>(x),
+                       static_cast<const float*>(weight), static_cast<float*>(y), rstd, (int)rows, (int)D, epsilon,
+                       vec);
+  else
+    hipLaunchKernelGGL(rms_fwd_kernel<uint16_t>, grid, dim3(256), 0, as_stream(stream),
+                       static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(weight),
+                       static_cast<uint16_t*>(y), rstd, (int)rows, (int)D, epsilon, vec);
+  return check_launch("rms_norm_fwd");
+}
+
+extern "C" int64_t mi355_rms_norm_bwd_workspace_bytes(int64_t rows, int64_t D) {
+  if (rows < 0 || D < 1) return 0;
+  const int64_t per = dw_rows_per_chunk(rows);
+  return ((rows + per - 1) / per) * D * 4;
+}
+
+extern "C" int mi355_rms_norm_bwd(const void* dy, const void* x, const void* weight, const float* rstd,
+                                  int dtype, void* dx, void* dweight, void* workspace, int64_t rows,
+                                  int64_t D, void* stream) {
+  if (int rc = check_shape("rms_norm_bwd", rows, D, dtype)) return rc;
+  MI355_REQUIRE(rows == 0 || (dy && x && weight && rstd), "rms_norm_bwd: null pointer");
+  MI355_REQUIRE(!dweight || rows == 0 || workspace, "rms_norm_bwd: workspace required for dweight");
+  hipStream_t s = as_stream(stream);
+  const int per = (int)dw_rows_per_chunk(rows);
+  const int chunks = (int)((rows + per - 1) / per);
+  const dim3 rgrid((unsigned)((rows + 3) / 4));
+  const dim3 cgrid((unsigned)((D + 255) / 256), (unsigned)std::max(chunks, 1));
+  const dim3 fgrid((unsigned)((D + 255) / 256));
+  auto run = [&](auto tag) {
+    using T = decltype(tag);
+    if (dx && rows > 0)
+      hipLaunchKernelGGL(rms_dx_kernel<T>, rgrid, dim3(256), 0, s, static_cast<const T*>(dy),
+                         static_cast<const T*>(x), static_cast<const T*>(weight), rstd, static_cast<T*>(dx),
+                         (int)rows, (int)D, rows_are_16_byte_aligned(D, dtype, {dy, x, weight, dx}));
+    if (dweight) {
+      if (rows > 0)
+        hipLaunchKernelGGL(rms_dw_partial_kernel<T>, cgrid, dim3(256), 0, s, static_cast<const T*>(dy),
+                           static_cast<const T*>(x), rstd, static_cast<float*>(workspace), (int)rows, (int)D,
+                           per);
+      // no rows: the sum over nothing, zeros
+      hipLaunchKernelGGL(rms_dw_final_kernel<T>, fgrid, dim3(256), 0, s, static_cast<const float*>(workspace),
+                         static_cast<T*>(dweight), chunks, (int)D);
+    }
+  };
+  if (dtype == MI355_F32) run(float{}); else run(uint16_t{});
+  return check_launch("rms_norm_bwd");
+}

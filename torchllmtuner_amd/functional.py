@@ -114,6 +114,23 @@ class RouteSelectCutoffFunction(torch.autograd.Function):
         return (dlogits,) + (None,) * 5
 
 
+class RMSNormFunction(torch.autograd.Function):
+    """y = x * rsqrt(mean(x^2) + eps) * weight over the last axis; keeps only rstd."""
+
+    @staticmethod
+    def forward(ctx, x, weight, epsilon):
+        y, rstd = ops.rms_norm_fwd(x, weight, epsilon)
+        ctx.save_for_backward(x, weight, rstd)
+        return y
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, dy):
+        x, weight, rstd = ctx.saved_tensors
+        dx, dw = ops.rms_norm_bwd(dy, x, weight, rstd, ctx.needs_input_grad[0], ctx.needs_input_grad[1])
+        return dx, dw, None
+
+
 class PermuteRowsFunction(torch.autograd.Function):
     """rows[r] = x[token of row r]; backward sums the K row gradients per token."""
 
@@ -210,6 +227,10 @@ def route_select(logits_TE, expert_bias_E, top_k, score_func, route_norm, route_
 
 def route_select_cutoff(logits_TE, expert_bias_E, top_k, score_func, route_norm, route_scale):
     return RouteSelectCutoffFunction.apply(logits_TE, expert_bias_E, top_k, score_func, route_norm, route_scale)
+
+
+def rms_norm(x, weight, epsilon):
+    return RMSNormFunction.apply(x, weight, epsilon)
 
 
 def permute_rows(x_TD, plan):

@@ -1,4 +1,4 @@
-"""Kernel-registry seam: ``moe_token_permute`` served by the MI355X kernels.
+"""Kernel-registry seam: ``moe_token_permute`` and ``rms_norm`` served by the MI355X kernels.
 
 The reference routes a handful of operators through a name -> {device type -> callable}
 registry (``llmtuner/kernel/registry.py:22-103``) and exposes the MoE row gather as
@@ -14,6 +14,10 @@ reference's own registry::
     from llmtuner.kernel import register_kernel
     from torchllmtuner_amd.kernel_registry import moe_token_permute_mi355
     register_kernel("moe_token_permute", "cuda")(moe_token_permute_mi355)
+    register_kernel("rms_norm", "cuda")(rms_norm_mi355)
+
+``rms_norm`` (``llmtuner/kernel/ops/rms_norm.py:10-31``) is the norm the decoder layer applies
+right before the MoE block; it gets a ``"cuda"`` backend the same way.
 
 There is no torch-math backend here: asking for one (``use_eager=True``, a CPU tensor,
 ``fallback_to_cpu=True`` with nothing registered for ``"cpu"``) raises.
@@ -22,6 +26,7 @@ There is no torch-math backend here: asking for one (``use_eager=True``, a CPU t
 from __future__ import annotations
 
 import logging
+import math
 from collections.abc import Callable
 from typing import Any, TypeVar
 
@@ -151,10 +156,47 @@ def moe_token_permute(hidden_states: torch.Tensor, expert_ids: torch.Tensor, *,
     return dispatch_kernel("moe_token_permute", hidden_states, expert_ids, **extra)
 
 
+def _check_rms_norm_inputs(hidden_states: torch.Tensor, weight: torch.Tensor, epsilon: float) -> None:
+    """Metadata-only validation, ``llmtuner/kernel/validation.py:110-120``."""
+    if hidden_states.device != weight.device:
+        raise ValueError(f"Kernel inputs must share a device, got {hidden_states.device} and {weight.device}")
+    if weight.ndim != 1 or hidden_states.ndim == 0:
+        raise ValueError("RMSNorm requires a 1-D weight and a non-scalar input")
+    if hidden_states.shape[-1] != weight.shape[0] or weight.numel() == 0:
+        raise ValueError("RMSNorm weight must match the nonzero final input dimension")
+    if not math.isfinite(epsilon) or epsilon < 0:
+        raise ValueError("RMSNorm epsilon must be finite and nonnegative")
+
+
+@register_kernel("rms_norm", "cuda")
+def rms_norm_mi355(hidden_states: torch.Tensor, weight: torch.Tensor, epsilon: float) -> torch.Tensor:
+    """``hidden_states * rsqrt(mean(hidden_states**2, -1) + epsilon) * weight`` on the GPU,
+    computed in fp32 and rounded once to the input dtype (what
+    ``torch.nn.functional.rms_norm``, the reference's CPU backend, returns); differentiable
+    in both arguments.  Input and weight share a dtype (fp32 or bf16), as the reference
+    leaves dtype conversion to the caller."""
+    _check_rms_norm_inputs(hidden_states, weight, epsilon)
+    if hidden_states.device.type != "cuda":
+        raise RuntimeError(f"rms_norm_mi355 needs tensors on a HIP device, got {hidden_states.device}")
+    return F.rms_norm(hidden_states, weight, epsilon)
+
+
+def rms_norm(hidden_states: torch.Tensor, weight: torch.Tensor, epsilon: float, *,
+             use_eager: bool = False) -> torch.Tensor:
+    """The public operator of ``llmtuner/kernel/ops/rms_norm.py:10-31``, dispatched on the
+    input's device.  ``use_eager`` asks for torch math, which this package does not carry."""
+    if use_eager:
+        raise NotImplementedError(
+            "rms_norm: no torch-math backend in this package; the HIP kernel is the only implementation")
+    return dispatch_kernel("rms_norm", hidden_states, weight, epsilon)
+
+
 __all__ = [
     "dispatch_kernel",
     "get_kernel",
     "moe_token_permute",
     "moe_token_permute_mi355",
     "register_kernel",
+    "rms_norm",
+    "rms_norm_mi355",
 ]

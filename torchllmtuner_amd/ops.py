@@ -186,6 +186,43 @@ def quantile_estimate(histogram_EB, expert_bias_E, top_k):
     return out.to(expert_bias_E.dtype)
 
 
+def rms_norm_fwd(x, weight, epsilon):
+    """Returns ``(y, rstd)``; ``x`` is ``(..., D)``, ``weight`` ``(D,)`` of the same dtype."""
+    dev = _dev(x, weight)
+    if x.dtype != weight.dtype:
+        raise TypeError(f"rms_norm: input ({x.dtype}) and weight ({weight.dtype}) must share a dtype")
+    x, weight = _c(x), _c(weight)
+    D = weight.numel()
+    rows = x.numel() // D
+    y = torch.empty_like(x)
+    rstd = torch.empty(rows, dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_rms_norm_fwd(_p(x), _p(weight), _dt(x), _p(y), _p(rstd), rows, D,
+                                            float(epsilon), _stream(dev))
+    _lib.check(rc, "rms_norm_fwd")
+    return y, rstd
+
+
+def rms_norm_bwd(dy, x, weight, rstd, need_dx=True, need_dw=True):
+    """Returns ``(dx or None, dweight or None)``."""
+    dev = _dev(dy, x, weight, rstd)
+    dy, x, weight = _c(dy), _c(x), _c(weight)
+    if dy.dtype != x.dtype:
+        dy = dy.to(x.dtype)
+    D = weight.numel()
+    rows = x.numel() // D
+    lib = _lib.load()
+    dx = torch.empty_like(x) if need_dx else None
+    dw = torch.empty_like(weight) if need_dw else None
+    ws = torch.empty(max(lib.mi355_rms_norm_bwd_workspace_bytes(rows, D), 4), dtype=torch.uint8,
+                     device=dev) if need_dw else None
+    with torch.cuda.device(dev):
+        rc = lib.mi355_rms_norm_bwd(_p(dy), _p(x), _p(weight), _p(rstd), _dt(x), _p(dx), _p(dw), _p(ws),
+                                    rows, D, _stream(dev))
+    _lib.check(rc, "rms_norm_bwd")
+    return dx, dw
+
+
 def router_select_bwd(logits_TE, ids_TK, dweights_TK, dscores_TE, score_func, route_norm,
                       route_scale, mode=SELECT_TOPK):
     dev = _dev(logits_TE, ids_TK, dweights_TK, dscores_TE)
