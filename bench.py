@@ -212,6 +212,21 @@ def main():
             "permute_rows_bwd": time_events(lambda: ops.permute_rows_bwd(buf["drows"], plan), it),
             "router_gate_bwd": time_events(lambda: ops.router_gate_bwd(logits, x, block.router.gate.weight), it),
         }
+        # the callers' side of the path, outside the timed step: the decoder layer's norm in
+        # front of the block and the statistics of a quantile-balanced router
+        norm_w = torch.ones(D, dtype=torch.bfloat16, device=dev)
+        normed, rstd = ops.rms_norm_fwd(x, norm_w, 1e-6)
+        q_bias = torch.zeros(E, dtype=torch.float32, device=dev)
+        _, _, q_scores, q_cut = ops.router_select_cutoff_fwd(logits, q_bias, K, "sigmoid", True, 1.0)
+        q_hist = torch.zeros(E, 1000, dtype=torch.int64, device=dev)
+        outside_ms = {
+            "rms_norm_fwd": time_events(lambda: ops.rms_norm_fwd(x, norm_w, 1e-6), it),
+            "rms_norm_bwd": time_events(lambda: ops.rms_norm_bwd(gout, x, norm_w, rstd), it),
+            "router_select_cutoff_fwd": time_events(
+                lambda: ops.router_select_cutoff_fwd(logits, q_bias, K, "sigmoid", True, 1.0), it),
+            "quantile_observe": time_events(lambda: ops.quantile_observe(q_hist, q_scores, q_cut, q_bias), it),
+        }
+        other_ms.update(outside_ms)
     # algorithmic work per launch (padding excluded): 2*R*D*F per projection
     proj = 2.0 * R_rows * D * F
     stage_flops = {"gate_up": 2 * proj, "down": proj, "dh": proj, "drows": 2 * proj,
@@ -222,6 +237,8 @@ def main():
         "combine_fwd": R_rows * D * s_bytes + 8 * T * K + T * D * s_bytes,
         "combine_bwd": T * D * s_bytes + 2 * R_rows * D * s_bytes + 4 * T * K,
         "permute_rows_bwd": R_rows * D * s_bytes + T * D * s_bytes,
+        "rms_norm_fwd": 2 * T * D * s_bytes,
+        "rms_norm_bwd": 3 * T * D * s_bytes,
     }
     kernels = {}
     for s, ms in stage_ms.items():
@@ -229,8 +246,10 @@ def main():
         kernels[f"grouped_{s}"] = {"ms": round(ms, 4), "TFLOP/s": round(tf, 1), "frac_mfma": round(tf / PEAK_BF16_TFLOPS, 4)}
     for s, ms in other_ms.items():
         ent = {"ms": round(ms, 4)}
-        if s == "permute_rows_fwd":
-            ent["in_step"] = False  # public dispatcher API only: the fused step gathers inside the GEMMs
+        if s == "permute_rows_fwd" or s in outside_ms:
+            # permute_rows_fwd: public dispatcher API only, the fused step gathers inside the
+            # GEMMs; the others belong to the block's callers
+            ent["in_step"] = False
         if s in other_bytes:
             gbs = other_bytes[s] / (ms * 1e-3) / 1e9
             ent.update({"GB/s": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4)})

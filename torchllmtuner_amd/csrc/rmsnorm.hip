@@ -13,6 +13,7 @@
 // second kernel in a fixed order (no atomics, deterministic).
 #include <algorithm>
 #include <initializer_list>
+#include <type_traits>
 
 #include "common.h"
 
@@ -147,6 +148,66 @@ __global__ __launch_bounds__(256) void rms_dx_kernel(const T* __restrict__ dy, c
   else row_dx<T, 1>(dy + o, x + o, w, dx + o, r, c, D, lane);
 }
 
+// dx and the column sums of dweight in one pass over dy and x: a workgroup walks a run of
+// rows, one wavefront per row; a lane keeps the dweight partial sums of the columns it owns
+// in registers across its rows (ITER 16-byte groups per lane), the four waves add theirs up
+// through LDS at the end and the workgroup writes one row of partial sums.
+constexpr int kFusedBlocks = 2048;  // at most; 512 until a workgroup would get more than 32 rows
+
+template <typename T, int ITER>
+__global__ __launch_bounds__(256) void rms_bwd_fused_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+                                                            const T* __restrict__ w,
+                                                            const float* __restrict__ rstd, T* __restrict__ dx,
+                                                            float* __restrict__ partial, int rows, int D,
+                                                            int rows_per_block) {
+  constexpr int N = kVec<T>;
+  extern __shared__ float colsum[];  // [D]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float acc[ITER][N];
+#pragma unroll
+  for (int k = 0; k < ITER; ++k)
+#pragma unroll
+    for (int j = 0; j < N; ++j) acc[k][j] = 0.0f;
+  const int r0 = blockIdx.x * rows_per_block;
+  const int r1 = min(r0 + rows_per_block, rows);
+  for (int row = r0 + wave; row < r1; row += 4) {
+    const int64_t o = static_cast<int64_t>(row) * D;
+    const float r = rstd[row];
+    const float c = wave_sum(row_dot<T, N>(dy + o, x + o, w, r, D, lane)) / static_cast<float>(D);
+#pragma unroll
+    for (int k = 0; k < ITER; ++k) {
+      const int i = (k * kWave + lane) * N;
+      if (i < D) {
+        float a[N], b[N], g[N], out[N];
+        Pack<T, N>::load(dy + o + i, a);
+        Pack<T, N>::load(x + o + i, b);
+        Pack<T, N>::load(w + i, g);
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+          const float xh = b[j] * r;
+          out[j] = r * (a[j] * g[j] - xh * c);
+          acc[k][j] += a[j] * xh;
+        }
+        if (dx) Pack<T, N>::store(dx + o + i, out);
+      }
+    }
+  }
+  for (int turn = 0; turn < 4; ++turn) {
+    if (wave == turn) {
+#pragma unroll
+      for (int k = 0; k < ITER; ++k) {
+        const int i = (k * kWave + lane) * N;
+        if (i < D) {
+#pragma unroll
+          for (int j = 0; j < N; ++j) colsum[i + j] = turn == 0 ? acc[k][j] : colsum[i + j] + acc[k][j];
+        }
+      }
+    }
+    __syncthreads();
+  }
+  for (int d = threadIdx.x; d < D; d += 256) partial[static_cast<int64_t>(blockIdx.x) * D + d] = colsum[d];
+}
+
 // rows per workgroup of the column sums: 64, more once that would exceed 4096 workgroups
 __host__ __device__ inline int64_t dw_rows_per_chunk(int64_t rows) {
   const int64_t per = (rows + 4095) / 4096;
@@ -174,15 +235,29 @@ __global__ __launch_bounds__(256) void rms_dw_partial_kernel(const T* __restrict
   partial[static_cast<int64_t>(blockIdx.y) * D + d] = acc;
 }
 
+// dw[d] = sum over the chunks of partial[chunk][d]: 16 columns x 16 slices per workgroup, slice
+// s adds chunks s, s+16, ... (independent loads, several in flight), the slices are then
+// added in order -- a fixed summation tree.
 template <typename T>
 __global__ __launch_bounds__(256) void rms_dw_final_kernel(const float* __restrict__ partial, T* __restrict__ dw,
                                                            int chunks, int D) {
-  const int d = blockIdx.x * 256 + threadIdx.x;
-  if (d >= D) return;
+  __shared__ float part[16][17];
+  const int col = threadIdx.x & 15, slice = threadIdx.x >> 4;
+  const int d = blockIdx.x * 16 + col;
   float acc = 0.0f;
-  for (int c = 0; c < chunks; ++c) acc += partial[static_cast<int64_t>(c) * D + d];
-  const float out[1] = {acc};
-  Pack<T, 1>::store(dw + d, out);
+  if (d < D) {
+#pragma unroll 8
+    for (int c = slice; c < chunks; c += 16) acc += partial[static_cast<int64_t>(c) * D + d];
+  }
+  part[slice][col] = acc;
+  __syncthreads();
+  if (slice == 0 && d < D) {
+    float total = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) total += part[k][col];
+    const float out[1] = {total};
+    Pack<T, 1>::store(dw + d, out);
+  }
 }
 
 int rows_are_16_byte_aligned(int64_t D, int dtype, std::initializer_list<const void*> ptrs) {
@@ -227,7 +302,7 @@ extern "C" int mi355_rms_norm_fwd(const void* x, const void* weight, int dtype, 
 extern "C" int64_t mi355_rms_norm_bwd_workspace_bytes(int64_t rows, int64_t D) {
   if (rows < 0 || D < 1) return 0;
   const int64_t per = dw_rows_per_chunk(rows);
-  return ((rows + per - 1) / per) * D * 4;
+  return std::max<int64_t>((rows + per - 1) / per, kFusedBlocks) * D * 4;
 }
 
 extern "C" int mi355_rms_norm_bwd(const void* dy, const void* x, const void* weight, const float* rstd,
@@ -241,9 +316,33 @@ extern "C" int mi355_rms_norm_bwd(const void* dy, const void* x, const void* wei
   const int chunks = (int)((rows + per - 1) / per);
   const dim3 rgrid((unsigned)((rows + 3) / 4));
   const dim3 cgrid((unsigned)((D + 255) / 256), (unsigned)std::max(chunks, 1));
-  const dim3 fgrid((unsigned)((D + 255) / 256));
+  const dim3 fgrid((unsigned)((D + 15) / 16));
   auto run = [&](auto tag) {
     using T = decltype(tag);
+    // one pass for both when rows are 16-byte aligned and a lane's columns fit in registers
+    constexpr int N = 16 / sizeof(T);
+    const int64_t groups = (D / N + kWave - 1) / kWave;  // 16-byte groups per lane
+    if (dweight && rows > 0 && groups <= 16 && D * 4 <= 64 * 1024 &&
+        rows_are_16_byte_aligned(D, dtype, {dy, x, weight, dx})) {
+      const int blocks = (int)std::min<int64_t>(std::min<int64_t>(kFusedBlocks, std::max<int64_t>(512, rows / 32)),
+                                                (rows + 3) / 4);
+      const int rpb = (int)((rows + blocks - 1) / blocks);
+      const int used = (int)((rows + rpb - 1) / rpb);
+      auto launch = [&](auto iter) {
+        constexpr int ITER = decltype(iter)::value;
+        hipLaunchKernelGGL((rms_bwd_fused_kernel<T, ITER>), dim3(used), dim3(256), (size_t)D * 4, s,
+                           static_cast<const T*>(dy), static_cast<const T*>(x), static_cast<const T*>(weight), rstd,
+                           static_cast<T*>(dx), static_cast<float*>(workspace), (int)rows, (int)D, rpb);
+      };
+      if (groups <= 1) launch(std::integral_constant<int, 1>{});
+      else if (groups <= 2) launch(std::integral_constant<int, 2>{});
+      else if (groups <= 4) launch(std::integral_constant<int, 4>{});
+      else if (groups <= 8) launch(std::integral_constant<int, 8>{});
+      else launch(std::integral_constant<int, 16>{});
+      hipLaunchKernelGGL(rms_dw_final_kernel<T>, fgrid, dim3(256), 0, s, static_cast<const float*>(workspace),
+                         static_cast<T*>(dweight), used, (int)D);
+      return;
+    }
     if (dx && rows > 0)
       hipLaunchKernelGGL(rms_dx_kernel<T>, rgrid, dim3(256), 0, s, static_cast<const T*>(dy),
                          static_cast<const T*>(x), static_cast<const T*>(weight), rstd, static_cast<T*>(dx),
