@@ -303,8 +303,9 @@ int mi355_combine_bwd(const void* dout, const void* y, int dtype,
  * into the operand loads, so the (R,D) expert-major copy is never written.  bf16 with
  * D and F multiples of 64 only (MI355_EUNSUP otherwise).
  * gate/up/h are saved for the backward (each (row_capacity,F)).
- * bf16 uses MFMA tiles of tile_m rows (the plan's tile list must have been built
- * with the value mi355_grouped_tile_m(dtype) returns).
+ * The kernels walk the plan's tile list in tiles of mi355_grouped_tile_m(dtype) rows, so
+ * the list must have been built with that value (256; 128 when the process runs with
+ * MI355_ROW_LAYOUT=wide, which selects the 128 x 512 row tile of the bf16 kernels).
  */
 int64_t mi355_grouped_tile_m(int dtype);
 int mi355_grouped_swiglu_fwd(const void* rows, const int32_t* token_of_row,

@@ -9,9 +9,12 @@
 
 namespace mi355 {
 
-constexpr int kTileM = 128;
-
 bool bf16_fast_path_ok(int64_t D, int64_t F);
+int bf16_row_tile_m();
+// rows per entry of the plan's tile list: the row-tile height of the bf16 MFMA kernels, for
+// every dtype (a plan is built from expert ids alone, before the dtype of its rows is known;
+// the generic kernels walk tiles of any multiple of 64 rows)
+inline int tile_m_for(int dtype) { (void)dtype; return bf16_row_tile_m(); }
 int bf16_grouped_fwd(const void* rows, const int32_t* token_of_row, const void* w1, const void* w3,
                      const void* w2, const int32_t* seg_offsets, const int32_t* seg_counts,
                      const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* num_tiles,
@@ -79,10 +82,10 @@ int rowseg(const Seg& sg, const void* A, int64_t lda, const void* B, int64_t b_r
   g.A = A; g.B = B; g.C = C;
   g.a_rs = lda; g.a_cs = 1; g.b_rs = b_rs; g.b_cs = b_cs; g.b_es = b_es;
   g.ldc = N; g.M = 0; g.N = (int)N; g.K = (int)K;
-  g.mode = GEMM_ROWSEG; g.accumulate = accumulate; g.ksplit = 1; g.tile_m = kTileM;
+  g.mode = GEMM_ROWSEG; g.accumulate = accumulate; g.ksplit = 1; g.tile_m = tile_m_for(dtype);
   g.seg_offsets = sg.seg_offsets; g.seg_counts = sg.seg_counts; g.tile_expert = sg.tile_expert;
   g.tile_row0 = sg.tile_row0; g.num_tiles = sg.num_tiles;
-  return launch_gemm(g, dtype, dtype, dtype, gemm_grid_rowseg(sg.tile_capacity, kTileM, (int)N), s);
+  return launch_gemm(g, dtype, dtype, dtype, gemm_grid_rowseg(sg.tile_capacity, tile_m_for(dtype), (int)N), s);
 }
 
 // C[e](M, N) = sum_{r in segment e} A[r][m] * B[r][n]
@@ -115,8 +118,7 @@ int check_common(const char* who, int dtype, int64_t El, int64_t D, int64_t F, i
 using namespace mi355;
 
 extern "C" int64_t mi355_grouped_tile_m(int dtype) {
-  (void)dtype;
-  return kTileM;
+  return tile_m_for(dtype);
 }
 
 extern "C" int mi355_grouped_swiglu_fwd(const void* rows, const int32_t* token_of_row,

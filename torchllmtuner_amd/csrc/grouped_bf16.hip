@@ -7,11 +7,14 @@
 //   drows    dgate . w1 + dup . w3      A KC, B KS   (one accumulator, K = 2F)
 //   dw*      a_e^T . b_e                A KS, B KS   K = the expert's rows
 //
-// Shape of the kernels.  128x512 output tiles for the row-tiled products (384 wide when
-// that divides the width and 512 does not) and 256x256 for the weight gradients, eight
-// waves per workgroup (two per SIMD, each wave a 64x128 accumulator tile), one workgroup
-// per CU with the 160 KiB of LDS holding two stages of the operand tiles.  Row tiles come
-// from the permutation plan's tile list (128 rows of one expert each).
+// Shape of the kernels.  256x256 output tiles for the row-tiled products and the weight
+// gradients alike, eight waves per workgroup as 4 (rows) x 2 (columns), two per SIMD, each
+// wave a 64x128 accumulator tile; one workgroup per CU, two 64 KiB LDS stages of operand
+// tiles (overlaid by the eight 17 KiB epilogue regions).  Row tiles come from the
+// permutation plan's tile list (up to 256 rows of one expert each).  A 128x512 shape of the
+// row tile (waves 2 x 4; 384 wide when that divides the width and 512 does not) is kept
+// behind MI355_ROW_LAYOUT=wide: it stages a quarter more operand bytes per flop and fetches
+// an expert's weights twice as often, and measured 2-3 % slower per training step.
 //
 // What bounds them, measured on MI355X.  With operands of random bits the card's power
 // management holds the core clock near 1.5-1.9 GHz (2.4 GHz with constant operands): a
@@ -29,7 +32,7 @@
 //     for LDS traffic only, so a tile's stores drain under the next tile's work;
 //   * hardware bf16 conversion and transcendental-unit sigmoid in the epilogues (they
 //     were VALU bound);
-//   * a wave skips the MFMAs of 32-row blocks that hold no real rows (last tile of an
+//   * a wave skips the MFMAs of 16-row blocks that hold no real rows (last tile of an
 //     expert).
 //
 // K loop: one barrier per K step of 64.  Per quarter step a wave reads its fragments,
@@ -89,9 +92,9 @@ struct RowArgs {
   int n_tiles;
 };
 
-// Row-tiled kernel: 128 rows of one expert x 512 output columns, 8 waves as 2 (rows) x 4
-// (columns), each wave 64 x 128.  GATEUP's 512 columns are 256 gate + 256 up columns of
-// the same f range, so a wave holds gate and up of the same 64 f.
+// Row-tiled kernel: 64 WM rows of one expert x 32 NJ (8 / WM) output columns, 8 waves as WM
+// (rows) x 8 / WM (columns), each wave 64 x 32 NJ.  GATEUP's columns are half gate and half
+// up columns of the same f range, so a wave holds gate and up of the same 16 NJ f.
 constexpr int RBM = 128, RBN = 512;
 constexpr int R_STAGE = (RBM + RBN) * BK;  // elements per LDS stage (80 KiB)
 
@@ -99,17 +102,20 @@ struct TileMeta {
   int e, row0, valid, n0;
 };
 
-template <int MODE, int NJ, bool GATHER>
+template <int MODE, int NJ, bool GATHER, int WM>
 __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
-  constexpr int BNT = 128 * NJ;            // output columns of the tile (4 waves x NJ x 32)
-  constexpr int NB = BNT / 64;             // 16-byte B chunks staged per thread and K step
-  constexpr int STAGE = (RBM + BNT) * BK;  // elements per LDS stage
+  constexpr int WN = 8 / WM;               // waves along the columns (WM along the rows)
+  constexpr int TBM = 64 * WM;             // rows of the tile
+  constexpr int BNT = 32 * NJ * WN;        // output columns of the tile (WN waves x NJ x 32)
+  constexpr int NA = TBM / 64;             // 16-byte A chunks staged per thread and K step
+  constexpr int NB = BNT / 64;             // the same for B
+  constexpr int STAGE = (TBM + BNT) * BK;  // elements per LDS stage
   constexpr bool B_KS = (MODE == RM_DH || MODE == RM_DX);
   static_assert(!GATHER || MODE == RM_GATEUP, "only the gate/up product gathers its rows");
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = (wave >> 2) * 64, wn = wave & 3;
+  const int wm = (wave / WN) * 64, wn = wave % WN;
   const int wave_m = __builtin_amdgcn_readfirstlane(wm);  // the same value, known to be wave-uniform
   const int D = p.D, F = p.F;
   const int Kdim = (MODE == RM_GATEUP || MODE == RM_DH) ? D : (MODE == RM_DOWN ? F : 2 * F);
@@ -138,7 +144,7 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
     TileMeta m;
     m.e = p.tile_expert[tile];
     m.row0 = p.tile_row0[tile];
-    m.valid = min(RBM, p.seg_offsets[m.e] + p.seg_counts[m.e] - m.row0);
+    m.valid = min(TBM, p.seg_offsets[m.e] + p.seg_counts[m.e] - m.row0);
     // a last tile that would overhang starts early instead and recomputes a few columns
     // of its neighbour (same values), so no column is ever clamped
     constexpr int W = (MODE == RM_GATEUP ? BNT / 2 : BNT);
@@ -149,7 +155,7 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
   // ---- global -> register staging: 16-byte chunks q = tid + 512*i ---------------------
   // KC tiles (8 chunks per row): row (tid>>3) + 64*i, chunk tid&7.
   // KS tile (BNT/8 chunks per k row): chunk q -> k = q / (BNT/8), chunk q % (BNT/8).
-  u32x4 ra[2], rb[NB];
+  u32x4 ra[NA], rb[NB];
   const int kc_row = tid >> 3, kc_chunk = tid & 7;
   const int kc_lds = kc_row * BK + ((kc_chunk ^ ((kc_row >> 1) & 7)) << 3);  // + i*64*BK (64 % 16 == 0)
   int b_lds[NB];
@@ -198,21 +204,21 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
   const char* ubA1;  // DX: second half of the contraction (dup)
   const char* ubB0;  // B tile origin in the first weight stack
   int64_t b1_bytes;  // second weight stack - first (one flat address space)
-  uint32_t voffA[2];
+  uint32_t voffA[NA];
   // source rows of the A tile: the tile's own rows, or token rows through the gather index
-  auto load_asrc = [&](const TileMeta& m, int (&asrc)[2]) {
+  auto load_asrc = [&](const TileMeta& m, int (&asrc)[NA]) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < NA; ++i) {
       const int r = max(min(kc_row + 64 * i, m.valid - 1), 0);
       asrc[i] = GATHER ? p.a_src[m.row0 + r] : r;
     }
   };
-  auto setup = [&](const TileMeta& m, const int (&asrc)[2]) {
+  auto setup = [&](const TileMeta& m, const int (&asrc)[NA]) {
     const int64_t arow = GATHER ? 0 : static_cast<int64_t>(m.row0) * lda;
     ubA0 = reinterpret_cast<const char*>(p.a0 + arow);
     ubA1 = (MODE == RM_DX) ? reinterpret_cast<const char*>(p.a1 + arow) : ubA0;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) voffA[i] = static_cast<uint32_t>(max(asrc[i], 0) * lda + kc_chunk * 8) * 2u;
+    for (int i = 0; i < NA; ++i) voffA[i] = static_cast<uint32_t>(max(asrc[i], 0) * lda + kc_chunk * 8) * 2u;
     const uint16_t* B0 = p.b0 + m.e * wsz;
     const uint16_t* B1 = (MODE == RM_GATEUP || MODE == RM_DX) ? p.b1 + m.e * wsz : B0;
     b1_bytes = (B1 - B0) * 2;
@@ -245,7 +251,7 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
   // request every chunk of K step `step` of the fetch tile
   auto issue = [&](int step) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) ra[i] = load_a(kofs(step), i);
+    for (int i = 0; i < NA; ++i) ra[i] = load_a(kofs(step), i);
 #pragma unroll
     for (int i = 0; i < NB; ++i) rb[i] = load_b(kofs(step), i);
   };
@@ -253,7 +259,7 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
   TileMeta cur = load_meta(within);
   TileMeta nxt = load_meta(exists(within + stride) ? within + stride : within);
   {
-    int asrc[2];
+    int asrc[NA];
     load_asrc(cur, asrc);
     setup(cur, asrc);
     issue(0);
@@ -263,7 +269,7 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
   const bool more = exists(within + stride);
   // the tile after the next: looked up now, used one tile later
   const TileMeta nxt2 = load_meta(exists(within + 2 * stride) ? within + 2 * stride : within);
-  int nsrc[2];
+  int nsrc[NA];
   load_asrc(nxt, nsrc);
   const int row0 = cur.row0, valid = cur.valid, n0 = cur.n0;
 
@@ -277,9 +283,9 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
 
   // K step 0 (requested before the previous epilogue) -> LDS stage 0, K step 1 -> registers
 #pragma unroll
-  for (int i = 0; i < 2; ++i) *reinterpret_cast<u32x4*>(smem + kc_lds + i * 64 * BK) = ra[i];
+  for (int i = 0; i < NA; ++i) *reinterpret_cast<u32x4*>(smem + kc_lds + i * 64 * BK) = ra[i];
 #pragma unroll
-  for (int i = 0; i < NB; ++i) *reinterpret_cast<u32x4*>(smem + RBM * BK + b_lds[i]) = rb[i];
+  for (int i = 0; i < NB; ++i) *reinterpret_cast<u32x4*>(smem + TBM * BK + b_lds[i]) = rb[i];
   if (ksteps > 1) issue(1);
   __syncthreads();
 
@@ -296,9 +302,9 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
     constexpr bool has_next = decltype(has_next_t)::value;
     constexpr bool has_next2 = decltype(has_next2_t)::value;
     const uint16_t* As = smem + (ks & 1) * STAGE;
-    const uint16_t* Bs = As + RBM * BK;
+    const uint16_t* Bs = As + TBM * BK;
     uint16_t* An = smem + ((ks + 1) & 1) * STAGE;
-    uint16_t* Bn = An + RBM * BK;
+    uint16_t* Bn = An + TBM * BK;
 #pragma unroll
     for (int kk = 0; kk < BK / 32; ++kk) {
       bf16x8 af[4];
@@ -319,13 +325,14 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
         // same registers with the same chunks of tile ks+2.
         const int q = kk * 2 + hb;
         if constexpr (has_next) {
-          if (q < 2) *reinterpret_cast<u32x4*>(An + kc_lds + q * 64 * BK) = ra[q];
+          // A: two chunks ride with the first two quarters, or one with each of the four
+          if (q < NA) *reinterpret_cast<u32x4*>(An + kc_lds + q * 64 * BK) = ra[q];
 #pragma unroll
           for (int i = (q * NB) / 4; i < ((q + 1) * NB) / 4; ++i)
             *reinterpret_cast<u32x4*>(Bn + b_lds[i]) = rb[i];
         }
         if constexpr (has_next2) {
-          if (q < 2) ra[q] = load_a(kofs(ks + 2), q);
+          if (q < NA) ra[q] = load_a(kofs(ks + 2), q);
 #pragma unroll
           for (int i = (q * NB) / 4; i < ((q + 1) * NB) / 4; ++i) rb[i] = load_b(kofs(ks + 2), i);
         }
@@ -716,6 +723,22 @@ int set_lds(K kernel, int bytes) {
 
 // The MFMA path needs whole 64-wide K steps, 16-byte aligned rows, and outputs at least
 // one tile wide (a last tile that would overhang is shifted back, never clamped).
+// Two shapes of the row tile: 128 rows x 512 columns (waves 2 x 4) or 256 x 256 (waves 4 x 2).
+// The square one stages a fifth fewer operand bytes per flop and halves how often an
+// expert's weights are fetched, at the price of a coarser last tile per expert.
+// The square one is the default (measured 2-3 % faster per training step on balanced, skewed
+// and few-rows-per-expert routing alike); MI355_ROW_LAYOUT=wide, read once per process,
+// selects the other.
+static bool tall_layout() {
+  static const bool tall = [] {
+    const char* v = std::getenv("MI355_ROW_LAYOUT");
+    return !(v && v[0] == 'w');
+  }();
+  return tall;
+}
+
+int bf16_row_tile_m() { return tall_layout() ? 256 : 128; }
+
 bool bf16_fast_path_ok(int64_t D, int64_t F) { return D % 64 == 0 && F % 64 == 0 && D >= 384 && F >= 384; }
 
 enum { STAGE_GATEUP = 1, STAGE_DOWN = 2, STAGE_DH = 4, STAGE_DX = 8, STAGE_DW2 = 16, STAGE_DW1 = 32, STAGE_DW3 = 64 };
@@ -738,21 +761,42 @@ static unsigned resident_blocks() {
 constexpr int R_LDS_BYTES = 2 * R_STAGE * 2;  // 163840
 constexpr int W_LDS_BYTES = 8 * 64 * 136 * 2;  // 139264: the 8 epilogue regions (> 2 stages = 131072)
 
-template <int MODE, int NJ, bool GATHER = false>
-static int launch_row(RowArgs& a, int64_t tile_capacity, hipStream_t s, const char* what) {
+template <int MODE, int NJ, bool GATHER, int WM>
+static int launch_row_as(RowArgs& a, int64_t tile_capacity, hipStream_t s, const char* what) {
+  constexpr int lds = WM == 4 ? W_LDS_BYTES : R_LDS_BYTES;
   static bool configured = false;  // per process; the attribute is per function
   if (!configured) {
-    if (int rc = set_lds(row_tiled_kernel<MODE, NJ, GATHER>, R_LDS_BYTES)) return rc;
+    if (int rc = set_lds(row_tiled_kernel<MODE, NJ, GATHER, WM>, lds)) return rc;
     configured = true;
   }
   const unsigned blocks = std::min(round8(tile_capacity * a.n_tiles), resident_blocks());
-  hipLaunchKernelGGL((row_tiled_kernel<MODE, NJ, GATHER>), dim3(blocks), dim3(NT), R_LDS_BYTES, s, a);
+  hipLaunchKernelGGL((row_tiled_kernel<MODE, NJ, GATHER, WM>), dim3(blocks), dim3(NT), lds, s, a);
   return check_launch(what);
 }
 
 // 384-column tiles when they divide the width and 512-column tiles do not (F = 768), or
 // when the output is narrower than 512 columns.
 static bool narrow_tiles(int64_t width) { return width < 512 || (width % 512 != 0 && width % 384 == 0); }
+
+// width: output columns; gate/up tiles hold both halves of their column range
+template <int MODE, bool GATHER = false>
+static int launch_row(RowArgs& a, int64_t width, int64_t tile_capacity, hipStream_t s, const char* what) {
+  constexpr int div = MODE == RM_GATEUP ? 2 : 1;
+  if (tall_layout()) {
+    // always 256 wide: a 192-wide KS tile would not hold the swizzle (24 chunks per row are
+    // not a multiple of the 16 the key permutes); an overhanging last tile shifts back
+    a.n_tiles = (int)((width + 256 / div - 1) / (256 / div));
+    return launch_row_as<MODE, 4, GATHER, 4>(a, tile_capacity, s, what);
+  }
+  if constexpr (MODE != RM_GATEUP) {
+    if (narrow_tiles(width)) {
+      a.n_tiles = (int)((width + 383) / 384);
+      return launch_row_as<MODE, 3, GATHER, 2>(a, tile_capacity, s, what);
+    }
+  }
+  a.n_tiles = (int)((width + RBN / div - 1) / (RBN / div));
+  return launch_row_as<MODE, 4, GATHER, 2>(a, tile_capacity, s, what);
+}
 
 int bf16_grouped_fwd(const void* rows, const int32_t* token_of_row, const void* w1, const void* w3,
                        const void* w2, const int32_t* seg_offsets, const int32_t* seg_counts,
@@ -765,23 +809,16 @@ int bf16_grouped_fwd(const void* rows, const int32_t* token_of_row, const void* 
   if (stages & STAGE_GATEUP) {
     a.a0 = (const uint16_t*)rows; a.a_src = token_of_row; a.b0 = (const uint16_t*)w1; a.b1 = (const uint16_t*)w3;
     a.o0 = (uint16_t*)gate; a.o1 = (uint16_t*)up; a.o2 = (uint16_t*)h;
-    a.n_tiles = (int)((F + RBN / 2 - 1) / (RBN / 2));
     if (token_of_row) {
-      if (int rc = launch_row<RM_GATEUP, 4, true>(a, tile_capacity, s, "grouped gate/up")) return rc;
+      if (int rc = launch_row<RM_GATEUP, true>(a, F, tile_capacity, s, "grouped gate/up")) return rc;
     } else {
-      if (int rc = launch_row<RM_GATEUP, 4>(a, tile_capacity, s, "grouped gate/up")) return rc;
+      if (int rc = launch_row<RM_GATEUP>(a, F, tile_capacity, s, "grouped gate/up")) return rc;
     }
   }
   if (stages & STAGE_DOWN) {
     RowArgs b = a;
     b.a0 = (const uint16_t*)h; b.b0 = (const uint16_t*)w2; b.o0 = (uint16_t*)y;
-    if (narrow_tiles(D)) {
-      b.n_tiles = (int)((D + 383) / 384);
-      if (int rc = launch_row<RM_DOWN, 3>(b, tile_capacity, s, "grouped down")) return rc;
-    } else {
-      b.n_tiles = (int)((D + RBN - 1) / RBN);
-      if (int rc = launch_row<RM_DOWN, 4>(b, tile_capacity, s, "grouped down")) return rc;
-    }
+    if (int rc = launch_row<RM_DOWN>(b, D, tile_capacity, s, "grouped down")) return rc;
   }
   return MI355_OK;
 }
@@ -800,25 +837,13 @@ int bf16_grouped_bwd(const void* dy, const void* rows, const int32_t* token_of_r
     a.a0 = (const uint16_t*)dy; a.b0 = (const uint16_t*)w2;
     a.gate = (const uint16_t*)gate; a.up = (const uint16_t*)up;
     a.o0 = (uint16_t*)dgate; a.o1 = (uint16_t*)dup;
-    if (narrow_tiles(F)) {
-      a.n_tiles = (int)((F + 383) / 384);
-      if (int rc = launch_row<RM_DH, 3>(a, tile_capacity, s, "grouped dh")) return rc;
-    } else {
-      a.n_tiles = (int)((F + RBN - 1) / RBN);
-      if (int rc = launch_row<RM_DH, 4>(a, tile_capacity, s, "grouped dh")) return rc;
-    }
+    if (int rc = launch_row<RM_DH>(a, F, tile_capacity, s, "grouped dh")) return rc;
   }
   if (drows && (stages & STAGE_DX)) {
     RowArgs b = a;
     b.a0 = (const uint16_t*)dgate; b.a1 = (const uint16_t*)dup;
     b.b0 = (const uint16_t*)w1; b.b1 = (const uint16_t*)w3; b.o0 = (uint16_t*)drows;
-    if (narrow_tiles(D)) {
-      b.n_tiles = (int)((D + 383) / 384);
-      if (int rc = launch_row<RM_DX, 3>(b, tile_capacity, s, "grouped drows")) return rc;
-    } else {
-      b.n_tiles = (int)((D + RBN - 1) / RBN);
-      if (int rc = launch_row<RM_DX, 4>(b, tile_capacity, s, "grouped drows")) return rc;
-    }
+    if (int rc = launch_row<RM_DX>(b, D, tile_capacity, s, "grouped drows")) return rc;
   }
   static bool wconfigured = false;
   if (!wconfigured) {
