@@ -4,6 +4,8 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+
+#include <atomic>
 #include <stdint.h>
 
 #include <cstdarg>
@@ -26,6 +28,22 @@ int check_launch(const char* what);
   } while (0)
 
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+
+// One-time set-up per device (kernel attributes are per device): `needed()` is true until
+// `done()` has been called with the same device current.  Safe to race: set-up is idempotent.
+class PerDeviceOnce {
+ public:
+  bool needed() const { return !(mask_.load(std::memory_order_acquire) & bit()); }
+  void done() { mask_.fetch_or(bit(), std::memory_order_release); }
+
+ private:
+  static uint64_t bit() {
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    return 1ull << (dev & 63);
+  }
+  std::atomic<uint64_t> mask_{0};
+};
 
 // ---- bf16 <-> f32, round to nearest even (what torch's .to(bfloat16) does) ----
 __device__ __forceinline__ float bf16_to_f32(uint16_t v) {

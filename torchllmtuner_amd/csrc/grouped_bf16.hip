@@ -764,10 +764,10 @@ constexpr int W_LDS_BYTES = 8 * 64 * 136 * 2;  // 139264: the 8 epilogue regions
 template <int MODE, int NJ, bool GATHER, int WM>
 static int launch_row_as(RowArgs& a, int64_t tile_capacity, hipStream_t s, const char* what) {
   constexpr int lds = WM == 4 ? W_LDS_BYTES : R_LDS_BYTES;
-  static bool configured = false;  // per process; the attribute is per function
-  if (!configured) {
+  static PerDeviceOnce configured;  // one per kernel instantiation
+  if (configured.needed()) {
     if (int rc = set_lds(row_tiled_kernel<MODE, NJ, GATHER, WM>, lds)) return rc;
-    configured = true;
+    configured.done();
   }
   const unsigned blocks = std::min(round8(tile_capacity * a.n_tiles), resident_blocks());
   hipLaunchKernelGGL((row_tiled_kernel<MODE, NJ, GATHER, WM>), dim3(blocks), dim3(NT), lds, s, a);
@@ -845,11 +845,11 @@ int bf16_grouped_bwd(const void* dy, const void* rows, const int32_t* token_of_r
     b.b0 = (const uint16_t*)w1; b.b1 = (const uint16_t*)w3; b.o0 = (uint16_t*)drows;
     if (int rc = launch_row<RM_DX>(b, D, tile_capacity, s, "grouped drows")) return rc;
   }
-  static bool wconfigured = false;
-  if (!wconfigured) {
+  static PerDeviceOnce wconfigured;
+  if (wconfigured.needed()) {
     if (int rc = set_lds(wgrad_kernel<false>, W_LDS_BYTES)) return rc;
     if (int rc = set_lds(wgrad_kernel<true>, W_LDS_BYTES)) return rc;
-    wconfigured = true;
+    wconfigured.done();
   }
   auto wgrad = [&](const void* A, const void* B, const int32_t* b_src, void* C, int64_t M, int64_t N, const char* what) {
     WgradArgs w{};

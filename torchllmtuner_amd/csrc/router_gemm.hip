@@ -317,10 +317,10 @@ int64_t router_x3_bwd_workspace(int64_t T, int64_t D, int64_t E) {
 
 int router_x3_fwd(const void* x, const float* w, const float* bias, float* logits, void* workspace, int64_t T,
                   int64_t D, int64_t E, hipStream_t s) {
-  static bool configured = false;
-  if (!configured) {
+  static PerDeviceOnce configured;
+  if (configured.needed()) {
     if (int rc = set_dyn_lds(gate_fwd_kernel, F_LDS)) return rc;
-    configured = true;
+    configured.done();
   }
   uint16_t* ws = static_cast<uint16_t*>(workspace);
   const int64_t n = E * D;
@@ -332,11 +332,11 @@ int router_x3_fwd(const void* x, const float* w, const float* bias, float* logit
 
 int router_x3_bwd(const float* dlogits, const void* x, const float* w, void* dx, float* dw, void* workspace,
                   int64_t T, int64_t D, int64_t E, hipStream_t s) {
-  static bool configured = false;
-  if (!configured) {
+  static PerDeviceOnce configured;
+  if (configured.needed()) {
     if (int rc = set_dyn_lds(gate_dx_kernel, X_LDS)) return rc;
     if (int rc = set_dyn_lds(gate_dw_kernel, W_LDS)) return rc;
-    configured = true;
+    configured.done();
   }
   uint16_t* ws = static_cast<uint16_t*>(workspace);
   const int64_t n = E * D;
