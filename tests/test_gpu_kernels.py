@@ -338,3 +338,20 @@ def test_balance_loss_fwd_bwd(ops, T, E, K, padded):
     # twice the upstream gradient, twice the result
     grad2 = ops.balance_loss_bwd(s.to(DEV), f_E, torch.tensor(2.0, device=DEV), None if pad is None else pad.to(DEV))
     assert torch.equal(grad2, grad * 2)
+
+
+def test_wide_row_tile_layout_in_a_child_process():
+    """The 128 x 512 row tile is chosen per process (MI355_ROW_LAYOUT=wide, read when the
+    library first launches a grouped kernel), so its parity cases run in a child."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, MI355_ROW_LAYOUT="wide")
+    child = subprocess.run(
+        [sys.executable, "-m", "pytest", os.path.join(root, "tests", "test_gpu_kernels.py"), "-q", "-x",
+         "-k", "bf16_mfma or plan_is_the_stable", "-p", "no:cacheprovider"],
+        cwd=root, env=env, capture_output=True, text=True, timeout=300)
+    assert child.returncode == 0, child.stdout[-2000:] + child.stderr[-2000:]
+    assert " passed" in child.stdout
