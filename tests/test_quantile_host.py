@@ -118,3 +118,22 @@ def test_quantile_entry_points_validate_shapes_without_a_gpu():
     assert lib.mi355_quantile_estimate(None, None, None, None, 4, 4, 10, None) != 0  # K must be < E
     assert lib.mi355_router_select_cutoff_fwd(None, None, None, None, None, None, 4, 8, 8, 0, 0, 1.0, None) != 0
     assert b"(K+1)-th" in lib.mi355_moe_last_error()
+
+
+def test_routing_load_metrics_follow_the_counters():
+    # llmtuner/models/common/moe/bias_update.py:100-137
+    from torchllmtuner_amd.moe import collect_routing_load_metrics
+
+    a = _moe(TokenChoiceTopKRouter(E, D, K), load_balance_coeff=0.1)
+    b = _moe(TokenChoiceTopKRouter(E, D, K), load_balance_coeff=0.1)
+    model = _Model([a, b])
+    assert collect_routing_load_metrics([model], None) == {}          # nothing observed yet
+    a.tokens_per_expert_E.copy_(torch.tensor([4.0, 0.0, 2.0, 2.0]))      # mean 2, max 4, one empty
+    metrics = collect_routing_load_metrics([model], None)               # b stays inactive
+    assert metrics["moe/empty_expert_fraction"] == pytest.approx(0.25)
+    assert metrics["moe/max_to_mean_load"] == pytest.approx(2.0)
+    assert metrics["moe/load_cv"] == pytest.approx(float(torch.tensor([4.0, 0, 2, 2]).std(unbiased=False)) / 2.0)
+    b.tokens_per_expert_E.fill_(3.0)                                    # perfectly even
+    metrics = collect_routing_load_metrics([model], None)
+    assert metrics["moe/empty_expert_fraction"] == pytest.approx(0.125)
+    assert metrics["moe/max_to_mean_load"] == pytest.approx(2.0)

@@ -4,6 +4,7 @@ from .activation import SwiGLU
 from .auxiliary_loss import AuxLoss, MicrobatchWiseLoadBalanceLoss
 from .bias_update import (
     collect_moe_layers,
+    collect_routing_load_metrics,
     register_moe_balancing_hook,
     reset_routing_statistics,
     update_expert_bias,
@@ -45,6 +46,7 @@ __all__ = [
     "SwiGLU",
     "TokenChoiceTopKRouter",
     "collect_moe_layers",
+    "collect_routing_load_metrics",
     "hf_expert_state_to_native",
     "moe_from_packed_experts",
     "native_ep_expert_key",

@@ -23,6 +23,7 @@ from .routing import QuantileBalancedTopKRouter
 
 __all__ = [
     "collect_moe_layers",
+    "collect_routing_load_metrics",
     "register_moe_balancing_hook",
     "reset_routing_statistics",
     "update_expert_bias",
@@ -55,6 +56,38 @@ def reset_routing_statistics(model_parts: Sequence[nn.Module]) -> None:
         moe.tokens_per_expert_E.zero_()
         if isinstance(moe.router, QuantileBalancedTopKRouter):
             moe.router.quantile_balancer.required_bias_histogram_EB.zero_()
+
+
+@torch.no_grad()
+def collect_routing_load_metrics(model_parts: Sequence[nn.Module], parallel_dims=None,
+                                 device: torch.device | None = None) -> dict[str, float]:
+    """Load-balance observability from the token counters, read before the optimizer hooks
+    drain them (bias_update.py:100-137): fraction of empty experts, coefficient of variation
+    and max-to-mean load, averaged (max: maximised) over the blocks that saw tokens.  A few
+    ``(E,)`` reductions and one host read-back per call; a logging path, not a hot one."""
+    _single_process(parallel_dims)
+    layers = collect_moe_layers(model_parts)
+    if not layers:
+        return {}
+    device = device if device is not None else layers[0].tokens_per_expert_E.device
+    totals = torch.zeros(4, device=device, dtype=torch.float32)
+    for values in {id(m.tokens_per_expert_E): m.tokens_per_expert_E for m in layers}.values():
+        values = values.to(device).float()
+        mean = values.mean()
+        active = (mean > 0).float()
+        denominator = mean.clamp_min(1e-12)
+        totals[0] += active
+        totals[1] += active * (values == 0).float().mean()
+        totals[2] += active * values.std(unbiased=False) / denominator
+        totals[3] = torch.maximum(totals[3], active * values.max() / denominator)
+    count, empty, cv, maximum = totals.tolist()
+    if not count:
+        return {}
+    return {
+        "moe/empty_expert_fraction": empty / count,
+        "moe/load_cv": cv / count,
+        "moe/max_to_mean_load": maximum,
+    }
 
 
 def _unique(moe_layers: Sequence[MoE]) -> list[MoE]:
