@@ -28,6 +28,15 @@ Pinning status (tests/test_oracle.py holds the checks):
   grouped_experts        pinned: per-segment hand reference, zero-count segments fp64
   combine                pinned: inverse-permute/reshape/sum reference, fp64 exactness
   moe_forward            pinned: analytic experts x(id+1), brute-force fp64 loop
+  balance_loss           pinned: the paper formula, even-load value, scale and order invariance
+  select_top_k_plus_one, quantile_observe, quantile_estimate
+                         pinned: the reference's worked example (bins 1/3/5/6, next bias
+                         [-0.55,-0.15,0.25,0.45]), its past-int32 and fractional-large-count
+                         literals, empty-window identity, mean-centring, padding filter,
+                         pair-by-pair brute force
+  rms_norm               pinned: the reference's fp64 formula + gradcheck, and bit-equality
+                         with torch.nn.functional.rms_norm (the reference's CPU backend) in
+                         fp32 and bf16
   local-share (experts [lo,hi) only)  parity unpinned against the reference: the
                          reference has no single-process form of "one EP rank's
                          share"; defined here as dropping the sorted rows outside
@@ -55,6 +64,11 @@ __all__ = [
     "grouped_experts",
     "combine",
     "shared_expert",
+    "balance_loss",
+    "select_top_k_plus_one",
+    "quantile_observe",
+    "quantile_estimate",
+    "rms_norm",
     "moe_forward",
     "MoEParams",
     "RouterSpec",
