@@ -109,3 +109,32 @@ def test_module_surface_matches_the_reference_block():
     assert "tokens_per_expert_E" not in block.state_dict()
     assert moe.MoE(8, experts, router, load_balance_coeff=None).expert_bias_E is None
     assert list(block.expert_parallel_parameters()) == list(ie.parameters())
+
+
+def test_header_is_plain_c_and_links_against_the_library(tmp_path):
+    """A C99 translation unit that includes the header, takes the address of every declared
+    entry point and links against the shared library: the boundary a cgo / JNI / ctypes binding
+    sees has no C++ or torch types in it."""
+    import shutil
+    import subprocess
+
+    from torchllmtuner_amd import _lib
+
+    if shutil.which("gcc") is None:
+        pytest.skip("no C compiler")
+    _lib.load()
+    names = _declared_functions()
+    src = tmp_path / "abi.c"
+    src.write_text(
+        '#include "mi355_moe.h"\n#include <stdio.h>\nint main(void) {\n  const void* fns[] = {\n'
+        + "".join(f"    (const void*)&{n},\n" for n in names)
+        + '  };\n  printf("%d %d\\n", (int)(sizeof(fns) / sizeof(fns[0])), mi355_moe_abi_version());\n  return 0;\n}\n'
+    )
+    exe = tmp_path / "abi"
+    libdir = os.path.dirname(_lib.LIB_PATH)
+    subprocess.run(
+        ["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe),
+         "-L", libdir, "-lmi355moe", f"-Wl,-rpath,{libdir}"],
+        check=True, capture_output=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
+    assert out == [str(len(names)), "1"]
