@@ -58,10 +58,12 @@ const char* mi355_moe_last_error(void);
  * Replaces RouterGateLinearFunction.forward and RouterGateLinear.forward,
  * llmtuner/models/common/linear.py:107-131,179-183.
  * x: (T,D) x_dtype row-major; w: (E,D) w_dtype; logit_bias: (E) fp32 or NULL.
- * workspace: mi355_router_gate_fwd_workspace_bytes() bytes or NULL.  With a workspace,
- * bf16 x, fp32 w and D, E multiples of 64, each fp32 weight is written as three bf16
- * pieces (24 mantissa bits) and the product runs as three bf16 MFMAs with fp32
- * accumulation; otherwise the strided fp32-MFMA kernel is used.
+ * workspace: mi355_router_gate_fwd_workspace_bytes(T,D,E) bytes (for the same T, D, E)
+ * or NULL.  With a workspace, bf16 x, fp32 w and D, E multiples of 64, each fp32 weight
+ * is written as three bf16 pieces (24 mantissa bits) and the product runs as three bf16
+ * MFMAs with fp32 accumulation (from 1024 tokens on in 128-token tiles with the
+ * contraction split over workgroups, partial sums added in a fixed order); otherwise the
+ * strided fp32-MFMA kernel is used.
  */
 int64_t mi355_router_gate_fwd_workspace_bytes(int64_t T, int64_t D, int64_t E);
 int mi355_router_gate_fwd(const void* x, int x_dtype, const void* w, int w_dtype,

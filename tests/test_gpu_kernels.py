@@ -31,7 +31,9 @@ def ops():
                                        (1000, 320, 72, torch.bfloat16), (0, 16, 4, torch.float32),
                                        # bf16 tokens, D and E multiples of 64: the three-piece bf16 MFMA path
                                        (1000, 320, 64, torch.bfloat16), (2048, 2048, 128, torch.bfloat16),
-                                       (77, 192, 192, torch.bfloat16), (8192, 128, 256, torch.bfloat16)])
+                                       (77, 192, 192, torch.bfloat16), (8192, 128, 256, torch.bfloat16),
+                                       # 128-token tiles: ragged T and E, with and without a split contraction
+                                       (1100, 448, 192, torch.bfloat16), (1100, 1024, 192, torch.bfloat16)])
 def test_router_gate_fwd_bwd(ops, T, D, E, xdt):
     print(f"router_gate T={T} D={D} E={E} {xdt}", flush=True)
     g = torch.Generator().manual_seed(0)

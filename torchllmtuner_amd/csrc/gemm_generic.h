@@ -54,7 +54,7 @@ int launch_splitk_reduce(const float* partial, void* out, int out_dtype, int64_t
 // Router projections as three bf16 MFMAs per fp32 product (router_gemm.hip): bf16 tokens,
 // fp32 weights, D and E multiples of 64.
 bool router_x3_ok(int x_dtype, int w_dtype, int64_t D, int64_t E);
-int64_t router_x3_fwd_workspace(int64_t D, int64_t E);
+int64_t router_x3_fwd_workspace(int64_t T, int64_t D, int64_t E);
 int64_t router_x3_bwd_workspace(int64_t T, int64_t D, int64_t E);
 int router_x3_fwd(const void* x, const float* w, const float* bias, float* logits, void* workspace,
                   int64_t T, int64_t D, int64_t E, hipStream_t s);

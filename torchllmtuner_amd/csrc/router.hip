@@ -296,8 +296,7 @@ int check_router_args(int64_t T, int64_t E, int64_t K) {
 using namespace mi355;
 
 extern "C" int64_t mi355_router_gate_fwd_workspace_bytes(int64_t T, int64_t D, int64_t E) {
-  (void)T;
-  return (D >= 1 && E >= 1 && router_x3_ok(MI355_BF16, MI355_F32, D, E)) ? router_x3_fwd_workspace(D, E) : 0;
+  return (T >= 0 && D >= 1 && E >= 1 && router_x3_ok(MI355_BF16, MI355_F32, D, E)) ? router_x3_fwd_workspace(T, D, E) : 0;
 }
 
 extern "C" int mi355_router_gate_fwd(const void* x, int x_dtype, const void* w, int w_dtype,

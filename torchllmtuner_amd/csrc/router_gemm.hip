@@ -130,6 +130,115 @@ __global__ __launch_bounds__(F_NT) void gate_fwd_kernel(const uint16_t* __restri
   }
 }
 
+// The same product for many tokens: 128 tokens x 128 experts per workgroup, 8 waves as 2 x 4
+// (each 64 tokens x 32 experts), the contraction split over gridDim.z so that the grid still
+// fills the chip.  The 32-token kernel above streams the three weight-piece tiles once per 32
+// tokens -- at T = 8192 that is 0.4 GB through L2 for a 37 MB problem, and all of its time;
+// this one streams them once per 128 tokens.  Partial sums go to the workspace and are added
+// (with the bias) in split order by logits_reduce_kernel; a single split writes logits itself.
+constexpr int G_BM = 128, G_BN = 128, G_NT = 512;
+constexpr int G_STAGE = (G_BM + 3 * G_BN) * BK;  // elements, 64 KiB
+
+__global__ __launch_bounds__(G_NT, 2) void gate_fwd_wide_kernel(const uint16_t* __restrict__ x,
+                                                                const uint16_t* __restrict__ ws,
+                                                                const float* __restrict__ bias,
+                                                                float* __restrict__ out, int T, int D, int E,
+                                                                int k_per_split) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = (wave >> 2) * 64, wn = (wave & 3) * 32;
+  const int t0 = blockIdx.x * G_BM, n0 = blockIdx.y * G_BN;
+  const int k_begin = blockIdx.z * k_per_split;
+  const int ksteps = min(k_per_split, D - k_begin) / BK;
+  const int row = tid >> 3, chunk = tid & 7;  // 64 rows per pass
+  const int64_t ED = static_cast<int64_t>(E) * D;
+  const uint16_t* ap[2];
+  const uint16_t* bp[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    ap[i] = x + static_cast<int64_t>(min(t0 + row + 64 * i, T - 1)) * D + k_begin + chunk * 8;
+    bp[i] = ws + static_cast<int64_t>(min(n0 + row + 64 * i, E - 1)) * D + k_begin + chunk * 8;
+  }
+  const int lds0 = kc_off(row, chunk);  // + 64 rows * BK per pass (64 % 16 == 0: same swizzle key)
+  u32x4 ra[2], rb[6];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) ra[i] = *reinterpret_cast<const u32x4*>(ap[i] + k0);
+#pragma unroll
+    for (int p = 0; p < 3; ++p)
+#pragma unroll
+      for (int i = 0; i < 2; ++i) rb[p * 2 + i] = *reinterpret_cast<const u32x4*>(bp[i] + p * ED + k0);
+  };
+  auto park = [&](uint16_t* st) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) *reinterpret_cast<u32x4*>(st + 64 * i * BK + lds0) = ra[i];
+#pragma unroll
+    for (int p = 0; p < 3; ++p)
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        *reinterpret_cast<u32x4*>(st + (G_BM + p * G_BN + 64 * i) * BK + lds0) = rb[p * 2 + i];
+  };
+  f32x16 acc[2];
+#pragma unroll
+  for (int m = 0; m < 2; ++m)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[m][i] = 0.0f;
+  if (ksteps > 0) {
+    fetch(0);
+    park(smem);
+    if (ksteps > 1) fetch(BK);
+  }
+  __syncthreads();
+  for (int ks = 0; ks < ksteps; ++ks) {
+    const uint16_t* As = smem + (ks & 1) * G_STAGE;
+    if (ks + 1 < ksteps) park(smem + ((ks + 1) & 1) * G_STAGE);
+    if (ks + 2 < ksteps) fetch((ks + 2) * BK);
+#pragma unroll
+    for (int kk = 0; kk < BK / 16; ++kk) {
+      bf16x8 af[2];
+#pragma unroll
+      for (int m = 0; m < 2; ++m) af[m] = frag_kc(As, wm + m * 32, kk, lane);
+#pragma unroll
+      for (int p = 0; p < 3; ++p) {
+        const bf16x8 bf = frag_kc(As + (G_BM + p * G_BN) * BK, wn, kk, lane);
+#pragma unroll
+        for (int m = 0; m < 2; ++m) acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf, af[m], acc[m], 0, 0, 0);
+      }
+    }
+    __syncthreads();
+  }
+  // lane = token row (lane & 31); registers = expert columns (i>>2)*8 + (lane>>5)*4 + (i&3)
+  float* dst = out + static_cast<int64_t>(blockIdx.z) * T * E;
+  const bool direct = gridDim.z == 1;
+#pragma unroll
+  for (int m = 0; m < 2; ++m) {
+    const int t = t0 + wm + m * 32 + (lane & 31);
+    if (t >= T) continue;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int n = n0 + wn + q * 8 + (lane >> 5) * 4;
+      if (n < E) {  // E % 4 == 0
+        f32x4 v = {acc[m][q * 4], acc[m][q * 4 + 1], acc[m][q * 4 + 2], acc[m][q * 4 + 3]};
+        if (direct && bias) v += *reinterpret_cast<const f32x4*>(bias + n);
+        *reinterpret_cast<f32x4*>(dst + static_cast<int64_t>(t) * E + n) = v;
+      }
+    }
+  }
+}
+
+// logits[t][e] = sum over the splits, in order, of partial[z][t][e], plus bias[e]
+__global__ __launch_bounds__(256) void logits_reduce_kernel(const float* __restrict__ partial,
+                                                            const float* __restrict__ bias,
+                                                            float* __restrict__ logits, int64_t TE, int E,
+                                                            int splits) {
+  const int64_t i = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
+  if (i >= TE) return;  // E % 4 == 0: a group of four never straddles a row
+  f32x4 acc = *reinterpret_cast<const f32x4*>(partial + i);
+  for (int z = 1; z < splits; ++z) acc += *reinterpret_cast<const f32x4*>(partial + z * TE + i);
+  if (bias) acc += *reinterpret_cast<const f32x4*>(bias + i % E);
+  *reinterpret_cast<f32x4*>(logits + i) = acc;
+}
+
 // ---- dx(T,D) = dlogits(T,E) . W(E,D), bf16 out ------------------------------------------
 // Tile 128 tokens x 128 columns, 8 waves as 2 x 4, each 64 x 32.  Per K step of 64
 // experts: dlogits tile split on the fly into hi / mid (KC), W hi / mid tiles KS.
@@ -291,6 +400,17 @@ int set_dyn_lds(K kernel, int bytes) {
 }
 
 constexpr int F_LDS = 2 * F_STAGE * 2;                         // 106496
+constexpr int G_LDS = 2 * G_STAGE * 2;                         // 131072
+
+// Splits of the contraction for the 128-token forward kernel: enough workgroups for the chip,
+// at least four K steps each, whole K steps.  0 = use the 32-token kernel (few tokens).
+int fwd_splits(int64_t T, int64_t D, int64_t E) {
+  if (T < 1024) return 0;
+  const int64_t tiles = ((T + G_BM - 1) / G_BM) * ((E + G_BN - 1) / G_BN);
+  int64_t s = 1;
+  while (s < 8 && tiles * s < 256 && D % (2 * s * BK) == 0 && D / (2 * s) >= 4 * BK) s *= 2;
+  return static_cast<int>(s);
+}
 constexpr int X_LDS = (2 * X_BM * BK + 2 * BK * X_BN) * 2;     // 65536
 constexpr int W_LDS = (3 * BK * W_BM + BK * W_BN) * 2;         // 65536
 
@@ -309,7 +429,10 @@ bool router_x3_ok(int x_dtype, int w_dtype, int64_t D, int64_t E) {
   return x_dtype == MI355_BF16 && w_dtype == MI355_F32 && D % 64 == 0 && E % 64 == 0 && D >= 128;
 }
 
-int64_t router_x3_fwd_workspace(int64_t D, int64_t E) { return 3 * E * D * 2; }
+int64_t router_x3_fwd_workspace(int64_t T, int64_t D, int64_t E) {
+  const int s = fwd_splits(T, D, E);
+  return 3 * E * D * 2 + (s > 1 ? static_cast<int64_t>(s) * T * E * 4 : 0);
+}
 
 int64_t router_x3_bwd_workspace(int64_t T, int64_t D, int64_t E) {
   return 2 * E * D * 2 + static_cast<int64_t>(dw_splits(T, D, E)) * E * D * 4;
@@ -325,6 +448,23 @@ int router_x3_fwd(const void* x, const float* w, const float* bias, float* logit
   uint16_t* ws = static_cast<uint16_t*>(workspace);
   const int64_t n = E * D;
   hipLaunchKernelGGL(split_kernel, dim3((unsigned)((n / 8 + 255) / 256)), dim3(256), 0, s, w, ws, n, 3);
+  if (const int splits = fwd_splits(T, D, E)) {
+    static PerDeviceOnce wide_configured;
+    if (wide_configured.needed()) {
+      if (int rc = set_dyn_lds(gate_fwd_wide_kernel, G_LDS)) return rc;
+      wide_configured.done();
+    }
+    float* partial = reinterpret_cast<float*>(ws + 3 * n);  // behind the weight pieces
+    const dim3 grid((unsigned)((T + G_BM - 1) / G_BM), (unsigned)((E + G_BN - 1) / G_BN), (unsigned)splits);
+    hipLaunchKernelGGL(gate_fwd_wide_kernel, grid, dim3(G_NT), G_LDS, s, static_cast<const uint16_t*>(x), ws, bias,
+                       splits > 1 ? partial : logits, (int)T, (int)D, (int)E, (int)(D / splits));
+    if (splits > 1) {
+      const int64_t te = T * E;
+      hipLaunchKernelGGL(logits_reduce_kernel, dim3((unsigned)((te / 4 + 255) / 256)), dim3(256), 0, s, partial, bias,
+                         logits, te, (int)E, splits);
+    }
+    return check_launch("router_gate_fwd");
+  }
   hipLaunchKernelGGL(gate_fwd_kernel, dim3((unsigned)((T + F_BM - 1) / F_BM), (unsigned)((E + F_BN - 1) / F_BN)),
                      dim3(F_NT), F_LDS, s, static_cast<const uint16_t*>(x), ws, bias, logits, (int)T, (int)D, (int)E);
   return check_launch("router_gate_fwd");
