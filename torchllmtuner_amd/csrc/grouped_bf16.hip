@@ -70,6 +70,9 @@ __device__ __forceinline__ float fast_sigmoid(float x) {
   return __builtin_amdgcn_rcpf(1.0f + __expf(-x));
 }
 
+// int32 data that no kernel of this file writes (the plan's arrays), for uniform lookups
+typedef const int32_t __attribute__((address_space(4))) * const_i32;
+
 enum RowMode { RM_GATEUP = 0, RM_DOWN = 1, RM_DH = 2, RM_DX = 3 };
 
 struct RowArgs {
@@ -142,9 +145,12 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
     const int pid = pid_base + w;
     const int tile = pid / p.n_tiles, nt = pid % p.n_tiles;
     TileMeta m;
-    m.e = p.tile_expert[tile];
-    m.row0 = p.tile_row0[tile];
-    m.valid = min(TBM, p.seg_offsets[m.e] + p.seg_counts[m.e] - m.row0);
+    // scalar loads (constant address space): as vector loads these lookups would share the
+    // counter of the operand stream and of the epilogue stores, and waiting for one of them
+    // would wait for all of those
+    m.e = ((const_i32)p.tile_expert)[tile];
+    m.row0 = ((const_i32)p.tile_row0)[tile];
+    m.valid = min(TBM, ((const_i32)p.seg_offsets)[m.e] + ((const_i32)p.seg_counts)[m.e] - m.row0);
     // a last tile that would overhang starts early instead and recomputes a few columns
     // of its neighbour (same values), so no column is ever clamped
     constexpr int W = (MODE == RM_GATEUP ? BNT / 2 : BNT);
@@ -400,9 +406,9 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
       for (int it = 0; it < 12; ++it) {
         const int idx = it * 64 + lane;
         const int m = idx / 24, rem = idx % 24, t = rem >> 3, c = rem & 7;
-        const int f = f0 + c * 8;
+        const int f = f0 + c * 8;  // < F: tiles never overhang in the columns
         const int mr = wm + half * 32 + m;
-        if (mr < valid && f < F) {
+        if (mr < valid) {
           const u32x4 v = *reinterpret_cast<const u32x4*>(sg + m * S::PITCH + t * 64 + c * 8);
           uint16_t* dst = (t == 0 ? p.o0 : (t == 1 ? p.o1 : p.o2)) + static_cast<int64_t>(row0 + mr) * F + f;
           *reinterpret_cast<u32x4*>(dst) = v;
@@ -422,19 +428,53 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
     __builtin_amdgcn_s_waitcnt(0xc07f);
     __builtin_amdgcn_wave_barrier();
     const int c0 = n0 + wn * (32 * NJ);
-    // 64 rows x CH chunks, CH per lane; a row's bytes go out contiguously
-#pragma unroll 4
-    for (int it = 0; it < CH; ++it) {
+    // 64 rows x CH chunks, CH per lane; a row's bytes go out contiguously; tiles never
+    // overhang in the columns.  Where the epilogue also LOADS (dH), lanes whose row lies past
+    // the tile's real rows redo the last real row instead (the same bytes to the same
+    // address), so that every load and store is unconditional: the compiler then knows how
+    // many are in flight and waits for exactly the ones it needs -- with predicated accesses
+    // every wait drains the whole queue, stores included (one counter serves both here).
+    const int last = valid - 1 - wm;  // >= 0 in this branch
+    auto chunk_at = [&](int it, int& m, int& c) {
       const int idx = it * 64 + lane;
-      const int m = idx / CH, c = idx % CH;
-      const int n = c0 + c * 8;
-      if (wm + m < valid && n < Ncols) {
-        const u32x4 v = *reinterpret_cast<const u32x4*>(st + m * S::PITCH + c * 8);
-        const int64_t o = static_cast<int64_t>(row0 + wm + m) * Ncols + n;
-        if constexpr (MODE == RM_DH) {
-          // SwiGLU backward on 8 consecutive f: dgate = dh*up*silu'(gate), dup = dh*silu(gate)
-          const u32x4 gv = *reinterpret_cast<const u32x4*>(p.gate + o);
-          const u32x4 uv = *reinterpret_cast<const u32x4*>(p.up + o);
+      m = min(idx / CH, last);
+      c = idx % CH;
+    };
+    auto offset_at = [&](int it) -> int64_t {
+      int m, c;
+      chunk_at(it, m, c);
+      return static_cast<int64_t>(row0 + wm + m) * Ncols + c0 + c * 8;
+    };
+    if constexpr (MODE == RM_DH) {
+      // SwiGLU backward on 8 consecutive f: dgate = dh*up*silu'(gate), dup = dh*silu(gate).
+      // gate and up of the next four chunks are requested before the current four are stored:
+      // a load issued behind a store cannot complete before it.
+      constexpr int G = 4;
+      static_assert(CH % G == 0, "chunks per row come in groups of four");
+      u32x4 gq[G], uq[G];
+#pragma unroll
+      for (int u = 0; u < G; ++u) {
+        const int64_t o = offset_at(u);
+        gq[u] = *reinterpret_cast<const u32x4*>(p.gate + o);
+        uq[u] = *reinterpret_cast<const u32x4*>(p.up + o);
+      }
+#pragma unroll
+      for (int g0 = 0; g0 < CH; g0 += G) {
+        u32x4 gn[G], un[G];
+        if (g0 + G < CH) {
+#pragma unroll
+          for (int u = 0; u < G; ++u) {
+            const int64_t o = offset_at(g0 + G + u);
+            gn[u] = *reinterpret_cast<const u32x4*>(p.gate + o);
+            un[u] = *reinterpret_cast<const u32x4*>(p.up + o);
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < G; ++u) {
+          int m, c;
+          chunk_at(g0 + u, m, c);
+          const u32x4 v = *reinterpret_cast<const u32x4*>(st + m * S::PITCH + c * 8);
+          const u32x4 gv = gq[u], uv = uq[u];
           u32x4 dg, du;
 #pragma unroll
           for (int w = 0; w < 4; ++w) {
@@ -443,21 +483,37 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
             for (int hlf = 0; hlf < 2; ++hlf) {
               const float dh = __uint_as_float(hlf ? (v[w] & 0xffff0000u) : (v[w] << 16));
               const float g = __uint_as_float(hlf ? (gv[w] & 0xffff0000u) : (gv[w] << 16));
-              const float u = __uint_as_float(hlf ? (uv[w] & 0xffff0000u) : (uv[w] << 16));
+              const float uu = __uint_as_float(hlf ? (uv[w] & 0xffff0000u) : (uv[w] << 16));
               const float sig = fast_sigmoid(g);
-              const float s = round_bf16(g * sig);
-              const float ds = round_bf16(dh * u);
-              r_du[hlf] = dh * s;
+              const float sl = round_bf16(g * sig);
+              const float ds = round_bf16(dh * uu);
+              r_du[hlf] = dh * sl;
               r_dg[hlf] = ds * (sig * (1.0f + g * (1.0f - sig)));
             }
             dg[w] = pack2(r_dg[0], r_dg[1]);
             du[w] = pack2(r_du[0], r_du[1]);
           }
+          const int64_t o = offset_at(g0 + u);
           *reinterpret_cast<u32x4*>(p.o0 + o) = dg;
           *reinterpret_cast<u32x4*>(p.o1 + o) = du;
-        } else {
-          *reinterpret_cast<u32x4*>(p.o0 + o) = v;
         }
+        if (g0 + G < CH) {
+#pragma unroll
+          for (int u = 0; u < G; ++u) {
+            gq[u] = gn[u];
+            uq[u] = un[u];
+          }
+        }
+      }
+    } else {
+      // plain copies: predicated (a partly empty tile then writes less; measured faster here)
+#pragma unroll 4
+      for (int it = 0; it < CH; ++it) {
+        const int idx = it * 64 + lane;
+        const int m = idx / CH, c = idx % CH;
+        if (m <= last)
+          *reinterpret_cast<u32x4*>(p.o0 + static_cast<int64_t>(row0 + wm + m) * Ncols + c0 + c * 8) =
+              *reinterpret_cast<const u32x4*>(st + m * S::PITCH + c * 8);
       }
     }
   }
@@ -521,7 +577,13 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
   // before its data.
   const int El = p.El;
   const int xcd = blockIdx.x & 7;
-  const int32_t* order = p.seg_counts + El;
+  // The plan arrays are read-only here and every lookup is workgroup-uniform: read through
+  // the constant address space they are scalar loads.  As vector loads (what the compiler
+  // makes of them inside this loop) each lookup would share the counter of the operand
+  // stream and of the epilogue stores, and waiting for it would wait for all of those.
+  const const_i32 order = (const_i32)(p.seg_counts + El);
+  const const_i32 seg_offsets = (const_i32)p.seg_offsets;
+  const const_i32 seg_counts = (const_i32)p.seg_counts;
   // Whole experts are dealt in rounds of eight, each round in the opposite direction of the
   // one before (so no XCD always gets the larger expert of its round); the El % 8 smallest
   // experts left over are cut into eight equal contiguous runs of tiles instead.
@@ -548,8 +610,11 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
 
   // state of the tile whose operands are being fetched
   int e = expert_of(within);
-  int m0 = (tile_in_expert(within) / p.n_tiles) * WBM, n0 = (tile_in_expert(within) % p.n_tiles) * WBN;
-  int seg0 = p.seg_offsets[e], cnt = p.seg_counts[e];
+  // a last tile that would overhang starts early instead (M, N >= 256) and recomputes a few
+  // rows or columns of its neighbour -- the same values -- so every tile is whole
+  int m0 = min((tile_in_expert(within) / p.n_tiles) * WBM, M - WBM);
+  int n0 = min((tile_in_expert(within) % p.n_tiles) * WBN, N - WBN);
+  int seg0 = seg_offsets[e], cnt = seg_counts[e];
   const uint16_t* a_base;
   const uint16_t* b_base;
   auto set_bases = [&]() {
@@ -585,14 +650,14 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
   // expert and segment of the next tile, expert of the one after it (its segment is
   // looked up inside the loop, the expert after that too)
   int ne = expert_of(within + stride);
-  int nseg0 = p.seg_offsets[ne], ncnt = p.seg_counts[ne];
+  int nseg0 = seg_offsets[ne], ncnt = seg_counts[ne];
   int e2 = expert_of(within + 2 * stride);
 
   for (;;) {
     const bool more = exists(within + stride);
     const int nw = within + stride;
     // two tiles ahead: segment bounds, used one tile later; three ahead: the expert
-    const int n2seg0 = p.seg_offsets[e2], n2cnt = p.seg_counts[e2];
+    const int n2seg0 = seg_offsets[e2], n2cnt = seg_counts[e2];
     const int e3 = expert_of(within + 3 * stride);
     // next tile: B rows of its first K step (its bounds were looked up a tile ago)
     int nidx[4];
@@ -666,8 +731,8 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
     if (more) {
       e = ne;
       const int nt = tile_in_expert(nw);
-      m0 = (nt / p.n_tiles) * WBM;
-      n0 = (nt % p.n_tiles) * WBN;
+      m0 = min((nt / p.n_tiles) * WBM, M - WBM);
+      n0 = min((nt % p.n_tiles) * WBN, N - WBN);
       seg0 = nseg0;
       cnt = ncnt;
       set_bases();
@@ -696,9 +761,11 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
     for (int it = 0; it < 16; ++it) {
       const int idx = it * 64 + lane;
       const int m = c_m0 + wm + (idx >> 4), n = c_n0 + wn + (idx & 15) * 8;
-      if (m < M && n < N)
-        *reinterpret_cast<u32x4*>(C + static_cast<int64_t>(m) * N + n) =
-            *reinterpret_cast<const u32x4*>(st + (idx >> 4) * S::PITCH + (idx & 15) * 8);
+      // whole tiles only: the stores are unconditional, so the compiler knows how many follow
+      // the operand loads requested above and the next tile's wait for those loads does not
+      // also wait for these stores (one counter serves both)
+      *reinterpret_cast<u32x4*>(C + static_cast<int64_t>(m) * N + n) =
+          *reinterpret_cast<const u32x4*>(st + (idx >> 4) * S::PITCH + (idx & 15) * 8);
     }
     // staging regions are free again before the next tile's operands are parked; only
     // the LDS traffic is waited for, the tile's stores keep draining
