@@ -1,7 +1,7 @@
 // Token permutation: the expert-major plan and the row movers.
 //
 // Plan = a stable counting sort of the N = T*K assignment slots by expert id.
-//   1. plan_rank    each wave walks 512 consecutive slots in 64-slot chunks; within
+//   1. plan_rank    each wave walks 256 consecutive slots in 64-slot chunks; within
 //                   a chunk a slot's rank among equal experts is counted with 64
 //                   lane reads, and the running per-wave expert counts live in LDS
 //                   (one writer per expert and chunk).  Emits the rank of every
@@ -17,9 +17,10 @@
 namespace mi355 {
 namespace {
 
-constexpr int kSlotsPerWave = 512;
+constexpr int kSlotsPerWave = 256;
 constexpr int kWavesPerBlock = 4;
 constexpr int kSlotsPerBlock = kSlotsPerWave * kWavesPerBlock;
+constexpr int kBatch = 16;  // histogram loads in flight per lane in the scan
 
 __global__ __launch_bounds__(256) void plan_rank_kernel(const int64_t* __restrict__ ids, int N,
                                                         int E, int32_t* __restrict__ rank_in_wave,
@@ -74,14 +75,25 @@ __global__ __launch_bounds__(1024) void plan_scan_kernel(
   int32_t* cnt_sh = part_sum + parts * E;  // E
   int32_t* seg_off_sh = cnt_sh + E;        // El + 1
   int32_t* tile_off_sh = seg_off_sh + El + 1;  // El + 1
+  int32_t* pad_sh = tile_off_sh + El + 1;      // El
+  int32_t* nt_sh = pad_sh + El;                // El
   const int tid = threadIdx.x;
   const int per = (num_waves + parts - 1) / parts;
 
   for (int idx = tid; idx < E * parts; idx += blockDim.x) {
     const int e = idx % E, part = idx / E;
     const int w0 = part * per, w1 = min(num_waves, w0 + per);
-    int sum = 0;
-    for (int w = w0; w < w1; ++w) sum += wave_hist[static_cast<int64_t>(w) * E + e];
+    // sixteen loads in flight at a time: one at a time, each would wait out a full memory
+    // round trip, and this workgroup has nothing else to hide it behind
+    int sum = 0, w = w0;
+    for (; w + kBatch <= w1; w += kBatch) {
+      int v[kBatch];
+#pragma unroll
+      for (int i = 0; i < kBatch; ++i) v[i] = wave_hist[static_cast<int64_t>(w + i) * E + e];
+#pragma unroll
+      for (int i = 0; i < kBatch; ++i) sum += v[i];
+    }
+    for (; w < w1; ++w) sum += wave_hist[static_cast<int64_t>(w) * E + e];
     part_sum[part * E + e] = sum;
   }
   __syncthreads();
@@ -100,39 +112,51 @@ __global__ __launch_bounds__(1024) void plan_scan_kernel(
   for (int idx = tid; idx < E * parts; idx += blockDim.x) {
     const int e = idx % E, part = idx / E;
     const int w0 = part * per, w1 = min(num_waves, w0 + per);
-    int run = part_sum[part * E + e];
-    for (int w = w0; w < w1; ++w) {
+    int run = part_sum[part * E + e], w = w0;
+    for (; w + kBatch <= w1; w += kBatch) {
+      int v[kBatch];
+#pragma unroll
+      for (int i = 0; i < kBatch; ++i) v[i] = wave_hist[static_cast<int64_t>(w + i) * E + e];
+#pragma unroll
+      for (int i = 0; i < kBatch; ++i) {
+        wave_prefix[static_cast<int64_t>(w + i) * E + e] = run;
+        run += v[i];
+      }
+    }
+    for (; w < w1; ++w) {
       const int64_t i = static_cast<int64_t>(w) * E + e;
       wave_prefix[i] = run;
       run += wave_hist[i];
     }
   }
-  if (tid == 0) {
-    // El is at most a few hundred: a serial scan by one lane costs about a microsecond.
-    int off = 0, toff = 0;
-    for (int j = 0; j < El; ++j) {
-      const int c = cnt_sh[lo + j];
-      seg_off_sh[j] = off;
-      tile_off_sh[j] = toff;
-      off += c + ((align - (c % align)) % align);
-      toff += (c + tile_m - 1) / tile_m;
-    }
-    seg_off_sh[El] = off;
-    tile_off_sh[El] = toff;
-    *num_tiles = toff < tile_capacity ? toff : tile_capacity;
-  }
-  __syncthreads();
-  // local experts by descending row count (ties to the lower index): the order in which the
-  // weight-gradient kernels start their tiles, longest contraction first
+  // padded rows and tiles per local expert, then every lane sums what lies before its
+  // expert: El broadcast LDS reads per lane, no serial chain (a one-lane scan with its two
+  // integer divisions per expert took longer than everything else in this kernel)
   for (int j = tid; j < El; j += blockDim.x) {
     const int c = cnt_sh[lo + j];
-    int rank = 0;
-    for (int o = 0; o < El; ++o) {
-      const int co = cnt_sh[lo + o];
-      rank += (co > c || (co == c && o < j)) ? 1 : 0;
-    }
-    seg_counts[El + rank] = j;
+    pad_sh[j] = c + ((align - (c % align)) % align);
+    nt_sh[j] = (c + tile_m - 1) / tile_m;
   }
+  __syncthreads();
+  // ... and its place among the local experts by descending row count (ties to the lower
+  // index): the order in which the weight-gradient kernels start their tiles, longest
+  // contraction first
+  for (int j = tid; j <= El; j += blockDim.x) {
+    const int c = j < El ? cnt_sh[lo + j] : 0;
+    int off = 0, toff = 0, rank = 0;
+    for (int o = 0; o < El; ++o) {
+      const bool before = o < j;
+      off += before ? pad_sh[o] : 0;
+      toff += before ? nt_sh[o] : 0;
+      const int co = cnt_sh[lo + o];
+      rank += (co > c || (co == c && before)) ? 1 : 0;
+    }
+    seg_off_sh[j] = off;
+    tile_off_sh[j] = toff;
+    if (j < El) seg_counts[El + rank] = j;
+    else *num_tiles = toff < tile_capacity ? toff : tile_capacity;
+  }
+  __syncthreads();
   for (int j = tid; j <= El; j += blockDim.x) seg_offsets[j] = seg_off_sh[j];
   for (int j = tid; j < El; j += blockDim.x) {
     const int c = cnt_sh[lo + j];
@@ -158,34 +182,37 @@ __global__ __launch_bounds__(256) void segments_from_counts_kernel(
   int32_t* seg_off_sh = sh;
   int32_t* tile_off_sh = sh + El + 1;
   int32_t* cnt_sh = sh + 2 * El + 2;
+  int32_t* raw_sh = cnt_sh + El;
   const int tid = threadIdx.x;
-  if (tid == 0) {
-    int off = 0, toff = 0;
-    for (int j = 0; j < El; ++j) {
-      // clamp so that no segment reaches past the rows that exist
-      const int c = min(max(counts[j], 0), row_capacity - off);
-      cnt_sh[j] = c;
-      seg_off_sh[j] = off;
-      tile_off_sh[j] = toff;
-      off += c;
-      toff += (c + tile_m - 1) / tile_m;
-    }
-    seg_off_sh[El] = off;
-    tile_off_sh[El] = toff;
-    *num_tiles = toff < tile_capacity ? toff : tile_capacity;
+  // Clamped so that no segment reaches past the rows that exist: the offset of expert j is
+  // min(sum of the counts before it, row_capacity) and it keeps what still fits -- what a
+  // serial walk would give, computed by every lane for its own expert.
+  for (int j = tid; j < El; j += blockDim.x) raw_sh[j] = max(counts[j], 0);
+  __syncthreads();
+  for (int j = tid; j <= El; j += blockDim.x) {
+    int64_t before = 0;
+    for (int o = 0; o < j; ++o) before += raw_sh[o];
+    const int off = static_cast<int>(min(before, static_cast<int64_t>(row_capacity)));
+    seg_off_sh[j] = off;
+    if (j < El) cnt_sh[j] = min(raw_sh[j], row_capacity - off);
   }
   __syncthreads();
-  // local experts by descending row count (ties to the lower index): the order in which the
-  // weight-gradient kernels start their tiles, longest contraction first
-  for (int j = tid; j < El; j += blockDim.x) {
-    const int c = cnt_sh[j];
-    int rank = 0;
+  // tiles before each expert, and the experts by descending row count (ties to the lower
+  // index): the order in which the weight-gradient kernels start their tiles
+  for (int j = tid; j <= El; j += blockDim.x) {
+    const int c = j < El ? cnt_sh[j] : 0;
+    int toff = 0, rank = 0;
     for (int o = 0; o < El; ++o) {
       const int co = cnt_sh[o];
-      rank += (co > c || (co == c && o < j)) ? 1 : 0;
+      const bool before = o < j;
+      toff += before ? (co + tile_m - 1) / tile_m : 0;
+      rank += (co > c || (co == c && before)) ? 1 : 0;
     }
-    seg_counts[El + rank] = j;
+    tile_off_sh[j] = toff;
+    if (j < El) seg_counts[El + rank] = j;
+    else *num_tiles = toff < tile_capacity ? toff : tile_capacity;
   }
+  __syncthreads();
   for (int j = tid; j <= El; j += blockDim.x) seg_offsets[j] = seg_off_sh[j];
   for (int j = tid; j < El; j += blockDim.x) {
     const int c = cnt_sh[j];
@@ -201,9 +228,13 @@ __global__ __launch_bounds__(256) void segments_from_counts_kernel(
   }
 }
 
-__global__ void fill_i32_kernel(int32_t* p, int64_t n, int32_t v) {
+// p[0..n) = v, and q[0..n) too when q is given
+__global__ void fill_i32_kernel(int32_t* p, int32_t* q, int64_t n, int32_t v) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (i < n) p[i] = v;
+  if (i < n) {
+    p[i] = v;
+    if (q) q[i] = v;
+  }
 }
 
 __global__ __launch_bounds__(256) void plan_rows_kernel(
@@ -369,13 +400,8 @@ extern "C" int mi355_permute_plan(const int64_t* ids, int64_t T, int64_t K, int6
   }
   if (row_capacity > 0) {
     hipLaunchKernelGGL(fill_i32_kernel, dim3((unsigned)((row_capacity + 255) / 256)), dim3(256), 0, s,
-                       slot_of_row, row_capacity, -1);
+                       slot_of_row, token_of_row, row_capacity, -1);
     if (int rc = check_launch("plan_fill")) return rc;
-    if (token_of_row) {
-      hipLaunchKernelGGL(fill_i32_kernel, dim3((unsigned)((row_capacity + 255) / 256)), dim3(256), 0, s,
-                         token_of_row, row_capacity, -1);
-      if (int rc = check_launch("plan_fill")) return rc;
-    }
   }
   const int El = (int)(hi - lo);
   int32_t* wave_prefix = wave_hist + (int64_t)nwaves * E;
@@ -383,7 +409,7 @@ extern "C" int mi355_permute_plan(const int64_t* ids, int64_t T, int64_t K, int6
   if (parts < 1) parts = 1;
   if (parts > 16) parts = 16;
   hipLaunchKernelGGL(plan_scan_kernel, dim3(1), dim3(1024),
-                     (size_t)((parts + 1) * E + 2 * El + 2) * 4, s, wave_hist, wave_prefix, nwaves,
+                     (size_t)((parts + 1) * E + 4 * El + 2) * 4, s, wave_hist, wave_prefix, nwaves,
                      (int)E, (int)lo, (int)hi, (int)align, (int)tile_m, counts_E, seg_offsets,
                      seg_counts, tile_expert, tile_row0, num_tiles, (int)tile_capacity, parts);
   if (int rc = check_launch("plan_scan")) return rc;
@@ -447,7 +473,7 @@ extern "C" int mi355_segments_from_counts(const int32_t* counts, int64_t El, int
                 "segments_from_counts: bad shape El=%lld", (long long)El);
   MI355_REQUIRE(counts && seg_offsets && seg_counts && num_tiles, "segments_from_counts: null pointer");
   MI355_REQUIRE(tile_capacity == 0 || (tile_expert && tile_row0), "segments_from_counts: null tile list");
-  hipLaunchKernelGGL(segments_from_counts_kernel, dim3(1), dim3(256), (size_t)(3 * El + 2) * 4,
+  hipLaunchKernelGGL(segments_from_counts_kernel, dim3(1), dim3(256), (size_t)(4 * El + 2) * 4,
                      as_stream(stream), counts, (int)El, (int)tile_m, (int)row_capacity, seg_offsets, seg_counts,
                      tile_expert, tile_row0, num_tiles, (int)tile_capacity);
   return check_launch("segments_from_counts");

@@ -10,6 +10,9 @@
 //   dx     = dlogits . W        rounded to bf16 on output, so hi.hi + hi.mid + mid.hi
 //                               (relative error 2^-16) is enough
 // Shapes: D and E multiples of 64; anything else stays on the strided fp32-MFMA kernels.
+#include <algorithm>
+#include <cstdint>
+
 #include "bf16_tiles.h"
 #include "common.h"
 #include "gemm_generic.h"
@@ -414,13 +417,22 @@ int fwd_splits(int64_t T, int64_t D, int64_t E) {
 constexpr int X_LDS = (2 * X_BM * BK + 2 * BK * X_BN) * 2;     // 65536
 constexpr int W_LDS = (3 * BK * W_BM + BK * W_BN) * 2;         // 65536
 
+// Splits of the token contraction for dW.  Two workgroups fit a CU, so the launch runs in
+// rounds of 512 and its length goes as rounds x tokens per split: one more split than fills a
+// round costs a whole extra round.  Each split also adds an (E, D) fp32 partial for the
+// reduction to read, priced here at twelve token rows of the kernel (measured: the sum is
+// within a few percent of the best split count at 8192 x 2048 x 128, 16384 x 2048 x 128 and
+// 4096 x 7168 x 256).  At least four K steps per split.
 int dw_splits(int64_t T, int64_t D, int64_t E) {
   const int64_t tiles = ((D + W_BN - 1) / W_BN) * ((E + W_BM - 1) / W_BM);
-  int64_t s = (512 + tiles - 1) / tiles;
-  const int64_t max_s = (T + 4 * BK - 1) / (4 * BK);  // at least four K steps per split
-  if (s > max_s) s = max_s;
-  if (s < 1) s = 1;
-  return static_cast<int>(s);
+  const int64_t max_s = std::max<int64_t>(1, std::min<int64_t>(64, (T + 4 * BK - 1) / (4 * BK)));
+  int64_t best = 1, best_cost = INT64_MAX;
+  for (int64_t s = 1; s <= max_s; ++s) {
+    const int64_t rows = ((T + s - 1) / s + BK - 1) / BK * BK;
+    const int64_t cost = ((tiles * s + 511) / 512) * rows + 12 * s;
+    if (cost < best_cost) { best = s; best_cost = cost; }
+  }
+  return static_cast<int>(best);
 }
 
 }  // namespace
