@@ -342,6 +342,48 @@ int mi355_grouped_swiglu_bwd(const void* dy, const void* rows,
                              int64_t row_capacity, void* stream);
 
 /*
+ * The backward of "experts, then combine" as one call, for the case the layer actually
+ * runs: out[t] = sum_k weights[t][k] * y[row(t,k)] with y from mi355_grouped_swiglu_fwd
+ * called with token_of_row (x = the (T,D) token matrix).  It computes what
+ * mi355_combine_bwd followed by mi355_grouped_swiglu_bwd compute (the autograd-derived
+ * backward of GroupedExperts.forward, experts.py:204-209 and :211-285, and of
+ * LocalTokenDispatcher.combine, token_dispatch.py:255-275) without ever writing the
+ * expert-major gradient dy = weights * dout or reading y:
+ *   dh[r]   = row_scale[r] * (dout[token_of_row[r]] . w2[e])     (scaled in the epilogue)
+ *   hs[r]   = row_scale[r] * h[r],  h recomputed from gate and up (h need not be kept)
+ *   dw2[e]  = dout[token_of_row]_e^T . hs_e
+ *   dot_partial[r][j] = sum over the j-th 128 columns f of (dout[token_of_row[r]] . w2[e])[f] * h[r][f]
+ * and dgate, dup, drows, dw1, dw3 as in mi355_grouped_swiglu_bwd.  The gradient of
+ * weights[t][k] is the sum over j of dot_partial[row(t,k)][j] (mi355_combine_scores_bwd).
+ * Two bf16 roundings move compared with the two-call form (dh is rounded once, after the
+ * scaling, instead of dy and dh each; dW2 rounds weights*h instead of weights*dout); both
+ * stay inside the bf16 tolerance of the path.
+ * bf16 only, D and F multiples of 64 and >= 384, 256-row tile layout:
+ * mi355_grouped_combine_bwd_slots returns the number of partials per row (the second
+ * dimension of dot_partial), or 0 when this entry point does not cover the case (then use
+ * the two-call form).  row_scale (row_capacity floats) comes from mi355_combine_row_scale:
+ * row_scale[r] = weights[slot_of_row[r]], 0 for rows that hold padding.
+ * dgate, dup, hs: caller-provided (row_capacity,F) each; dot_partial (row_capacity,slots) fp32.
+ */
+int64_t mi355_grouped_combine_bwd_slots(int dtype, int64_t D, int64_t F);
+int mi355_grouped_swiglu_combine_bwd(const void* dout, const void* x, const int32_t* token_of_row,
+                                     const float* row_scale, const void* w1, const void* w3,
+                                     const void* w2, const void* gate, const void* up, int dtype,
+                                     const int32_t* seg_offsets, const int32_t* seg_counts,
+                                     const int32_t* tile_expert, const int32_t* tile_row0,
+                                     const int32_t* num_tiles, int64_t tile_capacity, void* dgate,
+                                     void* dup, void* hs, float* dot_partial, void* drows,
+                                     void* dw1, void* dw3, void* dw2, int64_t El, int64_t D,
+                                     int64_t F, int64_t row_capacity, void* stream);
+int mi355_combine_row_scale(const float* weights_TK, const int32_t* slot_of_row, float* row_scale,
+                            int64_t T, int64_t K, int64_t row_capacity, void* stream);
+/* dweights[t][k] = sum_j dot_partial[row_of_slot[t*K+k]][j], summed in ascending j; 0 for
+ * slots without a row. */
+int mi355_combine_scores_bwd(const float* dot_partial, int64_t slots, const int32_t* row_of_slot,
+                             float* dweights_TK, int64_t T, int64_t K, int64_t row_capacity,
+                             void* stream);
+
+/*
  * One of the seven bf16 MFMA kernels behind the two calls above, by itself, on the
  * same buffers: for profilers and for callers that schedule the stages themselves.
  * No counterpart in the reference.  bf16 only, D and F multiples of 64.

@@ -342,6 +342,74 @@ def test_balance_loss_fwd_bwd(ops, T, E, K, padded):
     assert torch.equal(grad2, grad * 2)
 
 
+# ------------------------------------------- experts + combine, one backward for both
+@pytest.mark.parametrize("T,K,E,D,Fd,align,local,skew", [
+    (700, 4, 16, 384, 768, 1, None, False),     # F a multiple of the 256-column dH tile
+    (700, 4, 16, 512, 448, 8, None, False),     # last dH tile starts early: shared columns counted once
+    (1500, 8, 32, 384, 384, 1, (8, 24), True),  # local expert range, skewed counts, dropped slots
+    (64, 2, 8, 384, 640, 128, None, False),     # few rows per expert, padded segments
+])
+def test_folded_combine_backward_matches_the_two_call_backward(ops, T, K, E, D, Fd, align, local, skew):
+    """mi355_grouped_swiglu_combine_bwd against mi355_combine_bwd + mi355_grouped_swiglu_bwd on
+    the same inputs (both bf16, two rounding points apart), and both against the fp32 oracle."""
+    print(f"folded combine bwd T={T} K={K} E={E} D={D} F={Fd} align={align} local={local} skew={skew}", flush=True)
+    g = torch.Generator().manual_seed(11)
+    if skew:
+        pr = torch.arange(1, E + 1, dtype=torch.float32) ** -1.2
+        ids = torch.stack([torch.multinomial(pr, K, generator=g) for _ in range(T)])
+    else:
+        ids = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(T)])
+    weights = torch.rand(T, K, generator=g) + 0.05
+    weights = weights / weights.sum(-1, keepdim=True)
+    lo, hi = local if local else (0, E)
+    El = hi - lo
+    x = torch.randn(T, D, generator=g).bfloat16()
+    dout = torch.randn(T, D, generator=g).bfloat16()
+    mk = lambda *s: (torch.randn(*s, generator=g) * 0.05).bfloat16()
+    w1, w3, w2 = mk(El, Fd, D), mk(El, Fd, D), mk(El, D, Fd)
+
+    plan = ops.permute_plan(ids.to(DEV), E, align=align, local_lo=lo, local_hi=hi)
+    assert ops.combine_bwd_slots(torch.bfloat16, D, Fd) > 0
+    xd, wd, dd = x.to(DEV), weights.to(DEV), dout.to(DEV)
+    w1d, w3d, w2d = w1.to(DEV), w3.to(DEV), w2.to(DEV)
+    y, gate, up, h = ops.grouped_swiglu_fwd(xd, w1d, w3d, w2d, plan, gather=True)
+
+    dy, dwt_a = ops.combine_bwd(dd, y, wd, plan)
+    drows_a, dw1_a, dw3_a, dw2_a = ops.grouped_swiglu_bwd(dy, xd, w1d, w3d, w2d, gate, up, h, plan, gather=True)
+    scale = ops.combine_row_scale(wd, plan)
+    drows_b, dw1_b, dw3_b, dw2_b, dwt_b = ops.grouped_swiglu_combine_bwd(dd, xd, scale, w1d, w3d, w2d, gate, up, plan)
+
+    # row_scale is the weights read through the plan, zero where a row holds padding
+    sor = plan.slot_of_row.cpu()
+    want_scale = torch.where(sor >= 0, weights.flatten()[sor.clamp(min=0)], torch.zeros(()))
+    assert torch.equal(scale.cpu(), want_scale)
+
+    dx_a, dx_b = ops.permute_rows_bwd(drows_a, plan), ops.permute_rows_bwd(drows_b, plan)
+    for name, a, b in (("dx", dx_a, dx_b), ("dw1", dw1_a, dw1_b), ("dw3", dw3_a, dw3_b), ("dw2", dw2_a, dw2_b),
+                       ("dweights", dwt_a, dwt_b)):
+        assert rel_l2(b, a) < BF16_TOL, f"{name}: folded vs two calls {rel_l2(b, a)}"
+
+    # the fp32 oracle of the whole thing: out = sum_k w * experts(x)[row], gradients by autograd
+    xr, wr = x.float().requires_grad_(), weights.clone().requires_grad_()
+    p1, p3, p2 = (w.float().requires_grad_() for w in (w1, w3, w2))
+    out = torch.zeros(T, D)
+    flat = ids.flatten()
+    for e in range(lo, hi):
+        sel = (flat == e).nonzero().squeeze(-1)
+        if sel.numel() == 0:
+            continue
+        tok = sel // K
+        hh = F.silu(xr[tok] @ p1[e - lo].T) * (xr[tok] @ p3[e - lo].T)
+        out = out.index_add(0, tok, (hh @ p2[e - lo].T) * wr.flatten()[sel, None])
+    out.backward(dout.float())
+    local_slot = ((ids >= lo) & (ids < hi))
+    for name, got, want in (("dx", dx_b, xr.grad), ("dw1", dw1_b, p1.grad), ("dw3", dw3_b, p3.grad),
+                            ("dw2", dw2_b, p2.grad), ("dweights", dwt_b, wr.grad)):
+        assert rel_l2(got, want) < BF16_TOL, f"{name}: folded vs fp32 oracle {rel_l2(got, want)}"
+    # slots that were dropped (experts outside the local range) get exactly zero
+    assert torch.equal(dwt_b.cpu()[~local_slot], torch.zeros_like(dwt_b.cpu()[~local_slot]))
+
+
 def test_wide_row_tile_layout_in_a_child_process():
     """The 128 x 512 row tile is chosen per process (MI355_ROW_LAYOUT=wide, read when the
     library first launches a grouped kernel), so its parity cases run in a child."""

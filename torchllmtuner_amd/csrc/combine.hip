@@ -223,3 +223,60 @@ extern "C" int mi355_combine_bwd(const void* dout, const void* y, int dtype, con
     return fail(MI355_EINVAL, "combine_bwd: unknown dtype %d", dtype);
   return check_launch("combine_bwd");
 }
+
+// ---- the two small ends of the backward that folds the combine into the expert kernels --
+namespace mi355 {
+namespace {
+
+__global__ __launch_bounds__(256) void row_scale_kernel(const float* __restrict__ weights,
+                                                        const int32_t* __restrict__ slot_of_row,
+                                                        float* __restrict__ row_scale, int rows, int slots) {
+  const int r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= rows) return;
+  const int slot = slot_of_row[r];
+  row_scale[r] = (slot >= 0 && slot < slots) ? weights[slot] : 0.0f;
+}
+
+__global__ __launch_bounds__(256) void scores_bwd_kernel(const float* __restrict__ partial, int pieces,
+                                                         const int32_t* __restrict__ row_of_slot,
+                                                         float* __restrict__ dweights, int slots, int rows) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= slots) return;
+  const int row = row_of_slot[i];
+  float acc = 0.0f;
+  if (row >= 0 && row < rows) {
+    const float* src = partial + static_cast<int64_t>(row) * pieces;
+    for (int s = 0; s < pieces; ++s) acc += src[s];  // fixed order: the same bits every run
+  }
+  dweights[i] = acc;
+}
+
+}  // namespace
+}  // namespace mi355
+
+extern "C" int mi355_combine_row_scale(const float* weights_TK, const int32_t* slot_of_row, float* row_scale,
+                                       int64_t T, int64_t K, int64_t row_capacity, void* stream) {
+  using namespace mi355;
+  MI355_REQUIRE(T >= 0 && K >= 1 && T * K < (1ll << 31) && row_capacity >= 0 && row_capacity < (1ll << 31),
+                "combine_row_scale: bad shape");
+  if (row_capacity == 0) return MI355_OK;
+  MI355_REQUIRE(slot_of_row && row_scale && (weights_TK || T == 0), "combine_row_scale: null pointer");
+  hipLaunchKernelGGL(row_scale_kernel, dim3((unsigned)((row_capacity + 255) / 256)), dim3(256), 0,
+                     as_stream(stream), weights_TK, slot_of_row, row_scale, (int)row_capacity, (int)(T * K));
+  return check_launch("combine_row_scale");
+}
+
+extern "C" int mi355_combine_scores_bwd(const float* dot_partial, int64_t pieces, const int32_t* row_of_slot,
+                                        float* dweights_TK, int64_t T, int64_t K, int64_t row_capacity,
+                                        void* stream) {
+  using namespace mi355;
+  MI355_REQUIRE(T >= 0 && K >= 1 && T * K < (1ll << 31) && pieces >= 1 && pieces <= 4096 && row_capacity >= 0 &&
+                    row_capacity < (1ll << 31),
+                "combine_scores_bwd: bad shape");
+  if (T == 0) return MI355_OK;
+  MI355_REQUIRE(row_of_slot && dweights_TK && (dot_partial || row_capacity == 0), "combine_scores_bwd: null pointer");
+  hipLaunchKernelGGL(scores_bwd_kernel, dim3((unsigned)((T * K + 255) / 256)), dim3(256), 0, as_stream(stream),
+                     dot_partial, (int)pieces, row_of_slot, dweights_TK, (int)(T * K), (int)row_capacity);
+  return check_launch("combine_scores_bwd");
+}
+

@@ -20,8 +20,10 @@ int bf16_grouped_fwd(const void* rows, const int32_t* token_of_row, const void* 
                      const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* num_tiles,
                      int64_t tile_capacity, void* gate, void* up, void* h, void* y, int64_t D,
                      int64_t F, int stages, hipStream_t s);
+int bf16_fused_dot_slots(int64_t F);
 int bf16_grouped_bwd(const void* dy, const void* rows, const int32_t* token_of_row, const void* w1,
                      const void* w3, const void* w2, const void* gate, const void* up, const void* h,
+                     const float* row_scale, float* dot_partial,
                      const int32_t* seg_offsets, const int32_t* seg_counts,
                      const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* num_tiles,
                      int64_t tile_capacity, void* dgate, void* dup, void* drows, void* dw1,
@@ -175,8 +177,8 @@ extern "C" int mi355_grouped_swiglu_bwd(const void* dy, const void* rows,
   hipStream_t s = as_stream(stream);
   if (dtype == MI355_BF16 && bf16_fast_path_ok(D, F) && row_capacity > 0 && tile_capacity > 0)
     return bf16_grouped_bwd(
-        dy, rows, token_of_row, w1, w3, w2, gate, up, h, seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles,
-        tile_capacity, dgate, dup, drows, dw1, dw3, dw2, El, D, F, 0x7c, s);
+        dy, rows, token_of_row, w1, w3, w2, gate, up, h, nullptr, nullptr, seg_offsets, seg_counts, tile_expert,
+        tile_row0, num_tiles, tile_capacity, dgate, dup, drows, dw1, dw3, dw2, El, D, F, 0x7c, s);
   if (token_of_row)
     return fail(MI355_EUNSUP, "grouped_swiglu_bwd: the token gather needs bf16 with D and F multiples of 64");
   const Seg sg{seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles, tile_capacity};
@@ -223,6 +225,36 @@ extern "C" int mi355_grouped_swiglu_stage(int stage, const void* dy, const void*
                                                              tile_expert, tile_row0, num_tiles,
                                                              tile_capacity, gate, up, h, y, D, F, stage, s);
   return bf16_grouped_bwd(
-      dy, rows, token_of_row, w1, w3, w2, gate, up, h, seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles,
-      tile_capacity, dgate, dup, drows, dw1, dw3, dw2, El, D, F, stage, s);
+      dy, rows, token_of_row, w1, w3, w2, gate, up, h, nullptr, nullptr, seg_offsets, seg_counts, tile_expert,
+      tile_row0, num_tiles, tile_capacity, dgate, dup, drows, dw1, dw3, dw2, El, D, F, stage, s);
+}
+
+extern "C" int64_t mi355_grouped_combine_bwd_slots(int dtype, int64_t D, int64_t F) {
+  if (dtype != MI355_BF16 || D < 1 || F < 1 || !bf16_fast_path_ok(D, F)) return 0;
+  return bf16_fused_dot_slots(F);
+}
+
+extern "C" int mi355_grouped_swiglu_combine_bwd(
+    const void* dout, const void* x, const int32_t* token_of_row, const float* row_scale, const void* w1,
+    const void* w3, const void* w2, const void* gate, const void* up, int dtype, const int32_t* seg_offsets,
+    const int32_t* seg_counts, const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* num_tiles,
+    int64_t tile_capacity, void* dgate, void* dup, void* hs, float* dot_partial, void* drows, void* dw1,
+    void* dw3, void* dw2, int64_t El, int64_t D, int64_t F, int64_t row_capacity, void* stream) {
+  if (int rc = check_common("grouped_swiglu_combine_bwd", dtype, El, D, F, row_capacity, tile_capacity)) return rc;
+  if (mi355_grouped_combine_bwd_slots(dtype, D, F) == 0)
+    return fail(MI355_EUNSUP, "grouped_swiglu_combine_bwd: needs bf16 with D and F multiples of 64 (>= 384) and the "
+                              "256-row tile layout; use mi355_combine_bwd + mi355_grouped_swiglu_bwd instead");
+  MI355_REQUIRE(seg_offsets && seg_counts && num_tiles, "grouped_swiglu_combine_bwd: null plan pointer");
+  if (row_capacity == 0 || tile_capacity == 0) {
+    // no rows: the weight gradients are still defined (zeros); the plain entry point writes them
+    return mi355_grouped_swiglu_bwd(dout, x, token_of_row, w1, w3, w2, gate, up, hs, dtype, seg_offsets, seg_counts,
+                                    tile_expert, tile_row0, num_tiles, tile_capacity, dgate, dup, drows, dw1, dw3,
+                                    dw2, El, D, F, row_capacity, stream);
+  }
+  MI355_REQUIRE(dout && x && token_of_row && row_scale && w1 && w3 && w2 && gate && up && dgate && dup && hs &&
+                    dot_partial && tile_expert && tile_row0,
+                "grouped_swiglu_combine_bwd: null pointer");
+  return bf16_grouped_bwd(dout, x, token_of_row, w1, w3, w2, gate, up, hs, row_scale, dot_partial, seg_offsets,
+                          seg_counts, tile_expert, tile_row0, num_tiles, tile_capacity, dgate, dup, drows, dw1, dw3,
+                          dw2, El, D, F, 0x7c, as_stream(stream));
 }

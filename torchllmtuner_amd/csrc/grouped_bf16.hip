@@ -85,7 +85,13 @@ struct RowArgs {
   uint16_t* o2;        // GATEUP h
   const uint16_t* gate;  // DH
   const uint16_t* up;    // DH
-  const int32_t* a_src;  // GATEUP: row -> row of a0 to read (token gather), or null
+  const int32_t* a_src;  // GATEUP, DH: row -> row of a0 to read (token gather), or null
+  // DH with a_src (the combine's backward folded in): a0 is the layer's output gradient (T, D),
+  // row r stands for row_scale[r] * a0[a_src[r]]; o2 receives row_scale * h and dot_partial
+  // [row][dot_slots] the pieces of <unscaled dh row, h row>, one per 128 output columns
+  const float* row_scale;
+  float* dot_partial;
+  int dot_slots;
   const int32_t* seg_offsets;
   const int32_t* seg_counts;
   const int32_t* tile_expert;
@@ -102,8 +108,17 @@ constexpr int RBM = 128, RBN = 512;
 constexpr int R_STAGE = (RBM + RBN) * BK;  // elements per LDS stage (80 KiB)
 
 struct TileMeta {
-  int e, row0, valid, n0;
+  int e, row0, valid, n0, nt;
 };
+
+// sum over each group of 16 consecutive lanes, left in all 16 (DPP row operations)
+__device__ __forceinline__ float row16_sum(float v) {
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, false));   // quad_perm [1,0,3,2]
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, false));   // quad_perm [2,3,0,1]
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, false));  // row_half_mirror
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, false));  // row_mirror
+  return v;
+}
 
 template <int MODE, int NJ, bool GATHER, int WM>
 __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
@@ -114,7 +129,8 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
   constexpr int NB = BNT / 64;             // the same for B
   constexpr int STAGE = (TBM + BNT) * BK;  // elements per LDS stage
   constexpr bool B_KS = (MODE == RM_DH || MODE == RM_DX);
-  static_assert(!GATHER || MODE == RM_GATEUP, "only the gate/up product gathers its rows");
+  static_assert(!GATHER || MODE == RM_GATEUP || MODE == RM_DH, "only gate/up and dH gather their rows");
+  static_assert(!(GATHER && MODE == RM_DH) || NJ == 4, "the fused dH epilogue reduces over 16 lanes per row");
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -155,6 +171,7 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
     // of its neighbour (same values), so no column is ever clamped
     constexpr int W = (MODE == RM_GATEUP ? BNT / 2 : BNT);
     m.n0 = min(nt * W, Ncols - W);
+    m.nt = nt;
     return m;
   };
 
@@ -277,7 +294,7 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
   const TileMeta nxt2 = load_meta(exists(within + 2 * stride) ? within + 2 * stride : within);
   int nsrc[NA];
   load_asrc(nxt, nsrc);
-  const int row0 = cur.row0, valid = cur.valid, n0 = cur.n0;
+  const int row0 = cur.row0, valid = cur.valid, n0 = cur.n0, ntile = cur.nt;
 
   f32x4 acc[4][NJ2];
 #pragma unroll
@@ -449,24 +466,39 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
       // SwiGLU backward on 8 consecutive f: dgate = dh*up*silu'(gate), dup = dh*silu(gate).
       // gate and up of the next four chunks are requested before the current four are stored:
       // a load issued behind a store cannot complete before it.
+      // With the combine's backward folded in (FUSE), the staged value is the unscaled dh row:
+      // its product with the row's h (recomputed from gate and up) summed over f is the
+      // gradient of the row's routing score, reduced here over the 16 lanes that share a row
+      // and written once per row and 128-column slot; dh itself is then scaled by the score,
+      // and score * h goes out as the operand of the dW2 product.
+      constexpr bool FUSE = GATHER;
       constexpr int G = 4;
       static_assert(CH % G == 0, "chunks per row come in groups of four");
+      auto row_at = [&](int it) -> int {
+        int m, c;
+        chunk_at(it, m, c);
+        return row0 + wm + m;
+      };
       u32x4 gq[G], uq[G];
+      float sq[G];
 #pragma unroll
       for (int u = 0; u < G; ++u) {
         const int64_t o = offset_at(u);
         gq[u] = *reinterpret_cast<const u32x4*>(p.gate + o);
         uq[u] = *reinterpret_cast<const u32x4*>(p.up + o);
+        if constexpr (FUSE) sq[u] = p.row_scale[row_at(u)];
       }
 #pragma unroll
       for (int g0 = 0; g0 < CH; g0 += G) {
         u32x4 gn[G], un[G];
+        float sn[G];
         if (g0 + G < CH) {
 #pragma unroll
           for (int u = 0; u < G; ++u) {
             const int64_t o = offset_at(g0 + G + u);
             gn[u] = *reinterpret_cast<const u32x4*>(p.gate + o);
             un[u] = *reinterpret_cast<const u32x4*>(p.up + o);
+            if constexpr (FUSE) sn[u] = p.row_scale[row_at(g0 + G + u)];
           }
         }
 #pragma unroll
@@ -475,33 +507,53 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
           chunk_at(g0 + u, m, c);
           const u32x4 v = *reinterpret_cast<const u32x4*>(st + m * S::PITCH + c * 8);
           const u32x4 gv = gq[u], uv = uq[u];
-          u32x4 dg, du;
+          const float sc = FUSE ? sq[u] : 1.0f;
+          float dot = 0.0f;
+          u32x4 dg, du, hs;
 #pragma unroll
           for (int w = 0; w < 4; ++w) {
-            float r_dg[2], r_du[2];
+            float r_dg[2], r_du[2], r_hs[2];
 #pragma unroll
             for (int hlf = 0; hlf < 2; ++hlf) {
-              const float dh = __uint_as_float(hlf ? (v[w] & 0xffff0000u) : (v[w] << 16));
+              float dh = __uint_as_float(hlf ? (v[w] & 0xffff0000u) : (v[w] << 16));
               const float g = __uint_as_float(hlf ? (gv[w] & 0xffff0000u) : (gv[w] << 16));
               const float uu = __uint_as_float(hlf ? (uv[w] & 0xffff0000u) : (uv[w] << 16));
               const float sig = fast_sigmoid(g);
               const float sl = round_bf16(g * sig);
+              if constexpr (FUSE) {
+                const float hv = round_bf16(sl * uu);  // h as the forward stored it
+                dot += dh * hv;
+                r_hs[hlf] = sc * hv;
+                dh *= sc;
+              }
               const float ds = round_bf16(dh * uu);
               r_du[hlf] = dh * sl;
               r_dg[hlf] = ds * (sig * (1.0f + g * (1.0f - sig)));
             }
             dg[w] = pack2(r_dg[0], r_dg[1]);
             du[w] = pack2(r_du[0], r_du[1]);
+            if constexpr (FUSE) hs[w] = pack2(r_hs[0], r_hs[1]);
           }
           const int64_t o = offset_at(g0 + u);
           *reinterpret_cast<u32x4*>(p.o0 + o) = dg;
           *reinterpret_cast<u32x4*>(p.o1 + o) = du;
+          if constexpr (FUSE) {
+            *reinterpret_cast<u32x4*>(p.o2 + o) = hs;
+            // columns below the tile's nominal start belong to its neighbour (a last tile
+            // that would overhang starts early): they must not be counted twice
+            if (c0 + c * 8 < ntile * BNT) dot = 0.0f;
+            const float total = row16_sum(dot);
+            // all 16 lanes of the row store the same value to the same address (unconditional,
+            // like every other access of this epilogue)
+            p.dot_partial[static_cast<int64_t>(row0 + wm + m) * p.dot_slots + ntile * WN + wn] = total;
+          }
         }
         if (g0 + G < CH) {
 #pragma unroll
           for (int u = 0; u < G; ++u) {
             gq[u] = gn[u];
             uq[u] = un[u];
+            if constexpr (FUSE) sq[u] = sn[u];
           }
         }
       }
@@ -536,6 +588,7 @@ struct WgradArgs {
   const uint16_t* a;  // (rows, M) row-major
   const uint16_t* b;  // (rows, N) row-major
   uint16_t* c;        // (El, M, N)
+  const int32_t* a_src;  // row -> row of a to read, or null (GATHER_A)
   const int32_t* b_src;  // row -> row of b to read (token gather), or null
   const int32_t* seg_offsets;
   const int32_t* seg_counts;  // (2 El): row counts, then the local experts by descending count
@@ -545,7 +598,7 @@ struct WgradArgs {
   int total;  // El * m_tiles * n_tiles
 };
 
-template <bool GATHER>
+template <bool GATHER, bool GATHER_A = false>
 __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -618,7 +671,7 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
   const uint16_t* a_base;
   const uint16_t* b_base;
   auto set_bases = [&]() {
-    a_base = p.a + static_cast<int64_t>(seg0) * M + min(m0 + ks_chunk * 8, M - 8);
+    a_base = p.a + (GATHER_A ? 0 : static_cast<int64_t>(seg0) * M) + min(m0 + ks_chunk * 8, M - 8);
     b_base = p.b + (GATHER ? 0 : static_cast<int64_t>(seg0) * N) + min(n0 + ks_chunk * 8, N - 8);
   };
   // B row of this thread's chunk i in K step `step` of segment (s0, c): its own row, or
@@ -627,10 +680,15 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
     const int k = min(step * BK + ks_k + 16 * i, c - 1);
     return GATHER ? max(p.b_src[s0 + k], 0) : k;
   };
+  // the same for the A row (its own row unless A is gathered too)
+  auto a_row_index = [&](int s0, int c, int step, int i) -> int {
+    const int k = min(step * BK + ks_k + 16 * i, c - 1);
+    return GATHER_A ? max(p.a_src[s0 + k], 0) : k;
+  };
   // Loads of one K step, unconditional: rows past the segment re-read its last row and
   // the A side is zeroed when it is parked, so the products vanish.  Needs cnt > 0.
-  auto load_ab = [&](int step, int i, int brow) {
-    const int k = min(step * BK + ks_k + 16 * i, cnt - 1);
+  auto load_ab = [&](int step, int i, int brow, int arow_g) {
+    const int k = GATHER_A ? arow_g : min(step * BK + ks_k + 16 * i, cnt - 1);
     ra[i] = *reinterpret_cast<const u32x4*>(a_base + static_cast<int64_t>(k) * M);
     rb[i] = *reinterpret_cast<const u32x4*>(b_base + static_cast<int64_t>(brow) * N);
   };
@@ -640,12 +698,16 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
     *reinterpret_cast<u32x4*>(Bn + lds_off[i]) = rb[i];
   };
   int bidx[4];  // B rows of the K step that is requested next
+  int aidx[4];  // A rows likewise (used when A is gathered)
   set_bases();
   if (cnt > 0) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) load_ab(0, i, row_index(seg0, cnt, 0, i));
+    for (int i = 0; i < 4; ++i) load_ab(0, i, row_index(seg0, cnt, 0, i), a_row_index(seg0, cnt, 0, i));
 #pragma unroll
-    for (int i = 0; i < 4; ++i) bidx[i] = row_index(seg0, cnt, 1, i);
+    for (int i = 0; i < 4; ++i) {
+      bidx[i] = row_index(seg0, cnt, 1, i);
+      aidx[i] = a_row_index(seg0, cnt, 1, i);
+    }
   }
   // expert and segment of the next tile, expert of the one after it (its segment is
   // looked up inside the loop, the expert after that too)
@@ -660,10 +722,13 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
     const int n2seg0 = seg_offsets[e2], n2cnt = seg_counts[e2];
     const int e3 = expert_of(within + 3 * stride);
     // next tile: B rows of its first K step (its bounds were looked up a tile ago)
-    int nidx[4];
+    int nidx[4], nidx_a[4];
     if (ncnt > 0) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) nidx[i] = row_index(nseg0, ncnt, 0, i);
+      for (int i = 0; i < 4; ++i) {
+        nidx[i] = row_index(nseg0, ncnt, 0, i);
+        nidx_a[i] = a_row_index(nseg0, ncnt, 0, i);
+      }
     }
     const int c_e = e, c_m0 = m0, c_n0 = n0, c_cnt = cnt, c_seg0 = seg0;
     const int ksteps = (cnt + BK - 1) / BK;
@@ -683,9 +748,12 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
       for (int i = 0; i < 4; ++i) park(0, i, smem, smem + WBM * BK, c_cnt);
       if (ksteps > 1) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) load_ab(1, i, bidx[i]);
+        for (int i = 0; i < 4; ++i) load_ab(1, i, bidx[i], aidx[i]);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) bidx[i] = row_index(c_seg0, c_cnt, 2, i);
+        for (int i = 0; i < 4; ++i) {
+          bidx[i] = row_index(c_seg0, c_cnt, 2, i);
+          aidx[i] = a_row_index(c_seg0, c_cnt, 2, i);
+        }
       }
     }
     __syncthreads();
@@ -709,8 +777,9 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
         for (int nj = 0; nj < 4; ++nj) bf[nj] = frag_ks<256>(Bs, wn + nj * 32, kk, lane);
         if constexpr (has_next) park(ks + 1, kk, An, Bn, c_cnt);
         if constexpr (has_next2) {
-          load_ab(ks + 2, kk, bidx[kk]);
+          load_ab(ks + 2, kk, bidx[kk], aidx[kk]);
           bidx[kk] = row_index(c_seg0, c_cnt, ks + 3, kk);
+          aidx[kk] = a_row_index(c_seg0, c_cnt, ks + 3, kk);
         }
 #pragma unroll
         for (int mi = 0; mi < 2; ++mi)
@@ -738,9 +807,12 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
       set_bases();
       if (cnt > 0) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) load_ab(0, i, nidx[i]);
+        for (int i = 0; i < 4; ++i) load_ab(0, i, nidx[i], nidx_a[i]);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) bidx[i] = row_index(seg0, cnt, 1, i);
+        for (int i = 0; i < 4; ++i) {
+          bidx[i] = row_index(seg0, cnt, 1, i);
+          aidx[i] = a_row_index(seg0, cnt, 1, i);
+        }
       }
     }
 
@@ -890,8 +962,17 @@ int bf16_grouped_fwd(const void* rows, const int32_t* token_of_row, const void* 
   return MI355_OK;
 }
 
+int bf16_fused_dot_slots(int64_t F) {
+  // one partial per 128 output columns of the dH tile (two waves across its 256 columns)
+  return tall_layout() ? (int)((F + 255) / 256) * 2 : 0;
+}
+
+// row_scale != null: the combine's backward is folded in.  dy is then the layer's output
+// gradient (T, D), read through token_of_row and scaled by row_scale; `h` is written (it
+// receives row_scale * h, the operand of dW2) and dot_partial gets the score-gradient pieces.
 int bf16_grouped_bwd(const void* dy, const void* rows, const int32_t* token_of_row, const void* w1,
                        const void* w3, const void* w2, const void* gate, const void* up, const void* h,
+                       const float* row_scale, float* dot_partial,
                        const int32_t* seg_offsets, const int32_t* seg_counts,
                        const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* num_tiles,
                        int64_t tile_capacity, void* dgate, void* dup, void* drows, void* dw1,
@@ -904,7 +985,17 @@ int bf16_grouped_bwd(const void* dy, const void* rows, const int32_t* token_of_r
     a.a0 = (const uint16_t*)dy; a.b0 = (const uint16_t*)w2;
     a.gate = (const uint16_t*)gate; a.up = (const uint16_t*)up;
     a.o0 = (uint16_t*)dgate; a.o1 = (uint16_t*)dup;
-    if (int rc = launch_row<RM_DH>(a, F, tile_capacity, s, "grouped dh")) return rc;
+    if (row_scale) {
+      if (!tall_layout()) return fail(MI355_EUNSUP, "grouped dh: the folded combine needs the 256-row tile layout");
+      a.a_src = token_of_row; a.row_scale = row_scale; a.dot_partial = dot_partial;
+      a.o2 = (uint16_t*)const_cast<void*>(h);
+      a.dot_slots = bf16_fused_dot_slots(F);
+      a.n_tiles = (int)((F + 255) / 256);
+      if (int rc = launch_row_as<RM_DH, 4, true, 4>(a, tile_capacity, s, "grouped dh + combine")) return rc;
+      a.a_src = nullptr;
+    } else {
+      if (int rc = launch_row<RM_DH>(a, F, tile_capacity, s, "grouped dh")) return rc;
+    }
   }
   if (drows && (stages & STAGE_DX)) {
     RowArgs b = a;
@@ -916,22 +1007,28 @@ int bf16_grouped_bwd(const void* dy, const void* rows, const int32_t* token_of_r
   if (wconfigured.needed()) {
     if (int rc = set_lds(wgrad_kernel<false>, W_LDS_BYTES)) return rc;
     if (int rc = set_lds(wgrad_kernel<true>, W_LDS_BYTES)) return rc;
+    if (int rc = set_lds(wgrad_kernel<false, true>, W_LDS_BYTES)) return rc;
     wconfigured.done();
   }
-  auto wgrad = [&](const void* A, const void* B, const int32_t* b_src, void* C, int64_t M, int64_t N, const char* what) {
+  auto wgrad = [&](const void* A, const void* B, const int32_t* b_src, void* C, int64_t M, int64_t N, const char* what,
+                   const int32_t* a_src = nullptr) {
     WgradArgs w{};
-    w.a = (const uint16_t*)A; w.b = (const uint16_t*)B; w.c = (uint16_t*)C; w.b_src = b_src;
+    w.a = (const uint16_t*)A; w.b = (const uint16_t*)B; w.c = (uint16_t*)C; w.b_src = b_src; w.a_src = a_src;
     w.seg_offsets = seg_offsets; w.seg_counts = seg_counts; w.El = (int)El; w.M = (int)M; w.N = (int)N;
     w.m_tiles = (int)((M + WBM - 1) / WBM); w.n_tiles = (int)((N + WBN - 1) / WBN);
     w.total = (int)(El * w.m_tiles * w.n_tiles);
     const dim3 grid(std::min(round8(w.total), resident_blocks()));
-    if (b_src)
+    if (a_src)
+      hipLaunchKernelGGL((wgrad_kernel<false, true>), grid, dim3(NT), W_LDS_BYTES, s, w);
+    else if (b_src)
       hipLaunchKernelGGL(wgrad_kernel<true>, grid, dim3(NT), W_LDS_BYTES, s, w);
     else
       hipLaunchKernelGGL(wgrad_kernel<false>, grid, dim3(NT), W_LDS_BYTES, s, w);
     return check_launch(what);
   };
-  if (dw2 && (stages & STAGE_DW2)) if (int rc = wgrad(dy, h, nullptr, dw2, D, F, "grouped dw2")) return rc;
+  // folded combine: dW2 = (gathered output gradient)^T . (row_scale * h)
+  if (dw2 && (stages & STAGE_DW2))
+    if (int rc = wgrad(dy, h, nullptr, dw2, D, F, "grouped dw2", row_scale ? token_of_row : nullptr)) return rc;
   if (dw1 && (stages & STAGE_DW1)) if (int rc = wgrad(dgate, rows, token_of_row, dw1, F, D, "grouped dw1")) return rc;
   if (dw3 && (stages & STAGE_DW3)) if (int rc = wgrad(dup, rows, token_of_row, dw3, F, D, "grouped dw3")) return rc;
   return MI355_OK;

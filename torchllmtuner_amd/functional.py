@@ -196,6 +196,39 @@ class GatherGroupedSwiGLUFunction(torch.autograd.Function):
         return dx, dw1, dw3, dw2, None
 
 
+class GatherExpertsCombineFunction(torch.autograd.Function):
+    """out[t] = sum_k weights[t,k] * experts(x)[row(t,k)] with one backward for both halves.
+
+    The forward is the gathered expert product followed by the combine.  The backward never
+    forms the expert-major output gradient ``weights * dout`` and never re-reads the expert
+    outputs: the dH kernel reads ``dout`` through the plan's token index and scales each row
+    in its epilogue, where the same pass yields the gradient of the routing weights (the row's
+    unscaled dh times its h, summed over the hidden columns); dW2 contracts the gathered
+    ``dout`` rows with ``weights * h``.  Nothing of size (R, D) is kept between forward and
+    backward, and of the (R, F) tensors only gate and up.
+    """
+
+    @staticmethod
+    def forward(ctx, x_TD, weights_TK, w1_EFD, w3_EFD, w2_EDF, plan, round_terms):
+        y, gate, up, _h = ops.grouped_swiglu_fwd(x_TD, w1_EFD, w3_EFD, w2_EDF, plan, gather=True)
+        out = ops.combine_fwd(y, weights_TK, plan, round_terms)
+        ctx.save_for_backward(x_TD, weights_TK, w1_EFD, w3_EFD, w2_EDF, gate, up)
+        ctx.plan = plan
+        return out
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, dout):
+        x, weights, w1, w3, w2, gate, up = ctx.saved_tensors
+        row_scale = ops.combine_row_scale(weights, ctx.plan)
+        drows, dw1, dw3, dw2, dweights = ops.grouped_swiglu_combine_bwd(
+            dout, x, row_scale, w1, w3, w2, gate, up, ctx.plan,
+            need_drows=ctx.needs_input_grad[0], need_dw=any(ctx.needs_input_grad[2:5]),
+        )
+        dx = ops.permute_rows_bwd(drows, ctx.plan) if drows is not None else None
+        return dx, dweights.to(weights.dtype), dw1, dw3, dw2, None, None
+
+
 class CombineFunction(torch.autograd.Function):
     """out[t] = sum_k weights[t,k] * y[row(t,k)]; backward gives dY and dWeights."""
 
@@ -243,6 +276,10 @@ def grouped_swiglu(rows_RD, w1_EFD, w3_EFD, w2_EDF, plan):
 
 def gather_grouped_swiglu(x_TD, w1_EFD, w3_EFD, w2_EDF, plan):
     return GatherGroupedSwiGLUFunction.apply(x_TD, w1_EFD, w3_EFD, w2_EDF, plan)
+
+
+def gather_experts_combine(x_TD, weights_TK, w1_EFD, w3_EFD, w2_EDF, plan, round_terms=True):
+    return GatherExpertsCombineFunction.apply(x_TD, weights_TK, w1_EFD, w3_EFD, w2_EDF, plan, round_terms)
 
 
 def combine(y_RD, weights_TK, plan, round_terms=True):

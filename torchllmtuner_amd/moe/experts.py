@@ -150,7 +150,13 @@ class RoutedExperts(nn.Module):
 
     def forward_planned(self, x_TD, topk_scores_TK, plan: ops.PermutePlan):
         experts = self.inner_experts
+        round_terms = not self.token_dispatcher.accumulate_in_fp32
         if ops.gather_supported(x_TD, experts.hidden_dim) and x_TD.is_contiguous():
+            if ops.combine_bwd_slots(x_TD.dtype, x_TD.shape[-1], experts.hidden_dim) > 0:
+                # ... and the combine's backward inside the expert kernels' backward
+                w1, w3, w2 = experts._weights_as(x_TD.dtype)
+                out = Fn.gather_experts_combine(x_TD, topk_scores_TK, w1, w3, w2, plan, round_terms)
+                return out.to(x_TD.dtype)
             # the dispatch gather rides inside the expert kernels' operand loads
             y = experts.compute_gathered(x_TD, plan)
         else:
@@ -161,7 +167,7 @@ class RoutedExperts(nn.Module):
             ):
                 rows = Fn.permute_rows(x_TD, plan)
             y = experts.compute_planned(rows, plan)
-        out = Fn.combine(y, topk_scores_TK, plan, not self.token_dispatcher.accumulate_in_fp32)
+        out = Fn.combine(y, topk_scores_TK, plan, round_terms)
         return out.to(x_TD.dtype)
 
 

@@ -9,6 +9,8 @@ from __future__ import annotations
 
 from dataclasses import dataclass
 
+import os
+
 import torch
 
 from . import _lib
@@ -502,6 +504,69 @@ def grouped_swiglu_bwd(dy_RD, rows_RD, w1_EFD, w3_EFD, w2_EDF, gate, up, h, plan
         )
     _lib.check(rc, "grouped_swiglu_bwd")
     return drows, dw1, dw3, dw2
+
+
+# False sends RoutedExperts through the two-call backward (combine, then experts) also where
+# the folded one applies (MI355_FOLD_COMBINE=0 in the environment does the same).
+FOLD_COMBINE = os.environ.get("MI355_FOLD_COMBINE", "1") != "0"
+
+
+def combine_bwd_slots(dtype, D, F):
+    """Partials per row of the folded experts+combine backward; 0 when it does not apply."""
+    if dtype != torch.bfloat16 or not FOLD_COMBINE:
+        return 0
+    return int(_lib.load().mi355_grouped_combine_bwd_slots(_DT[dtype], int(D), int(F)))
+
+
+def combine_row_scale(weights_TK, plan: PermutePlan):
+    """row_scale[r] = weights[slot_of_row[r]] (0 for padding rows), fp32."""
+    dev = _dev(weights_TK, plan.slot_of_row)
+    weights_TK = _c(weights_TK.float())
+    R = plan.row_capacity
+    out = torch.empty(R, dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_combine_row_scale(
+            _p(weights_TK), _p(plan.slot_of_row), _p(out), plan.num_tokens, plan.top_k, R, _stream(dev),
+        )
+    _lib.check(rc, "combine_row_scale")
+    return out
+
+
+def grouped_swiglu_combine_bwd(dout_TD, x_TD, row_scale_R, w1_EFD, w3_EFD, w2_EDF, gate, up, plan: PermutePlan,
+                               need_drows=True, need_dw=True):
+    """Backward of gathered experts + combine in one pass; returns (drows, dw1, dw3, dw2, dweights_TK)."""
+    dev = _dev(dout_TD, x_TD)
+    dout_TD, x_TD = _c(dout_TD), _c(x_TD)
+    if dout_TD.dtype != x_TD.dtype:
+        dout_TD = dout_TD.to(x_TD.dtype)
+    w1_EFD, w3_EFD, w2_EDF = _c(w1_EFD), _c(w3_EFD), _c(w2_EDF)
+    D = x_TD.shape[1]
+    R = gate.shape[0]
+    El, F, _ = w1_EFD.shape
+    lib = _lib.load()
+    slots = combine_bwd_slots(x_TD.dtype, D, F)
+    if slots <= 0:
+        raise _lib.MI355LibraryError("grouped_swiglu_combine_bwd does not cover this dtype/shape/layout")
+    dgate, dup, hs = torch.empty_like(gate), torch.empty_like(up), torch.empty_like(gate)
+    partial = torch.empty(R, slots, dtype=torch.float32, device=dev)
+    drows = torch.empty(R, D, dtype=x_TD.dtype, device=dev) if need_drows else None
+    dw1 = torch.empty_like(w1_EFD) if need_dw else None
+    dw3 = torch.empty_like(w3_EFD) if need_dw else None
+    dw2 = torch.empty_like(w2_EDF) if need_dw else None
+    dweights = torch.empty(plan.num_tokens, plan.top_k, dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        rc = lib.mi355_grouped_swiglu_combine_bwd(
+            _p(dout_TD), _p(x_TD), _p(plan.token_of_row), _p(row_scale_R), _p(w1_EFD), _p(w3_EFD), _p(w2_EDF),
+            _p(gate), _p(up), _dt(x_TD), _p(plan.seg_offsets), _p(plan.seg_counts), _p(plan.tile_expert),
+            _p(plan.tile_row0), _p(plan.num_tiles), plan.tile_capacity, _p(dgate), _p(dup), _p(hs), _p(partial),
+            _p(drows), _p(dw1), _p(dw3), _p(dw2), El, D, F, R, _stream(dev),
+        )
+        _lib.check(rc, "grouped_swiglu_combine_bwd")
+        rc = lib.mi355_combine_scores_bwd(
+            _p(partial), slots, _p(plan.row_of_slot), _p(dweights), plan.num_tokens, plan.top_k, R, _stream(dev),
+        )
+    _lib.check(rc, "combine_scores_bwd")
+    return drows, dw1, dw3, dw2, dweights
 
 
 STAGES = {"gate_up": 1, "down": 2, "dh": 4, "drows": 8, "dw2": 16, "dw1": 32, "dw3": 64}
