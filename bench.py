@@ -200,7 +200,22 @@ def main():
                    dw1=torch.empty_like(w1), dw3=torch.empty_like(w3), dw2=torch.empty_like(w2))
         R_rows = int(plan.total_rows.item())
         it = args.stage_iters
-        stage_ms = {s: time_events(lambda s=s: ops.grouped_swiglu_stage(s, buf, plan), it) for s in ops.STAGES}
+        # The step's backward folds the combine into the expert kernels: dH reads the output
+        # gradient through the token index and scales rows in its epilogue, dW2 contracts the
+        # gathered rows with score * h.  Those two are timed in that form.
+        folded = ops.combine_bwd_slots(x.dtype, D, F) > 0
+        if folded:
+            buf.update(dout=gout, row_scale=ops.combine_row_scale(scores, plan), hs=torch.empty_like(h),
+                       dot_partial=torch.empty(rows.shape[0], ops.combine_bwd_slots(x.dtype, D, F),
+                                               dtype=torch.float32, device=dev))
+
+        def run_stage(s):
+            if folded and s in ("dh", "dw2"):
+                ops.grouped_swiglu_combine_stage(s, buf, plan)
+            else:
+                ops.grouped_swiglu_stage(s, buf, plan)
+
+        stage_ms = {s: time_events(lambda s=s: run_stage(s), it) for s in ops.STAGES}
         logits = ops.router_gate_fwd(x, block.router.gate.weight)
         other_ms = {
             "router_gate_fwd": time_events(lambda: ops.router_gate_fwd(x, block.router.gate.weight), it),
@@ -212,6 +227,9 @@ def main():
             "permute_rows_bwd": time_events(lambda: ops.permute_rows_bwd(buf["drows"], plan), it),
             "router_gate_bwd": time_events(lambda: ops.router_gate_bwd(logits, x, block.router.gate.weight), it),
         }
+        if folded:
+            other_ms["combine_row_scale"] = time_events(lambda: ops.combine_row_scale(scores, plan), it)
+            other_ms["combine_scores_bwd"] = time_events(lambda: ops.combine_scores_bwd(buf["dot_partial"], plan), it)
         # the callers' side of the path, outside the timed step: the decoder layer's norm in
         # front of the block and the statistics of a quantile-balanced router
         norm_w = torch.ones(D, dtype=torch.bfloat16, device=dev)
@@ -246,9 +264,10 @@ def main():
         kernels[f"grouped_{s}"] = {"ms": round(ms, 4), "TFLOP/s": round(tf, 1), "frac_mfma": round(tf / PEAK_BF16_TFLOPS, 4)}
     for s, ms in other_ms.items():
         ent = {"ms": round(ms, 4)}
-        if s == "permute_rows_fwd" or s in outside_ms:
-            # permute_rows_fwd: public dispatcher API only, the fused step gathers inside the
-            # GEMMs; the others belong to the block's callers
+        if s == "permute_rows_fwd" or (s == "combine_bwd" and folded) or s in outside_ms:
+            # permute_rows_fwd, combine_bwd: public dispatcher API only, the step gathers inside
+            # the GEMMs and folds the combine's backward into them; the others belong to the
+            # block's callers
             ent["in_step"] = False
         if s in other_bytes:
             gbs = other_bytes[s] / (ms * 1e-3) / 1e9

@@ -364,6 +364,8 @@ int mi355_grouped_swiglu_bwd(const void* dy, const void* rows,
  * the two-call form).  row_scale (row_capacity floats) comes from mi355_combine_row_scale:
  * row_scale[r] = weights[slot_of_row[r]], 0 for rows that hold padding.
  * dgate, dup, hs: caller-provided (row_capacity,F) each; dot_partial (row_capacity,slots) fp32.
+ * stages: 0 for the whole backward, or a mask of MI355_STAGE_DH ... MI355_STAGE_DW3 (below) to
+ * launch only those kernels on the same buffers (profilers, callers that schedule the stages).
  */
 int64_t mi355_grouped_combine_bwd_slots(int dtype, int64_t D, int64_t F);
 int mi355_grouped_swiglu_combine_bwd(const void* dout, const void* x, const int32_t* token_of_row,
@@ -374,7 +376,7 @@ int mi355_grouped_swiglu_combine_bwd(const void* dout, const void* x, const int3
                                      const int32_t* num_tiles, int64_t tile_capacity, void* dgate,
                                      void* dup, void* hs, float* dot_partial, void* drows,
                                      void* dw1, void* dw3, void* dw2, int64_t El, int64_t D,
-                                     int64_t F, int64_t row_capacity, void* stream);
+                                     int64_t F, int64_t row_capacity, int stages, void* stream);
 int mi355_combine_row_scale(const float* weights_TK, const int32_t* slot_of_row, float* row_scale,
                             int64_t T, int64_t K, int64_t row_capacity, void* stream);
 /* dweights[t][k] = sum_j dot_partial[row_of_slot[t*K+k]][j], summed in ascending j; 0 for

@@ -55,7 +55,7 @@ SIGNATURES = {
     "mi355_grouped_combine_bwd_slots": (L, [I, L, L]),
     "mi355_grouped_swiglu_combine_bwd": (
         I,
-        [P, P, P, P, P, P, P, P, P, I, P, P, P, P, P, L, P, P, P, P, P, P, P, P, L, L, L, L, P],
+        [P, P, P, P, P, P, P, P, P, I, P, P, P, P, P, L, P, P, P, P, P, P, P, P, L, L, L, L, I, P],
     ),
     "mi355_combine_row_scale": (I, [P, P, P, L, L, L, P]),
     "mi355_combine_scores_bwd": (I, [P, L, P, P, L, L, L, P]),

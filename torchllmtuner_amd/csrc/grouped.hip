@@ -239,12 +239,13 @@ extern "C" int mi355_grouped_swiglu_combine_bwd(
     const void* w3, const void* w2, const void* gate, const void* up, int dtype, const int32_t* seg_offsets,
     const int32_t* seg_counts, const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* num_tiles,
     int64_t tile_capacity, void* dgate, void* dup, void* hs, float* dot_partial, void* drows, void* dw1,
-    void* dw3, void* dw2, int64_t El, int64_t D, int64_t F, int64_t row_capacity, void* stream) {
+    void* dw3, void* dw2, int64_t El, int64_t D, int64_t F, int64_t row_capacity, int stages, void* stream) {
   if (int rc = check_common("grouped_swiglu_combine_bwd", dtype, El, D, F, row_capacity, tile_capacity)) return rc;
   if (mi355_grouped_combine_bwd_slots(dtype, D, F) == 0)
     return fail(MI355_EUNSUP, "grouped_swiglu_combine_bwd: needs bf16 with D and F multiples of 64 (>= 384) and the "
                               "256-row tile layout; use mi355_combine_bwd + mi355_grouped_swiglu_bwd instead");
   MI355_REQUIRE(seg_offsets && seg_counts && num_tiles, "grouped_swiglu_combine_bwd: null plan pointer");
+  MI355_REQUIRE(stages >= 0 && (stages & ~0x7c) == 0, "grouped_swiglu_combine_bwd: stages must be 0 or a mask of the backward stages");
   if (row_capacity == 0 || tile_capacity == 0) {
     // no rows: the weight gradients are still defined (zeros); the plain entry point writes them
     return mi355_grouped_swiglu_bwd(dout, x, token_of_row, w1, w3, w2, gate, up, hs, dtype, seg_offsets, seg_counts,
@@ -256,5 +257,5 @@ extern "C" int mi355_grouped_swiglu_combine_bwd(
                 "grouped_swiglu_combine_bwd: null pointer");
   return bf16_grouped_bwd(dout, x, token_of_row, w1, w3, w2, gate, up, hs, row_scale, dot_partial, seg_offsets,
                           seg_counts, tile_expert, tile_row0, num_tiles, tile_capacity, dgate, dup, drows, dw1, dw3,
-                          dw2, El, D, F, 0x7c, as_stream(stream));
+                          dw2, El, D, F, stages ? stages : 0x7c, as_stream(stream));
 }

@@ -553,23 +553,53 @@ def grouped_swiglu_combine_bwd(dout_TD, x_TD, row_scale_R, w1_EFD, w3_EFD, w2_ED
     dw1 = torch.empty_like(w1_EFD) if need_dw else None
     dw3 = torch.empty_like(w3_EFD) if need_dw else None
     dw2 = torch.empty_like(w2_EDF) if need_dw else None
-    dweights = torch.empty(plan.num_tokens, plan.top_k, dtype=torch.float32, device=dev)
     with torch.cuda.device(dev):
         rc = lib.mi355_grouped_swiglu_combine_bwd(
             _p(dout_TD), _p(x_TD), _p(plan.token_of_row), _p(row_scale_R), _p(w1_EFD), _p(w3_EFD), _p(w2_EDF),
             _p(gate), _p(up), _dt(x_TD), _p(plan.seg_offsets), _p(plan.seg_counts), _p(plan.tile_expert),
             _p(plan.tile_row0), _p(plan.num_tiles), plan.tile_capacity, _p(dgate), _p(dup), _p(hs), _p(partial),
-            _p(drows), _p(dw1), _p(dw3), _p(dw2), El, D, F, R, _stream(dev),
+            _p(drows), _p(dw1), _p(dw3), _p(dw2), El, D, F, R, 0, _stream(dev),
         )
-        _lib.check(rc, "grouped_swiglu_combine_bwd")
-        rc = lib.mi355_combine_scores_bwd(
-            _p(partial), slots, _p(plan.row_of_slot), _p(dweights), plan.num_tokens, plan.top_k, R, _stream(dev),
-        )
-    _lib.check(rc, "combine_scores_bwd")
-    return drows, dw1, dw3, dw2, dweights
+    _lib.check(rc, "grouped_swiglu_combine_bwd")
+    return drows, dw1, dw3, dw2, combine_scores_bwd(partial, plan)
 
 
 STAGES = {"gate_up": 1, "down": 2, "dh": 4, "drows": 8, "dw2": 16, "dw1": 32, "dw3": 64}
+
+
+def grouped_swiglu_combine_stage(stage: str, buf: dict, plan: PermutePlan):
+    """One backward kernel of the folded experts+combine backward on pre-allocated buffers.
+
+    ``buf`` maps dout, rows (the (T, D) tokens), row_scale, w1, w3, w2, gate, up, dgate, dup,
+    hs, dot_partial, drows, dw1, dw3, dw2 to device tensors; ``stage`` is one of dh, drows,
+    dw2, dw1, dw3.
+    """
+    x = buf["rows"]
+    dev = _dev(x)
+    D = x.shape[1]
+    R = buf["gate"].shape[0]
+    El, F, _ = buf["w1"].shape
+    g = lambda k: _p(buf.get(k))
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_grouped_swiglu_combine_bwd(
+            g("dout"), g("rows"), _p(plan.token_of_row), g("row_scale"), g("w1"), g("w3"), g("w2"), g("gate"),
+            g("up"), _dt(x), _p(plan.seg_offsets), _p(plan.seg_counts), _p(plan.tile_expert), _p(plan.tile_row0),
+            _p(plan.num_tiles), plan.tile_capacity, g("dgate"), g("dup"), g("hs"), g("dot_partial"), g("drows"),
+            g("dw1"), g("dw3"), g("dw2"), El, D, F, R, STAGES[stage], _stream(dev),
+        )
+    _lib.check(rc, f"grouped_swiglu_combine_bwd[{stage}]")
+
+
+def combine_scores_bwd(dot_partial, plan: PermutePlan):
+    dev = _dev(dot_partial)
+    dweights = torch.empty(plan.num_tokens, plan.top_k, dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_combine_scores_bwd(
+            _p(dot_partial), dot_partial.shape[1], _p(plan.row_of_slot), _p(dweights), plan.num_tokens, plan.top_k,
+            dot_partial.shape[0], _stream(dev),
+        )
+    _lib.check(rc, "combine_scores_bwd")
+    return dweights
 
 
 def grouped_swiglu_stage(stage: str, buf: dict, plan: PermutePlan):
