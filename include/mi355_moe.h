@@ -209,8 +209,11 @@ int mi355_balance_loss_bwd(const float* scores_TE, const float* f_E,
  *                 unused; optional (NULL = skip): the gather index of the fused expert
  *                 kernels below
  *   tile_expert, tile_row0 (tile_capacity each) and num_tiles (1): the list of
- *       tile_m-row tiles covering the real rows of every segment (local expert
- *       index and first row of each tile)
+ *       row tiles covering the real rows of every segment (local expert index and
+ *       first row of each tile).  A segment of c rows has ceil(c / tile_m) tiles, all
+ *       of the same height ceil(c / that number) rounded up to 16 rows (at most
+ *       tile_m; the last one ends with the segment): equal tiles of an expert run in
+ *       step and share its weights in L2, a short rest tile would not
  * row_capacity  >= N + El*(align-1) is always enough;
  * tile_capacity >= N/tile_m + El + 1 is always enough.
  * workspace: mi355_permute_plan_workspace_bytes(T,K,E) bytes.

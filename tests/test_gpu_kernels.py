@@ -161,7 +161,11 @@ def test_permute_plan_is_the_stable_argsort(ops, T, K, E, align, local):
     # tile list covers exactly the real rows
     nt = int(plan.num_tiles.item()); tm = plan.tile_m
     te, tr = plan.tile_expert.cpu()[:nt].long(), plan.tile_row0.cpu()[:nt].long()
-    exp_tiles = [(j, int(seg_off[j]) + i * tm) for j in range(hi - lo) for i in range((int(lc[j]) + tm - 1) // tm)]
+    def tile_rows(c):  # an expert's tiles are equally tall, to a multiple of 16 rows
+        n = (c + tm - 1) // tm
+        return tm if n <= 1 else (-(-c // n) + 15) // 16 * 16
+    exp_tiles = [(j, int(seg_off[j]) + i * tile_rows(int(lc[j]))) for j in range(hi - lo)
+                 for i in range((int(lc[j]) + tm - 1) // tm)]
     assert list(zip(te.tolist(), tr.tolist())) == exp_tiles
     assert total <= plan.row_capacity
 

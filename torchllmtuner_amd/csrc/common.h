@@ -62,6 +62,19 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 }
 __device__ __forceinline__ float round_bf16(float f) { return bf16_to_f32(f32_to_bf16(f)); }
 
+// Height of the row tiles of a segment of `count` rows: its ceil(count / tile_m) tiles are made
+// equally tall (to a multiple of the 16-row MFMA block) instead of tile_m, tile_m, ..., rest.
+// A rest of a few rows costs most of a full tile (its weight tile is staged all the same) and
+// runs out of step with its neighbours, which then miss each other's operands in L2; equal
+// tiles cost their share of the rows and stay in step.  Never more than tile_m, never leaves
+// a tile empty.  The plan kernels and every kernel that walks the tile list use this one rule.
+__host__ __device__ inline int even_tile_rows(int count, int tile_m) {
+  const int nt = (count + tile_m - 1) / tile_m;
+  if (nt <= 1) return tile_m;
+  const int per = (count + nt - 1) / nt;
+  return (per + 15) / 16 * 16;
+}
+
 template <typename T>
 __device__ __forceinline__ float load_as_f32(const T* p);
 template <>

@@ -44,8 +44,10 @@ __global__ __launch_bounds__(256) void ggemm_kernel(GemmArgs g) {
     if (tile >= *g.num_tiles) return;
     const int e = g.tile_expert[tile];
     const int r0 = g.tile_row0[tile] + sub * TM;
-    const int seg_end = g.seg_offsets[e] + g.seg_counts[e];
-    m_valid = min(TM, seg_end - r0);
+    // the tile's rows end with its (equalised) height or with the segment
+    const int cnt = g.seg_counts[e];
+    const int tile_end = min(g.tile_row0[tile] + even_tile_rows(cnt, g.tile_m), g.seg_offsets[e] + cnt);
+    m_valid = min(TM, tile_end - r0);
     if (m_valid <= 0) return;
     row_base = r0;
     m0 = 0;

@@ -166,7 +166,8 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
     // would wait for all of those
     m.e = ((const_i32)p.tile_expert)[tile];
     m.row0 = ((const_i32)p.tile_row0)[tile];
-    m.valid = min(TBM, ((const_i32)p.seg_offsets)[m.e] + ((const_i32)p.seg_counts)[m.e] - m.row0);
+    const int cnt_e = ((const_i32)p.seg_counts)[m.e];
+    m.valid = min(even_tile_rows(cnt_e, TBM), ((const_i32)p.seg_offsets)[m.e] + cnt_e - m.row0);
     // a last tile that would overhang starts early instead and recomputes a few columns
     // of its neighbour (same values), so no column is ever clamped
     constexpr int W = (MODE == RM_GATEUP ? BNT / 2 : BNT);

@@ -161,11 +161,12 @@ __global__ __launch_bounds__(1024) void plan_scan_kernel(
   for (int j = tid; j < El; j += blockDim.x) {
     const int c = cnt_sh[lo + j];
     const int nt = (c + tile_m - 1) / tile_m;
+    const int rows = even_tile_rows(c, tile_m);
     for (int i = 0; i < nt; ++i) {
       const int idx = tile_off_sh[j] + i;
       if (idx < tile_capacity) {
         tile_expert[idx] = j;
-        tile_row0[idx] = seg_off_sh[j] + i * tile_m;
+        tile_row0[idx] = seg_off_sh[j] + i * rows;
       }
     }
   }
@@ -218,11 +219,12 @@ __global__ __launch_bounds__(256) void segments_from_counts_kernel(
     const int c = cnt_sh[j];
     seg_counts[j] = c;
     const int nt = (c + tile_m - 1) / tile_m;
+    const int rows = even_tile_rows(c, tile_m);
     for (int i = 0; i < nt; ++i) {
       const int idx = tile_off_sh[j] + i;
       if (idx < tile_capacity) {
         tile_expert[idx] = j;
-        tile_row0[idx] = seg_off_sh[j] + i * tile_m;
+        tile_row0[idx] = seg_off_sh[j] + i * rows;
       }
     }
   }
