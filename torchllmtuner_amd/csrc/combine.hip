@@ -83,16 +83,31 @@ __global__ __launch_bounds__(256) void combine_fwd_kernel(
       float a[V];
 #pragma unroll
       for (int q = 0; q < V; ++q) a[q] = 0.0f;
-      for (int p = 0; p < nvalid; ++p) {
-        const int r = __shfl(o_row, p, kWave);
-        const float ww = __shfl(o_w, p, kWave);
-        if (!on) continue;
-        float f[V];
-        Vec<T>::unpack(reinterpret_cast<const uint4*>(y + static_cast<int64_t>(r) * D)[i], f);
+      // eight rows requested before the first is used (one load at a time leaves a wave with
+      // 1 KiB in flight); the terms are still added in visiting order
+      constexpr int B = 8;
+      for (int p0 = 0; p0 < nvalid; p0 += B) {
+        uint4 v[B];
+        float ww[B];
 #pragma unroll
-        for (int q = 0; q < V; ++q) {
-          const float term = f[q] * ww;
-          a[q] += round_terms ? round_to<T>(term) : term;
+        for (int j = 0; j < B; ++j) {
+          const int p = min(p0 + j, nvalid - 1);  // past the end: the last row again, not used
+          const int r = __shfl(o_row, p, kWave);
+          ww[j] = __shfl(o_w, p, kWave);
+          v[j] = make_uint4(0, 0, 0, 0);
+          if (on && p0 + j < nvalid) v[j] = reinterpret_cast<const uint4*>(y + static_cast<int64_t>(r) * D)[i];
+        }
+#pragma unroll
+        for (int j = 0; j < B; ++j) {
+          if (p0 + j < nvalid) {
+            float f[V];
+            Vec<T>::unpack(v[j], f);
+#pragma unroll
+            for (int q = 0; q < V; ++q) {
+              const float term = f[q] * ww[j];
+              a[q] += round_terms ? round_to<T>(term) : term;
+            }
+          }
         }
       }
       if (on) reinterpret_cast<uint4*>(dst)[i] = Vec<T>::pack(a);

@@ -336,10 +336,21 @@ __global__ __launch_bounds__(256) void permute_rows_bwd_kernel(
       float a[V];
 #pragma unroll
       for (int q = 0; q < V; ++q) a[q] = 0.0f;
-      for (int k = 0; k < K; ++k) {
-        const int row = __shfl(my_row, k, kWave);
-        if (row < 0 || !on) continue;
-        acc_vec<T>(a, reinterpret_cast<const uint4*>(drows + static_cast<int64_t>(row) * D)[i]);
+      // eight rows requested before the first is summed: one load at a time leaves a wave
+      // with 1 KiB in flight, too little to keep HBM busy; the sum still runs in ascending k
+      constexpr int B = 8;
+      for (int k0 = 0; k0 < K; k0 += B) {
+        uint4 v[B];
+#pragma unroll
+        for (int j = 0; j < B; ++j) {
+          const int k = k0 + j;
+          const int row = __shfl(my_row, k < K ? k : 0, kWave);
+          v[j] = make_uint4(0, 0, 0, 0);
+          if (k < K && row >= 0 && on)
+            v[j] = reinterpret_cast<const uint4*>(drows + static_cast<int64_t>(row) * D)[i];
+        }
+#pragma unroll
+        for (int j = 0; j < B; ++j) acc_vec<T>(a, v[j]);  // absent rows add zeros
       }
       if (on) reinterpret_cast<uint4*>(dst)[i] = pack_vec<T>(a);
     }
