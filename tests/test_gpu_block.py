@@ -66,10 +66,16 @@ def test_c1_tiny_fp32_forward_backward():
         assert rel_max(got[k], want[k]) < 1e-5, f"{k}: {rel_max(got[k], want[k])}"
 
 
-@pytest.mark.parametrize("dispatcher,T", [("local", 1024), ("padded", 1536)])
-def test_qwen3_shape_bf16_forward_backward(dispatcher, T):
-    """hidden 2048, 128 experts, top-8, intermediate 768, softmax + norm, bf16."""
-    print(f"block qwen3 bf16 {dispatcher} T={T}", flush=True)
+@pytest.mark.parametrize("dispatcher,T,fold", [("local", 1024, True), ("padded", 1536, True), ("local", 1024, False)])
+def test_qwen3_shape_bf16_forward_backward(dispatcher, T, fold, monkeypatch):
+    """hidden 2048, 128 experts, top-8, intermediate 768, softmax + norm, bf16.
+
+    fold: the backward of experts + combine as one pass (the default where it applies), or the
+    two-call form (combine's backward, then the experts') that other layouts and dtypes use."""
+    print(f"block qwen3 bf16 {dispatcher} T={T} fold={fold}", flush=True)
+    from torchllmtuner_amd import ops as _ops
+    monkeypatch.setattr(_ops, "FOLD_COMBINE", fold)
+    assert (_ops.combine_bwd_slots(torch.bfloat16, 2048, 768) > 0) == fold
     D, E, K, F = 2048, 128, 8, 768
     spec = R.RouterSpec(E, K, score_func="softmax", route_norm=True)
     p = make_params(E, D, F, torch.bfloat16, seed=0)
@@ -156,6 +162,38 @@ def test_block_api_contract():
     assert [k for k in block.state_dict()] == [
         "expert_bias_E", "routed_experts.inner_experts.w1_EFD", "routed_experts.inner_experts.w3_EFD",
         "routed_experts.inner_experts.w2_EDF", "router.gate.weight"]
+
+
+@pytest.mark.parametrize("fold", [True, False])
+@pytest.mark.parametrize("T", [0, 3])
+def test_bf16_block_with_no_or_few_tokens(T, fold, monkeypatch):
+    """The MFMA path with nothing or almost nothing to do: no tokens at all (every weight
+    gradient is zeros, dx is empty) and three tokens (most experts have no rows)."""
+    print(f"block bf16 edge T={T} fold={fold}", flush=True)
+    from torchllmtuner_amd import ops as _ops
+    monkeypatch.setattr(_ops, "FOLD_COMBINE", fold)
+    D, E, K, F = 384, 16, 2, 384
+    spec = R.RouterSpec(E, K, score_func="softmax", route_norm=True)
+    p = make_params(E, D, F, torch.bfloat16, seed=5)
+    x = torch.randn(T, D, generator=torch.Generator().manual_seed(0)).bfloat16()
+    gout = torch.randn(T, D, generator=torch.Generator().manual_seed(1)).bfloat16()
+    got, want, aux, block = _run_pair(p, spec, x, gout, torch.bfloat16, D, F)
+    assert got["out"].shape == (T, D)
+    ie = block.routed_experts.inner_experts
+    for w in (ie.w1_EFD, ie.w3_EFD, ie.w2_EDF, block.router.gate.weight):
+        assert w.grad is not None and bool(torch.isfinite(w.grad.float()).all())
+    if T == 0:
+        for w in (ie.w1_EFD, ie.w3_EFD, ie.w2_EDF):
+            assert not bool(w.grad.any())
+        return
+    counts = aux["counts_E"]
+    unused = (counts == 0).nonzero().squeeze(-1)
+    assert unused.numel() >= E - T * K
+    for w in (ie.w1_EFD, ie.w3_EFD, ie.w2_EDF):
+        assert not bool(w.grad[unused.to(DEV)].any()), "experts without rows get zero gradients"
+    for k in want:
+        err = rel_l2(got[k], want[k])
+        assert err < 2e-2, f"{k}: rel-L2 {err}"
 
 
 def test_dispatcher_api_matches_reference_contract():

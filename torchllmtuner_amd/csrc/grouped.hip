@@ -179,7 +179,8 @@ extern "C" int mi355_grouped_swiglu_bwd(const void* dy, const void* rows,
     return bf16_grouped_bwd(
         dy, rows, token_of_row, w1, w3, w2, gate, up, h, nullptr, nullptr, seg_offsets, seg_counts, tile_expert,
         tile_row0, num_tiles, tile_capacity, dgate, dup, drows, dw1, dw3, dw2, El, D, F, 0x7c, s);
-  if (token_of_row)
+  // (with no rows at all nothing is gathered: only the zero weight gradients remain to be written)
+  if (token_of_row && row_capacity > 0 && tile_capacity > 0)
     return fail(MI355_EUNSUP, "grouped_swiglu_bwd: the token gather needs bf16 with D and F multiples of 64");
   const Seg sg{seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles, tile_capacity};
   if (row_capacity > 0 && tile_capacity > 0) {
