@@ -155,7 +155,7 @@ class MoE(nn.Module):
         if self.training and not in_checkpoint_recompute.get():
             with torch.no_grad():
                 if padding_mask is None:
-                    valid_counts_E = plan.counts_E.to(torch.float32)
+                    valid_counts_E = plan.counts_E  # int32; add_ promotes inside its one kernel
                 else:
                     keep = (~padding_mask).to(torch.float32).repeat_interleave(plan.top_k)
                     valid_counts_E = torch.zeros_like(self.tokens_per_expert_E).scatter_add_(
