@@ -30,8 +30,8 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # WRITE_SIZE (scaled by a 256 MiB copy: x2.0 and x1.0); the table these come from is
 # profiles/moe_layer_qwen3_t8192_hbm_traffic.txt.  Only reported for the default workload.
 MEASURED_HBM_BYTES = {
-    "gate_up": 1697.6e6, "down": 971.9e6, "dh": 1281.1e6, "drows": 1761.2e6,
-    "dw2": 829.2e6, "dw1": 896.0e6, "dw3": 896.0e6,
+    "gate_up": 1511.8e6, "down": 844.8e6, "dh": 1255.4e6, "drows": 1434.6e6,
+    "dw2": 828.0e6, "dw1": 895.9e6, "dw3": 895.9e6,
 }
 
 WORKLOADS = {

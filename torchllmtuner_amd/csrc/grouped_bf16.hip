@@ -159,15 +159,32 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
   auto exists = [&](int w) { return w < chunk && pid_base + w < total; };
   auto load_meta = [&](int w) -> TileMeta {
     const int pid = pid_base + w;
-    const int tile = pid / p.n_tiles, nt = pid % p.n_tiles;
-    TileMeta m;
     // scalar loads (constant address space): as vector loads these lookups would share the
     // counter of the operand stream and of the epilogue stores, and waiting for one of them
     // would wait for all of those
-    m.e = ((const_i32)p.tile_expert)[tile];
-    m.row0 = ((const_i32)p.tile_row0)[tile];
-    const int cnt_e = ((const_i32)p.seg_counts)[m.e];
-    m.valid = min(even_tile_rows(cnt_e, TBM), ((const_i32)p.seg_offsets)[m.e] + cnt_e - m.row0);
+    const int t = pid / p.n_tiles;  // some tile of the expert this work item belongs to
+    TileMeta m;
+    m.e = ((const_i32)p.tile_expert)[t];
+    const int cnt_e = ((const_i32)p.seg_counts)[m.e], off_e = ((const_i32)p.seg_offsets)[m.e];
+    const int h = even_tile_rows(cnt_e, TBM);
+    const int nrt = max((cnt_e + TBM - 1) / TBM, 1);  // row tiles of the expert
+    // Within an expert the work items run column-tile-major over groups of three row tiles:
+    // the row tiles of one column tile are neighbours, so the weight tile they share -- the
+    // larger operand: an expert's weights are several times its rows -- is in L2 when the next
+    // one asks for it, and a row tile's column tiles are still at most 3 x n_tiles work items
+    // apart, inside what an XCD has in flight.  Row-tile-major throughout (neighbours share
+    // the row tile only) left a quarter of the weight tiles to be fetched twice;
+    // column-tile-major throughout fetches the rows of an expert with many row tiles once per
+    // column tile.
+    constexpr int G = 3;
+    const int t0 = t - (((const_i32)p.tile_row0)[t] - off_e) / h;  // the expert's first tile
+    const int q = pid - t0 * p.n_tiles;
+    const int blk = q / (G * p.n_tiles);
+    const int qb = q - blk * (G * p.n_tiles);
+    const int g = min(G, nrt - blk * G);  // row tiles of this group (>= 1)
+    const int nt = qb / g, rt = blk * G + (qb - nt * g);
+    m.row0 = off_e + rt * h;
+    m.valid = min(h, cnt_e - rt * h);
     // a last tile that would overhang starts early instead and recomputes a few columns
     // of its neighbour (same values), so no column is ever clamped
     constexpr int W = (MODE == RM_GATEUP ? BNT / 2 : BNT);
