@@ -221,11 +221,10 @@ class GatherExpertsCombineFunction(torch.autograd.Function):
     def backward(ctx, dout):
         x, weights, w1, w3, w2, gate, up = ctx.saved_tensors
         row_scale = ops.combine_row_scale(weights, ctx.plan)
-        drows, dw1, dw3, dw2, dweights = ops.grouped_swiglu_combine_bwd(
+        dx, dw1, dw3, dw2, dweights = ops.grouped_swiglu_combine_bwd(
             dout, x, row_scale, w1, w3, w2, gate, up, ctx.plan,
-            need_drows=ctx.needs_input_grad[0], need_dw=any(ctx.needs_input_grad[2:5]),
+            need_drows=ctx.needs_input_grad[0], need_dw=any(ctx.needs_input_grad[2:5]), sum_rows=True,
         )
-        dx = ops.permute_rows_bwd(drows, ctx.plan) if drows is not None else None
         return dx, dweights.to(weights.dtype), dw1, dw3, dw2, None, None
 
 

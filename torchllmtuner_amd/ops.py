@@ -533,8 +533,14 @@ def combine_row_scale(weights_TK, plan: PermutePlan):
 
 
 def grouped_swiglu_combine_bwd(dout_TD, x_TD, row_scale_R, w1_EFD, w3_EFD, w2_EDF, gate, up, plan: PermutePlan,
-                               need_drows=True, need_dw=True):
-    """Backward of gathered experts + combine in one pass; returns (drows, dw1, dw3, dw2, dweights_TK)."""
+                               need_drows=True, need_dw=True, sum_rows=False):
+    """Backward of gathered experts + combine in one pass; returns (drows, dw1, dw3, dw2, dweights_TK).
+
+    ``sum_rows``: return ``dx`` (T, D), the K-way row sum of ``drows``, in its place.  The sum
+    then runs right behind the kernel that wrote ``drows``, while those rows are still in the
+    memory-side cache, and the weight-gradient kernels follow; summed after them it finds its
+    input gone to HBM.
+    """
     dev = _dev(dout_TD, x_TD)
     dout_TD, x_TD = _c(dout_TD), _c(x_TD)
     if dout_TD.dtype != x_TD.dtype:
@@ -553,15 +559,26 @@ def grouped_swiglu_combine_bwd(dout_TD, x_TD, row_scale_R, w1_EFD, w3_EFD, w2_ED
     dw1 = torch.empty_like(w1_EFD) if need_dw else None
     dw3 = torch.empty_like(w3_EFD) if need_dw else None
     dw2 = torch.empty_like(w2_EDF) if need_dw else None
-    with torch.cuda.device(dev):
-        rc = lib.mi355_grouped_swiglu_combine_bwd(
-            _p(dout_TD), _p(x_TD), _p(plan.token_of_row), _p(row_scale_R), _p(w1_EFD), _p(w3_EFD), _p(w2_EDF),
-            _p(gate), _p(up), _dt(x_TD), _p(plan.seg_offsets), _p(plan.seg_counts), _p(plan.tile_expert),
-            _p(plan.tile_row0), _p(plan.num_tiles), plan.tile_capacity, _p(dgate), _p(dup), _p(hs), _p(partial),
-            _p(drows), _p(dw1), _p(dw3), _p(dw2), El, D, F, R, 0, _stream(dev),
-        )
-    _lib.check(rc, "grouped_swiglu_combine_bwd")
-    return drows, dw1, dw3, dw2, combine_scores_bwd(partial, plan)
+    def run(stages):
+        with torch.cuda.device(dev):
+            rc = lib.mi355_grouped_swiglu_combine_bwd(
+                _p(dout_TD), _p(x_TD), _p(plan.token_of_row), _p(row_scale_R), _p(w1_EFD), _p(w3_EFD), _p(w2_EDF),
+                _p(gate), _p(up), _dt(x_TD), _p(plan.seg_offsets), _p(plan.seg_counts), _p(plan.tile_expert),
+                _p(plan.tile_row0), _p(plan.num_tiles), plan.tile_capacity, _p(dgate), _p(dup), _p(hs), _p(partial),
+                _p(drows), _p(dw1), _p(dw3), _p(dw2), El, D, F, R, stages, _stream(dev),
+            )
+        _lib.check(rc, "grouped_swiglu_combine_bwd")
+
+    if not (sum_rows and need_drows and need_dw and R > 0):
+        run(0)
+        if sum_rows and drows is not None:
+            drows = permute_rows_bwd(drows, plan)
+        return drows, dw1, dw3, dw2, combine_scores_bwd(partial, plan)
+    run(STAGES["dh"] | STAGES["drows"])
+    dx = permute_rows_bwd(drows, plan)
+    dweights = combine_scores_bwd(partial, plan)
+    run(STAGES["dw2"] | STAGES["dw1"] | STAGES["dw3"])
+    return dx, dw1, dw3, dw2, dweights
 
 
 STAGES = {"gate_up": 1, "down": 2, "dh": 4, "drows": 8, "dw2": 16, "dw1": 32, "dw3": 64}
