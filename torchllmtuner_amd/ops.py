@@ -7,9 +7,8 @@ implementation.
 
 from __future__ import annotations
 
-from dataclasses import dataclass
-
 import os
+from dataclasses import dataclass
 
 import torch
 
