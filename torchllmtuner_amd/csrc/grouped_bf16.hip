@@ -790,6 +790,11 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
       uint16_t* Bn = An + WBM * BK;
 #pragma unroll
       for (int kk = 0; kk < BK / 16; ++kk) {
+        // the last K step of a segment is usually ragged: its 16-row slices past the last real
+        // row hold zeros and are skipped (workgroup-uniform; only this instantiation branches)
+        if constexpr (!has_next) {
+          if (ks * BK + kk * 16 >= c_cnt) continue;
+        }
         bf16x8 af[2], bf[4];
 #pragma unroll
         for (int mi = 0; mi < 2; ++mi) af[mi] = frag_ks<256>(As, wm + mi * 32, kk, lane);
