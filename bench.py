@@ -1,14 +1,20 @@
 #!/usr/bin/env python3
-"""Benchmark: MoE layer forward+backward tokens/s at the Qwen3-30B-A3B shape.
+"""Benchmark: MoE layer tokens/s on one MI355X, at each of the five workload shapes.
 
-One step = one forward + backward of the MoE block (router, permute, grouped
-SwiGLU experts, combine and every gradient: dX, dW1/dW3/dW2, dW_router) over one
-batch of T tokens that is already resident in HBM.  Prints one JSON line.
+One step = one pass of the MoE block (router, permute, grouped SwiGLU experts, combine; with
+the backward every gradient: dX, dW1/dW3/dW2, dW_router, shared-expert weights) over one batch
+of tokens that is already resident in HBM.  Prints one JSON line.
 
-Besides the whole-step rate it reports, for the dominant kernel, the achieved
-fraction of its roofline (timed alone with HIP events on the launch stream) and a
-CPU baseline: the oracle restatement of the reference block timed on this
-machine's host cores over a bounded token sample.
+``--workload c3`` (the default) is the headline: the Qwen3-30B-A3B-shaped layer, T=8192,
+forward + backward in bf16.  c1 (tiny fp32), c2 (forward only), c4 (T=16384, skewed routing,
+128-row padded segments) and c5 (DeepSeek-V3 shape, one rank's expert share, shared expert) are
+the other configurations; all are built by ``torchllmtuner_amd.workloads`` from the product's
+own modules.
+
+Besides the whole-step rate the line carries per-kernel times (HIP events on the launch
+stream), the roofline fraction of the kernel that takes the largest share of the step, and a
+CPU baseline: the oracle restatement of the reference block timed on this machine's host cores
+over a bounded token sample (warm-up, then the median of three runs).
 """
 
 from __future__ import annotations
@@ -16,6 +22,7 @@ from __future__ import annotations
 import argparse
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -24,19 +31,14 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_FP32_TFLOPS = 157.3   # MI355X dense fp32 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 
-# HBM bytes per launch at the default workload, measured with rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE (scaled by a 256 MiB copy: x2.0 and x1.0); the table these come from is
-# profiles/moe_layer_qwen3_t8192_hbm_traffic.txt.  Only reported for the default workload.
+# HBM bytes per launch, measured with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (scaled by a
+# 256 MiB copy: x2.0 and x1.0); the tables these come from are profiles/*_hbm_traffic.txt.
 MEASURED_HBM_BYTES = {
-    "gate_up": 1511.8e6, "down": 844.8e6, "dh": 1255.4e6, "drows": 1434.6e6,
-    "dw2": 828.0e6, "dw1": 895.9e6, "dw3": 895.9e6,
-}
-
-WORKLOADS = {
-    # name: T, D, E, K, F
-    "qwen3-30b-a3b-moe-layer fwd+bwd T=8192 bf16": dict(T=8192, D=2048, E=128, K=8, F=768),
+    "c3": {"gate_up": 1511.8e6, "down": 844.8e6, "dh": 1255.4e6, "drows": 1434.6e6,
+           "dw2": 828.0e6, "dw1": 895.9e6, "dw3": 895.9e6},
 }
 
 
@@ -45,12 +47,12 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--tokens", type=int, default=8192)
+    ap.add_argument("--workload", choices=["c1", "c2", "c3", "c4", "c5"], default="c3")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-sample-tokens", type=int, default=1024)
+    ap.add_argument("--cpu-sample-tokens", type=int, default=512)
     ap.add_argument("--stage-iters", type=int, default=10)
     ap.add_argument("--no-probe", action="store_true",
-                    help="skip the sustained-MFMA probe (about 0.8 s of matrix-core work)")
+                    help="skip the sustained-MFMA probe (about 0.8 s of matrix-core work) and the vendor GEMM")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (known traffic, for scaling rocprof FETCH_SIZE / WRITE_SIZE)")
     return ap.parse_args()
@@ -74,14 +76,14 @@ def time_events(fn, iters, warmup=2):
 
 
 def sustained_mfma(dev):
-    """What the matrix cores hold on v_mfma_f32_32x32x16_bf16 with register-resident
-    operands of random bits (libmi355probe.so): rate and core clock, both under the
-    card's own power management.  Returns None when the probe library is not built."""
+    """What the matrix cores hold on the two MFMA shapes the grouped GEMMs use, with
+    register-resident operands of random bits (bench_probe/libmi355probe.so): rate and core
+    clock, both under the card's own power management.  None when the probe is not built."""
     import ctypes
 
     import torch
 
-    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "torchllmtuner_amd", "libmi355probe.so")
+    path = os.path.join(ROOT, "bench_probe", "libmi355probe.so")
     if not os.path.exists(path):
         return None
     lib = ctypes.CDLL(path)
@@ -108,40 +110,232 @@ def sustained_mfma(dev):
     return out
 
 
-def cpu_baseline(cfg, sample_tokens):
-    """The oracle's forward+backward on host cores over ``sample_tokens`` tokens."""
+def cpu_baseline(wl, sample_tokens):
+    """The oracle's pass (forward, + backward where the workload has one) on host cores:
+    a warm-up, then the median of three runs, over ``sample_tokens`` tokens of the workload's
+    layer (the full C1 block when it is that small); bf16 workloads are timed in fp32 as well."""
     import torch
 
     from oracle import moe_ref as R
-    from tests.helpers import make_params
+    from torchllmtuner_amd import workloads as W
 
     cores = os.cpu_count() or 1
     cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
     torch.set_num_threads(cores)
-    D, E, K, F = cfg["D"], cfg["E"], cfg["K"], cfg["F"]
-    spec = R.RouterSpec(E, K, score_func="softmax", route_norm=True)
-    p = make_params(E, D, F, torch.bfloat16, seed=0)
-    for name in ("router_w_ED", "w1_EFD", "w3_EFD", "w2_EDF"):
-        getattr(p, name).requires_grad_()
 
-    def run(tokens):
-        x = torch.randn(tokens, D, generator=torch.Generator().manual_seed(0)).bfloat16().requires_grad_()
-        g = torch.randn(tokens, D, generator=torch.Generator().manual_seed(1)).bfloat16()
-        t0 = time.perf_counter()
-        out, _ = R.moe_forward(x, p, spec)
-        out.backward(g)
-        return time.perf_counter() - t0
+    def measure(wl, tokens, dtype):
+        w = W.make_weights(wl)
+        cast = lambda t: t.to(dtype)
+        p = R.MoEParams(router_w_ED=w["router"].clone(), w1_EFD=cast(w["w1"]), w3_EFD=cast(w["w3"]),
+                        w2_EDF=cast(w["w2"]))
+        if wl.shared_hidden_dim:
+            p.shared_gate_FD, p.shared_up_FD, p.shared_down_DF = (cast(w[k]) for k in
+                                                                  ("shared_gate", "shared_up", "shared_down"))
+        if wl.expert_bias:
+            p.expert_bias_E = w["expert_bias"]
+        leaves = [getattr(p, n) for n in ("router_w_ED", "w1_EFD", "w3_EFD", "w2_EDF", "shared_gate_FD", "shared_up_FD",
+                                          "shared_down_DF") if getattr(p, n) is not None]
+        for t in leaves:
+            t.requires_grad_(wl.backward)
+        spec = R.RouterSpec(wl.num_experts, wl.top_k, score_func=wl.score_func, route_norm=wl.route_norm,
+                            route_scale=wl.route_scale, num_expert_groups=wl.num_expert_groups,
+                            num_limited_groups=wl.num_limited_groups)
+        kw = {}
+        if wl.pad_multiple:
+            kw["pad_multiple"] = wl.pad_multiple
+        if wl.local_experts:
+            kw["local_experts"] = wl.local_experts
 
-    run(128)  # warm-up: thread pool, allocator
-    dt = run(sample_tokens)
-    return {
-        "value": sample_tokens / dt,
+        def run(n):
+            x = torch.randn(n, wl.dim, generator=torch.Generator().manual_seed(0)).to(dtype).requires_grad_(wl.backward)
+            g = torch.randn(n, wl.dim, generator=torch.Generator().manual_seed(1)).to(dtype)
+            for t in leaves:
+                t.grad = None
+            t0 = time.perf_counter()
+            with torch.set_grad_enabled(wl.backward):
+                out, _ = R.moe_forward(x, p, spec, **kw)
+                if wl.backward:
+                    out.backward(g)
+            return time.perf_counter() - t0
+
+        run(min(128, tokens))  # warm-up: thread pool, allocator
+        times = [run(tokens) for _ in range(3)]
+        return tokens / statistics.median(times), times
+
+    tokens = min(sample_tokens, wl.tokens)
+    rate, times = measure(wl, tokens, wl.dtype)
+    name = {torch.float32: "fp32", torch.bfloat16: "bf16"}[wl.dtype]
+    out = {
+        "value": round(rate, 2),
         "unit": "tokens/s",
         "cores": cores,
         "kind": "port",
-        "sample": f"oracle fwd+bwd, {sample_tokens} tokens of the same layer (D={D},E={E},K={K},F={F}), "
-                  f"bf16, 1 run after a 128-token warm-up, {dt:.2f} s",
+        "sample": f"oracle {'fwd+bwd' if wl.backward else 'fwd'}, {tokens} tokens of the {wl.key} layer "
+                  f"(D={wl.dim},E={wl.num_experts},K={wl.top_k},F={wl.hidden_dim}), {name}, 128-token warm-up then "
+                  f"the median of 3 runs ({', '.join(f'{t:.2f}' for t in times)} s)",
     }
+    if wl.dtype == torch.bfloat16:
+        rate32, times32 = measure(wl, tokens, torch.float32)
+        out["fp32"] = {"value": round(rate32, 2), "unit": "tokens/s",
+                       "sample": f"the same sample with fp32 weights and activations "
+                                 f"({', '.join(f'{t:.2f}' for t in times32)} s)"}
+    if wl.key != "c1":
+        c1 = W.WORKLOADS["c1"]
+        rate1, times1 = measure(c1, c1.tokens, c1.dtype)
+        out["c1_full_size"] = {"value": round(rate1, 1), "unit": "tokens/s",
+                               "sample": f"oracle fwd+bwd of the whole C1 block (T={c1.tokens}, fp32), median of 3"}
+    return out
+
+
+def per_kernel_times(args, wl, block, x, gout, dev):
+    """HIP-event averages of the kernels of one step, each launched alone on the buffers of a
+    real step.  Returns (kernels, stage_ms, stage_flops, routed_rows)."""
+    import torch
+
+    from torchllmtuner_amd import ops
+
+    it = args.stage_iters
+    T, D, E, K, F = x.shape[0], wl.dim, wl.num_experts, wl.top_k, wl.hidden_dim
+    s_bytes = x.element_size()
+    peak = PEAK_BF16_TFLOPS if wl.dtype == torch.bfloat16 else PEAK_FP32_TFLOPS
+    with torch.no_grad():
+        scores, ids = block.router.route(x, block.expert_bias_E)
+        plan = block.routed_experts.token_dispatcher.plan(ids)
+        R_rows = int(plan.seg_counts.sum().item())       # real rows
+        R_cover = int(plan.total_rows.item())            # rows in use, padding included
+        ie = block.routed_experts.inner_experts
+        w1, w3, w2 = ie.w1_EFD.detach(), ie.w3_EFD.detach(), ie.w2_EDF.detach()
+        rows = ops.permute_rows_fwd(x, plan)
+        y, gate, up, h = ops.grouped_swiglu_fwd(rows, w1, w3, w2, plan)
+        dy, _ = ops.combine_bwd(gout, y, scores, plan)
+        logits = ops.router_gate_fwd(x, block.router.gate.weight, block.router.gate.bias)
+        proj = 2.0 * R_rows * D * F
+        stage_flops = {"gate_up": 2 * proj, "down": proj, "dh": proj, "drows": 2 * proj,
+                       "dw2": proj, "dw1": proj, "dw3": proj}
+        if not wl.backward:
+            stage_flops = {k: stage_flops[k] for k in ("gate_up", "down")}
+        stage_ms = {}
+        folded = ops.gather_supported(x, F) and ops.combine_bwd_slots(x.dtype, D, F) > 0
+        if folded:
+            # as in the step: the token matrix is read through the gather index (gate/up A operand,
+            # dW1/dW3 B operand), dH reads the output gradient through it and scales rows in its
+            # epilogue, dW2 contracts the gathered rows with score * h
+            buf = dict(rows=x, token_of_row=plan.token_of_row, w1=w1, w3=w3, w2=w2, gate=gate, up=up, h=h, y=y,
+                       dy=dy, dgate=torch.empty_like(gate), dup=torch.empty_like(up), drows=torch.empty_like(rows),
+                       dw1=torch.empty_like(w1), dw3=torch.empty_like(w3), dw2=torch.empty_like(w2),
+                       dout=gout, row_scale=ops.combine_row_scale(scores, plan), hs=torch.empty_like(h),
+                       dot_partial=torch.empty(rows.shape[0], ops.combine_bwd_slots(x.dtype, D, F),
+                                               dtype=torch.float32, device=dev))
+
+            def run_stage(s):
+                if s in ("dh", "dw2"):
+                    ops.grouped_swiglu_combine_stage(s, buf, plan)
+                else:
+                    ops.grouped_swiglu_stage(s, buf, plan)
+
+            stage_ms = {s: time_events(lambda s=s: run_stage(s), it) for s in stage_flops}
+            drows = buf["drows"]
+        else:
+            # fp32 / odd shapes: the generic kernels, timed per call (forward: gate, up, SwiGLU, down;
+            # backward: dh, SwiGLU', drows, three weight gradients)
+            stage_flops = {"experts_fwd": 3 * proj}
+            stage_ms["experts_fwd"] = time_events(lambda: ops.grouped_swiglu_fwd(rows, w1, w3, w2, plan), it)
+            if wl.backward:
+                stage_flops["experts_bwd"] = 6 * proj
+                stage_ms["experts_bwd"] = time_events(
+                    lambda: ops.grouped_swiglu_bwd(dy, rows, w1, w3, w2, gate, up, h, plan), it)
+            drows = torch.empty_like(rows)
+        gw, gb = block.router.gate.weight, block.router.gate.bias
+        sel = lambda: ops.router_select_fwd(logits, block.expert_bias_E, K, wl.score_func, wl.route_norm,
+                                            wl.route_scale, wl.num_expert_groups or 0, wl.num_limited_groups or 0,
+                                            want_map=True)
+        lo, hi = wl.local_experts or (0, E)
+        other_ms = {
+            "router_gate_fwd": time_events(lambda: ops.router_gate_fwd(x, gw, gb), it),
+            "router_select_fwd": time_events(sel, it),
+            "permute_plan": time_events(lambda: ops.permute_plan(ids, E, lo, hi, wl.pad_multiple or 1), it),
+            "permute_rows_fwd": time_events(lambda: ops.permute_rows_fwd(x, plan), it),
+            "combine_fwd": time_events(lambda: ops.combine_fwd(y, scores, plan), it),
+        }
+        in_step = {"router_gate_fwd", "router_select_fwd", "permute_plan", "combine_fwd"}
+        if not folded:
+            in_step.add("permute_rows_fwd")
+        if wl.backward:
+            other_ms.update({
+                "combine_bwd": time_events(lambda: ops.combine_bwd(gout, y, scores, plan), it),
+                "permute_rows_bwd": time_events(lambda: ops.permute_rows_bwd(drows, plan), it),
+                "router_gate_bwd": time_events(lambda: ops.router_gate_bwd(logits, x, gw), it),
+                "router_select_bwd": time_events(
+                    lambda: ops.router_select_bwd(logits, ids, scores, None, wl.score_func, wl.route_norm,
+                                                  wl.route_scale), it),
+            })
+            in_step |= {"permute_rows_bwd", "router_gate_bwd", "router_select_bwd"}
+            if folded:
+                other_ms["combine_row_scale"] = time_events(lambda: ops.combine_row_scale(scores, plan), it)
+                other_ms["combine_scores_bwd"] = time_events(
+                    lambda: ops.combine_scores_bwd(buf["dot_partial"], plan), it)
+                in_step |= {"combine_row_scale", "combine_scores_bwd"}
+            else:
+                in_step.add("combine_bwd")
+        shared_ms, shared_flops = {}, {}
+        if wl.shared_hidden_dim and ops.gather_supported(x, wl.shared_hidden_dim):
+            # the shared expert: a dense SwiGLU over all tokens on the same kernels (one segment)
+            sh = block.shared_experts
+            Fs = wl.shared_hidden_dim
+            sp = ops.segments_from_counts(torch.full((1,), T, dtype=torch.int32, device=dev), T)
+            s1, s3, s2 = (w.detach().unsqueeze(0) for w in (sh.gate_proj.weight, sh.up_proj.weight, sh.down_proj.weight))
+            sy, sg, su, shh = ops.grouped_swiglu_fwd(x, s1, s3, s2, sp)
+            sbuf = dict(rows=x, w1=s1, w3=s3, w2=s2, gate=sg, up=su, h=shh, y=sy, dy=gout,
+                        dgate=torch.empty_like(sg), dup=torch.empty_like(su), drows=torch.empty_like(x),
+                        dw1=torch.empty_like(s1), dw3=torch.empty_like(s3), dw2=torch.empty_like(s2))
+            sproj = 2.0 * T * D * Fs
+            shared_flops = {"gate_up": 2 * sproj, "down": sproj, "dh": sproj, "drows": 2 * sproj, "dw2": sproj,
+                            "dw1": sproj, "dw3": sproj}
+            if not wl.backward:
+                shared_flops = {k: shared_flops[k] for k in ("gate_up", "down")}
+            shared_ms = {s: time_events(lambda s=s: ops.grouped_swiglu_stage(s, sbuf, sp), it) for s in shared_flops}
+        # the callers' side of the path, outside the timed step: the decoder layer's norm in
+        # front of the block and the statistics of a quantile-balanced router
+        outside_ms = {}
+        if wl.key == "c3":
+            norm_w = torch.ones(D, dtype=x.dtype, device=dev)
+            _, rstd = ops.rms_norm_fwd(x, norm_w, 1e-6)
+            q_bias = torch.zeros(E, dtype=torch.float32, device=dev)
+            _, _, q_scores, q_cut = ops.router_select_cutoff_fwd(logits, q_bias, K, "sigmoid", True, 1.0)
+            q_hist = torch.zeros(E, 1000, dtype=torch.int64, device=dev)
+            outside_ms = {
+                "rms_norm_fwd": time_events(lambda: ops.rms_norm_fwd(x, norm_w, 1e-6), it),
+                "rms_norm_bwd": time_events(lambda: ops.rms_norm_bwd(gout, x, norm_w, rstd), it),
+                "router_select_cutoff_fwd": time_events(
+                    lambda: ops.router_select_cutoff_fwd(logits, q_bias, K, "sigmoid", True, 1.0), it),
+                "quantile_observe": time_events(lambda: ops.quantile_observe(q_hist, q_scores, q_cut, q_bias), it),
+            }
+            other_ms.update(outside_ms)
+    other_bytes = {
+        "permute_rows_fwd": T * D * s_bytes + R_cover * D * s_bytes + 4 * T * K,
+        "combine_fwd": R_rows * D * s_bytes + 8 * T * K + T * D * s_bytes,
+        "combine_bwd": T * D * s_bytes + 2 * R_rows * D * s_bytes + 4 * T * K,
+        "permute_rows_bwd": R_rows * D * s_bytes + T * D * s_bytes,
+        "rms_norm_fwd": 2 * T * D * s_bytes,
+        "rms_norm_bwd": 3 * T * D * s_bytes,
+    }
+    kernels = {}
+    for s, ms in stage_ms.items():
+        tf = stage_flops[s] / (ms * 1e-3) / 1e12 if ms > 0 else 0.0
+        kernels[f"grouped_{s}"] = {"ms": round(ms, 4), "TFLOP/s": round(tf, 1), "frac_mfma": round(tf / peak, 4)}
+    for s, ms in shared_ms.items():
+        tf = shared_flops[s] / (ms * 1e-3) / 1e12
+        kernels[f"shared_{s}"] = {"ms": round(ms, 4), "TFLOP/s": round(tf, 1), "frac_mfma": round(tf / peak, 4)}
+    for s, ms in other_ms.items():
+        ent = {"ms": round(ms, 4)}
+        if s not in in_step:
+            # public dispatcher API / the block's callers: not launched by the timed step
+            ent["in_step"] = False
+        if s in other_bytes:
+            gbs = other_bytes[s] / (ms * 1e-3) / 1e9
+            ent.update({"GB/s": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4)})
+        kernels[s] = ent
+    return kernels, stage_ms, stage_flops, shared_ms, shared_flops, R_rows, folded
 
 
 def main():
@@ -151,27 +345,26 @@ def main():
         sys.exit(2)
     import torch
 
-    from oracle import moe_ref as R
-    from tests.helpers import build_block, make_params
-    from torchllmtuner_amd import ops
+    from torchllmtuner_amd import workloads as W
 
-    name = next(iter(WORKLOADS))
-    cfg = dict(WORKLOADS[name])
-    cfg["T"] = args.tokens
-    T, D, E, K, F = cfg["T"], cfg["D"], cfg["E"], cfg["K"], cfg["F"]
+    wl = W.WORKLOADS[args.workload]
     dev = "cuda:0"
-    spec = R.RouterSpec(E, K, score_func="softmax", route_norm=True)
-    p = make_params(E, D, F, torch.bfloat16, seed=0)
-    block = build_block(p, spec, D, F, torch.bfloat16, dev)
-    block.train()
-    x = torch.randn(T, D, generator=torch.Generator().manual_seed(0)).bfloat16().to(dev)
-    gout = torch.randn(T, D, generator=torch.Generator().manual_seed(1)).bfloat16().to(dev)
+    x_cpu, gout_cpu = W.make_inputs(wl)
+    block = W.build_block(wl, dev, x_for_skew=x_cpu)
+    block.train(wl.backward)
+    x, gout = x_cpu.to(dev), gout_cpu.to(dev)
+    T = wl.tokens
 
-    def step():
-        block.zero_grad(set_to_none=True)
-        xin = x.detach().requires_grad_()
-        out = block(xin)
-        out.backward(gout)
+    if wl.backward:
+        def step():
+            block.zero_grad(set_to_none=True)
+            xin = x.detach().requires_grad_()
+            out = block(xin)
+            out.backward(gout)
+    else:
+        def step():
+            with torch.no_grad():
+                block(x)
 
     for _ in range(args.warmup):
         step()
@@ -184,133 +377,82 @@ def main():
     ms_per_step = dt / args.steps * 1e3
     tokens_per_s = T * args.steps / dt
 
-    # ---- per-kernel timing on the launch stream ---------------------------------
-    with torch.no_grad():
-        scores, ids = block.router.route(x)
-        plan = block.routed_experts.token_dispatcher.plan(ids)
-        rows = ops.permute_rows_fwd(x, plan)
-        ie = block.routed_experts.inner_experts
-        w1, w3, w2 = ie.w1_EFD.detach(), ie.w3_EFD.detach(), ie.w2_EDF.detach()
-        y, gate, up, h = ops.grouped_swiglu_fwd(rows, w1, w3, w2, plan)
-        dy, _ = ops.combine_bwd(gout, y, scores, plan)
-        # as in the training step: the token matrix is read through the gather index
-        # (gate/up A operand, dW1/dW3 B operand); no expert-major copy of the tokens
-        buf = dict(rows=x, token_of_row=plan.token_of_row, w1=w1, w3=w3, w2=w2, gate=gate, up=up, h=h, y=y, dy=dy,
-                   dgate=torch.empty_like(gate), dup=torch.empty_like(up), drows=torch.empty_like(rows),
-                   dw1=torch.empty_like(w1), dw3=torch.empty_like(w3), dw2=torch.empty_like(w2))
-        R_rows = int(plan.total_rows.item())
-        it = args.stage_iters
-        # The step's backward folds the combine into the expert kernels: dH reads the output
-        # gradient through the token index and scales rows in its epilogue, dW2 contracts the
-        # gathered rows with score * h.  Those two are timed in that form.
-        folded = ops.combine_bwd_slots(x.dtype, D, F) > 0
-        if folded:
-            buf.update(dout=gout, row_scale=ops.combine_row_scale(scores, plan), hs=torch.empty_like(h),
-                       dot_partial=torch.empty(rows.shape[0], ops.combine_bwd_slots(x.dtype, D, F),
-                                               dtype=torch.float32, device=dev))
+    x2, g2 = x.reshape(-1, wl.dim), gout.reshape(-1, wl.dim)
+    kernels, stage_ms, stage_flops, shared_ms, shared_flops, R_rows, folded = per_kernel_times(
+        args, wl, block, x2, g2, dev)
+    peak = PEAK_BF16_TFLOPS if wl.dtype == torch.bfloat16 else PEAK_FP32_TFLOPS
 
-        def run_stage(s):
-            if folded and s in ("dh", "dw2"):
-                ops.grouped_swiglu_combine_stage(s, buf, plan)
-            else:
-                ops.grouped_swiglu_stage(s, buf, plan)
-
-        stage_ms = {s: time_events(lambda s=s: run_stage(s), it) for s in ops.STAGES}
-        logits = ops.router_gate_fwd(x, block.router.gate.weight)
-        other_ms = {
-            "router_gate_fwd": time_events(lambda: ops.router_gate_fwd(x, block.router.gate.weight), it),
-            "router_select_fwd": time_events(lambda: ops.router_select_fwd(logits, None, K, "softmax", True, 1.0), it),
-            "permute_plan": time_events(lambda: ops.permute_plan(ids, E), it),
-            "permute_rows_fwd": time_events(lambda: ops.permute_rows_fwd(x, plan), it),
-            "combine_fwd": time_events(lambda: ops.combine_fwd(y, scores, plan), it),
-            "combine_bwd": time_events(lambda: ops.combine_bwd(gout, y, scores, plan), it),
-            "permute_rows_bwd": time_events(lambda: ops.permute_rows_bwd(buf["drows"], plan), it),
-            "router_gate_bwd": time_events(lambda: ops.router_gate_bwd(logits, x, block.router.gate.weight), it),
-        }
-        if folded:
-            other_ms["combine_row_scale"] = time_events(lambda: ops.combine_row_scale(scores, plan), it)
-            other_ms["combine_scores_bwd"] = time_events(lambda: ops.combine_scores_bwd(buf["dot_partial"], plan), it)
-        # the callers' side of the path, outside the timed step: the decoder layer's norm in
-        # front of the block and the statistics of a quantile-balanced router
-        norm_w = torch.ones(D, dtype=torch.bfloat16, device=dev)
-        normed, rstd = ops.rms_norm_fwd(x, norm_w, 1e-6)
-        q_bias = torch.zeros(E, dtype=torch.float32, device=dev)
-        _, _, q_scores, q_cut = ops.router_select_cutoff_fwd(logits, q_bias, K, "sigmoid", True, 1.0)
-        q_hist = torch.zeros(E, 1000, dtype=torch.int64, device=dev)
-        outside_ms = {
-            "rms_norm_fwd": time_events(lambda: ops.rms_norm_fwd(x, norm_w, 1e-6), it),
-            "rms_norm_bwd": time_events(lambda: ops.rms_norm_bwd(gout, x, norm_w, rstd), it),
-            "router_select_cutoff_fwd": time_events(
-                lambda: ops.router_select_cutoff_fwd(logits, q_bias, K, "sigmoid", True, 1.0), it),
-            "quantile_observe": time_events(lambda: ops.quantile_observe(q_hist, q_scores, q_cut, q_bias), it),
-        }
-        other_ms.update(outside_ms)
-    # algorithmic work per launch (padding excluded): 2*R*D*F per projection
-    proj = 2.0 * R_rows * D * F
-    stage_flops = {"gate_up": 2 * proj, "down": proj, "dh": proj, "drows": 2 * proj,
-                   "dw2": proj, "dw1": proj, "dw3": proj}
-    s_bytes = 2
-    other_bytes = {
-        "permute_rows_fwd": T * D * s_bytes + R_rows * D * s_bytes + 4 * R_rows,
-        "combine_fwd": R_rows * D * s_bytes + 8 * T * K + T * D * s_bytes,
-        "combine_bwd": T * D * s_bytes + 2 * R_rows * D * s_bytes + 4 * T * K,
-        "permute_rows_bwd": R_rows * D * s_bytes + T * D * s_bytes,
-        "rms_norm_fwd": 2 * T * D * s_bytes,
-        "rms_norm_bwd": 3 * T * D * s_bytes,
-    }
-    kernels = {}
-    for s, ms in stage_ms.items():
-        tf = stage_flops[s] / (ms * 1e-3) / 1e12
-        kernels[f"grouped_{s}"] = {"ms": round(ms, 4), "TFLOP/s": round(tf, 1), "frac_mfma": round(tf / PEAK_BF16_TFLOPS, 4)}
-    for s, ms in other_ms.items():
-        ent = {"ms": round(ms, 4)}
-        if s == "permute_rows_fwd" or (s == "combine_bwd" and folded) or s in outside_ms:
-            # permute_rows_fwd, combine_bwd: public dispatcher API only, the step gathers inside
-            # the GEMMs and folds the combine's backward into them; the others belong to the
-            # block's callers
-            ent["in_step"] = False
-        if s in other_bytes:
-            gbs = other_bytes[s] / (ms * 1e-3) / 1e9
-            ent.update({"GB/s": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4)})
-        kernels[s] = ent
-    dominant = max(stage_ms, key=stage_ms.get)
-    ach = stage_flops[dominant] / (stage_ms[dominant] * 1e-3) / 1e12
-    gemm_flops = sum(stage_flops.values())
-    gemm_ms = sum(stage_ms.values())
+    # The kernel with the largest share of the step.  dW1 and dW3 are two launches of one kernel
+    # (the gathered weight gradient), so they count together; the shared expert's stages are
+    # launches of the same kernels over one dense segment and are listed under their own names.
+    groups = {}
+    for s in stage_ms:
+        key = "dw1+dw3" if s in ("dw1", "dw3") else s
+        g = groups.setdefault(f"grouped_{key}", {"ms": 0.0, "flops": 0.0, "launches": 0})
+        g["ms"] += stage_ms[s]; g["flops"] += stage_flops[s]; g["launches"] += 1
+    for s in shared_ms:
+        key = "dw1+dw3" if s in ("dw1", "dw3") else s
+        g = groups.setdefault(f"shared_{key}", {"ms": 0.0, "flops": 0.0, "launches": 0})
+        g["ms"] += shared_ms[s]; g["flops"] += shared_flops[s]; g["launches"] += 1
+    dominant = max(groups, key=lambda k: groups[k]["ms"])
+    dg = groups[dominant]
+    ach = dg["flops"] / (dg["ms"] * 1e-3) / 1e12
+    gemm_flops = sum(stage_flops.values()) + sum(shared_flops.values())
+    gemm_ms = sum(stage_ms.values()) + sum(shared_ms.values())
+    traffic = None
+    if args.workload in MEASURED_HBM_BYTES and dominant.startswith("grouped_"):
+        tb = MEASURED_HBM_BYTES[args.workload]
+        parts = dominant[len("grouped_"):].split("+")
+        if all(p in tb for p in parts):
+            traffic = sum(tb[p] for p in parts) / len(parts)
     roofline = {
-        "kernel": f"grouped_{dominant}",
+        "kernel": dominant,
+        "launches_per_step": dg["launches"],
+        "share_of_step": round(dg["ms"] / ms_per_step, 4),
         "bound": "mfma",
         "achieved": round(ach, 2),
-        "peak": PEAK_BF16_TFLOPS,
+        "peak": peak,
         "unit": "TFLOP/s",
-        "frac": round(ach / PEAK_BF16_TFLOPS, 4),
-        "traffic": MEASURED_HBM_BYTES.get(dominant) if T == 8192 else None,
-        "avg_launch_ms": round(stage_ms[dominant], 4),
+        "frac": round(ach / peak, 4),
+        "traffic": traffic,
+        "avg_launch_ms": round(dg["ms"] / dg["launches"], 4),
         "all_grouped_gemms": {"TFLOP/s": round(gemm_flops / (gemm_ms * 1e-3) / 1e12, 1),
-                              "frac": round(gemm_flops / (gemm_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4)},
+                              "frac": round(gemm_flops / (gemm_ms * 1e-3) / 1e12 / peak, 4),
+                              "ms": round(gemm_ms, 4)},
     }
 
-    probe = None if args.no_probe else sustained_mfma(dev)
+    probe = None if (args.no_probe or wl.dtype != torch.bfloat16) else sustained_mfma(dev)
     if probe is not None:
         # the same instruction with operands in registers: the rate the card holds under
         # its own power management, next to the data-sheet peak above
         roofline["sustained_mfma"] = probe
-        shape = "32x32x16" if dominant.startswith("dw") else "16x16x32"
+        shape = "32x32x16" if "dw" in dominant else "16x16x32"
         roofline["frac_of_sustained"] = round(ach / probe[shape]["random_bits"]["TFLOP/s"], 4)
-
-    if not args.no_probe:
-        # The vendor library's dense GEMM with the dominant kernel's flops (all rows against
-        # ONE expert's gate and up weights, random values, no SwiGLU, no routing): what a
-        # tuned kernel holds on this card at this size, next to the data-sheet peak.
-        a = torch.randn(R_rows, D, device=dev).bfloat16()
-        b = torch.randn(2 * F, D, device=dev).bfloat16()
+        # The vendor library's dense GEMM with the gate/up kernel's flops (all rows against ONE
+        # expert's gate and up weights, random values, no SwiGLU, no routing): what a tuned
+        # kernel holds on this card at this size, next to the data-sheet peak.
+        a = torch.randn(max(R_rows, 1), wl.dim, device=dev).bfloat16()
+        b = torch.randn(2 * wl.hidden_dim, wl.dim, device=dev).bfloat16()
         ms = time_events(lambda: torch.mm(a, b.t()), 10, warmup=3)
-        roofline["vendor_dense_gemm"] = {"shape_mnk": [R_rows, 2 * F, D], "ms": round(ms, 4),
-                                         "TFLOP/s": round(2.0 * R_rows * 2 * F * D / (ms * 1e-3) / 1e12, 1)}
+        roofline["vendor_dense_gemm"] = {"shape_mnk": [a.shape[0], 2 * wl.hidden_dim, wl.dim], "ms": round(ms, 4),
+                                         "TFLOP/s": round(2.0 * a.shape[0] * 2 * wl.hidden_dim * wl.dim / (ms * 1e-3) / 1e12, 1)}
         del a, b
 
+    config = W.describe(wl)
+    config["routed_rows"] = R_rows
+    if getattr(block, "skew_top20_share", None) is not None:
+        config["skew_top20_share_solved"] = round(block.skew_top20_share, 4)
+    if wl.zipf_top20_share:
+        with torch.no_grad():
+            _, ids = block.router.route(x2)
+        load = torch.bincount(ids.reshape(-1), minlength=wl.num_experts).sort(descending=True).values
+        config["load_histogram_sorted"] = {"max": int(load[0]), "median": int(load[wl.num_experts // 2]),
+                                           "min": int(load[-1]),
+                                           "top20_share": round(float(load[: wl.num_experts // 5].sum()) / ids.numel(), 4)}
+    metric = ("MoE layer fwd+bwd tokens/s (Qwen3-30B-A3B shape, 1 GPU)" if args.workload == "c3"
+              else f"MoE layer {'fwd+bwd' if wl.backward else 'fwd'} tokens/s ({wl.key}, 1 GPU)")
     result = {
-        "metric": "MoE layer fwd+bwd tokens/s (Qwen3-30B-A3B shape, 1 GPU)",
+        "metric": metric,
         "value": round(tokens_per_s, 1),
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -320,11 +462,9 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16",
+        "dtype": "bf16" if wl.dtype == torch.bfloat16 else "fp32",
         "data": "synthetic",
-        "config": {"workload": name if T == 8192 else f"{name} (tokens overridden to {T})",
-                   "tokens": T, "hidden": D, "experts": E, "top_k": K, "moe_intermediate": F,
-                   "router": "fp32 softmax top-k, norm_topk_prob", "routed_rows": R_rows},
+        "config": config,
         "roofline": roofline,
         "kernels": kernels,
     }
@@ -334,7 +474,7 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(cfg, args.cpu_sample_tokens)
+        result["cpu_baseline"] = cpu_baseline(wl, args.cpu_sample_tokens)
     print(json.dumps(result))
 
 

@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define MI355_MOE_ABI_VERSION 1
+#define MI355_MOE_ABI_VERSION 2
 
 /* element types of activation / weight buffers */
 #define MI355_F32 0
@@ -92,15 +92,21 @@ int mi355_router_gate_bwd(const float* dlogits_TE, const void* x, int x_dtype,
  * the rest masked to -inf), unbiased gather, route_norm with +1e-20, route_scale
  * (:311-315), and the fixed / balanced debug routings (:291-309, :146-166).
  * Selection order is "higher choice score first, ties to the lower expert id";
- * ids are emitted in that order.
+ * ids are emitted in that order.  Without a bias and without groups the choice is made
+ * on the logits (every score function is non-decreasing in its logit), so it does not
+ * depend on the last ulp of exp(): for equal logits in, the ids equal those of any
+ * correct top-k over the scores wherever the scores themselves do not tie.
  * expert_bias: (E) fp32 or NULL.  num_groups = 0 disables grouping.
  * scores_TE: optional (T,E) fp32 output of the score function (NULL = skip).
+ * routing_map_TE: optional (T,E) bytes, 1 where the token chose the expert (the bool
+ * routing map of routing.py:320-324; NULL = skip).
  */
 int mi355_router_select_fwd(const float* logits_TE, const float* expert_bias,
                             float* weights_TK, int64_t* ids_TK, float* scores_TE,
-                            int64_t T, int64_t E, int64_t K, int score_func,
-                            int route_norm, float route_scale, int num_groups,
-                            int num_limited, int select_mode, void* stream);
+                            uint8_t* routing_map_TE, int64_t T, int64_t E, int64_t K,
+                            int score_func, int route_norm, float route_scale,
+                            int num_groups, int num_limited, int select_mode,
+                            void* stream);
 
 /*
  * The same selection for a quantile-balanced router in training
@@ -217,7 +223,8 @@ int mi355_balance_loss_bwd(const float* scores_TE, const float* f_E,
  * row_capacity  >= N + El*(align-1) is always enough;
  * tile_capacity >= N/tile_m + El + 1 is always enough.
  * workspace: mi355_permute_plan_workspace_bytes(T,K,E) bytes.
- * ids outside [0,E) make the result undefined but never write out of bounds.
+ * A slot whose id lies outside [0,E) is not counted and gets row -1 (its token simply
+ * misses that expert); nothing is read or written out of bounds.  E <= 2048.
  */
 int64_t mi355_permute_plan_workspace_bytes(int64_t T, int64_t K, int64_t E);
 int mi355_permute_plan(const int64_t* ids_TK, int64_t T, int64_t K, int64_t E,
@@ -243,15 +250,16 @@ int mi355_segments_from_counts(const int32_t* counts, int64_t El, int64_t tile_m
                                int32_t* num_tiles, int64_t tile_capacity, void* stream);
 
 /*
- * rows[r] = x[slot_of_row[r] / K], zero for padding rows; rows at or beyond
- * seg_offsets[El] are left untouched.  Replaces the gather x[token_indices],
- * token_dispatch.py:197-199, and the sentinel-row padding of the padded layout.
- * total_rows points at seg_offsets[El] on the device.
+ * rows[row_of_slot[t*K+k]] = x[t] for every slot with a row (each token row is read once
+ * and stored K times), zero for padding rows; rows at or beyond seg_offsets[El] are left
+ * untouched.  Replaces the gather x[token_indices], token_dispatch.py:197-199, and the
+ * sentinel-row padding of the padded layout.  slot_of_row may be NULL when the plan has no
+ * padding rows (align = 1); with it, total_rows points at seg_offsets[El] on the device.
  */
-int mi355_permute_rows_fwd(const void* x, int dtype, const int32_t* slot_of_row,
-                           const int32_t* total_rows, void* rows, int64_t T,
-                           int64_t D, int64_t K, int64_t row_capacity,
-                           void* stream);
+int mi355_permute_rows_fwd(const void* x, int dtype, const int32_t* row_of_slot,
+                           const int32_t* slot_of_row, const int32_t* total_rows,
+                           void* rows, int64_t T, int64_t D, int64_t K,
+                           int64_t row_capacity, void* stream);
 
 /*
  * dx[t] = sum_k drows[row_of_slot[t*K+k]] (slots with row -1 contribute nothing),
@@ -306,14 +314,17 @@ int mi355_combine_bwd(const void* dout, const void* y, int dtype,
  * token_of_row (optional): when given, `rows` is the UNPERMUTED (T,D) token matrix and
  * row r reads rows[token_of_row[r]] -- the gather of token_dispatch.py:197-199 fused
  * into the operand loads, so the (R,D) expert-major copy is never written.  bf16 with
- * D and F multiples of 64 only (MI355_EUNSUP otherwise).
+ * D and F multiples of 64 only (MI355_EUNSUP otherwise).  num_tokens = T bounds the
+ * index: entries are clamped to [0, T) on the device (a corrupt index reads a wrong row,
+ * never out of bounds), and the call returns MI355_EINVAL without launching when
+ * token_of_row is given with T < 1 or with T*D*2 >= 2^32 bytes (the gather addresses its
+ * source with 32-bit byte offsets).  Ignored when token_of_row is NULL.
  * gate/up/h are saved for the backward (each (row_capacity,F)).
- * The kernels walk the plan's tile list in tiles of mi355_grouped_tile_m(dtype) rows, so
- * the list must have been built with that value (256; 128 when the process runs with
- * MI355_ROW_LAYOUT=wide, which selects the 128 x 512 row tile of the bf16 kernels).
+ * The kernels walk the plan's tile list in tiles of mi355_grouped_tile_m(dtype) rows
+ * (256), so the list must have been built with that value.
  */
 int64_t mi355_grouped_tile_m(int dtype);
-int mi355_grouped_swiglu_fwd(const void* rows, const int32_t* token_of_row,
+int mi355_grouped_swiglu_fwd(const void* rows, const int32_t* token_of_row, int64_t num_tokens,
                              const void* w1, const void* w3, const void* w2, int dtype,
                              const int32_t* seg_offsets,
                              const int32_t* seg_counts, const int32_t* tile_expert,
@@ -329,12 +340,12 @@ int mi355_grouped_swiglu_fwd(const void* rows, const int32_t* token_of_row,
  *   dw2[e] = dy_e^T . h_e;  dw1[e] = dgate_e^T . rows_e;  dw3[e] = dup_e^T . rows_e
  * dgate/dup are caller-provided scratch of (row_capacity,F) each.  Weight
  * gradients are written (not accumulated) in `dtype`; experts with no rows get
- * zeros.  Any of drows/dw1/dw3/dw2 may be NULL to skip it.  token_of_row has the
- * meaning it has in the forward (`rows` = the (T,D) token matrix); drows is always
+ * zeros.  Any of drows/dw1/dw3/dw2 may be NULL to skip it.  token_of_row and num_tokens
+ * have the meaning they have in the forward (`rows` = the (T,D) token matrix); drows is always
  * expert-major (row_capacity,D) and goes through mi355_permute_rows_bwd.
  */
 int mi355_grouped_swiglu_bwd(const void* dy, const void* rows,
-                             const int32_t* token_of_row, const void* w1,
+                             const int32_t* token_of_row, int64_t num_tokens, const void* w1,
                              const void* w3, const void* w2, const void* gate,
                              const void* up, const void* h, int dtype,
                              const int32_t* seg_offsets, const int32_t* seg_counts,
@@ -361,7 +372,8 @@ int mi355_grouped_swiglu_bwd(const void* dy, const void* rows,
  * Two bf16 roundings move compared with the two-call form (dh is rounded once, after the
  * scaling, instead of dy and dh each; dW2 rounds weights*h instead of weights*dout); both
  * stay inside the bf16 tolerance of the path.
- * bf16 only, D and F multiples of 64 and >= 384, 256-row tile layout:
+ * bf16 only, D and F multiples of 64 and >= 384; token_of_row is required here and
+ * num_tokens = T bounds it as in mi355_grouped_swiglu_fwd (dout and x are both (T,D)):
  * mi355_grouped_combine_bwd_slots returns the number of partials per row (the second
  * dimension of dot_partial), or 0 when this entry point does not cover the case (then use
  * the two-call form).  row_scale (row_capacity floats) comes from mi355_combine_row_scale:
@@ -372,7 +384,7 @@ int mi355_grouped_swiglu_bwd(const void* dy, const void* rows,
  */
 int64_t mi355_grouped_combine_bwd_slots(int dtype, int64_t D, int64_t F);
 int mi355_grouped_swiglu_combine_bwd(const void* dout, const void* x, const int32_t* token_of_row,
-                                     const float* row_scale, const void* w1, const void* w3,
+                                     int64_t num_tokens, const float* row_scale, const void* w1, const void* w3,
                                      const void* w2, const void* gate, const void* up, int dtype,
                                      const int32_t* seg_offsets, const int32_t* seg_counts,
                                      const int32_t* tile_expert, const int32_t* tile_row0,
@@ -401,7 +413,7 @@ int mi355_combine_scores_bwd(const float* dot_partial, int64_t slots, const int3
 #define MI355_STAGE_DW1 32   /* dw1           <- dgate, rows  */
 #define MI355_STAGE_DW3 64   /* dw3           <- dup, rows    */
 int mi355_grouped_swiglu_stage(int stage, const void* dy, const void* rows,
-                               const int32_t* token_of_row, const void* w1,
+                               const int32_t* token_of_row, int64_t num_tokens, const void* w1,
                                const void* w3, const void* w2, void* gate, void* up,
                                void* h, void* y, const int32_t* seg_offsets,
                                const int32_t* seg_counts, const int32_t* tile_expert,

@@ -23,3 +23,12 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+def pytest_terminal_summary(terminalreporter):
+    from tests import helpers
+
+    if helpers.PARITY_NOTES:
+        terminalreporter.section("routing parity and load figures")
+        for line in helpers.PARITY_NOTES:
+            terminalreporter.write_line(line)

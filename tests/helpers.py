@@ -7,6 +7,16 @@ import torch
 from oracle import moe_ref as R
 
 
+# Lines for the end-of-run summary (tests/conftest.py prints them whatever the verbosity): how
+# many tokens differed from the oracle, load histograms -- figures a passing test would hide.
+PARITY_NOTES: list[str] = []
+
+
+def note(line: str) -> None:
+    print(line, flush=True)
+    PARITY_NOTES.append(line)
+
+
 def rel_l2(a: torch.Tensor, b: torch.Tensor) -> float:
     a, b = a.detach().double().cpu(), b.detach().double().cpu()
     return float((a - b).norm() / b.norm().clamp_min(1e-30))
@@ -34,6 +44,16 @@ def stable_tokens(logits_TE, spec: R.RouterSpec, expert_bias_E=None, trials=4, e
         ids = R.select_experts(base * noise, expert_bias_E, spec.top_k, spec.num_expert_groups, spec.num_limited_groups)
         ok &= (ids == ref).all(dim=-1)
     return ok
+
+
+def exact_score_ties(logits_TE, spec: R.RouterSpec, expert_bias_E=None):
+    """Tokens whose K+1 best choice scores (oracle arithmetic, fp32) contain two EQUAL values:
+    there the reference's ``torch.topk`` may pick either expert, and so may any correct
+    implementation.  Everywhere else the selection -- ids and their order -- is determined."""
+    s = R.score(logits_TE, spec.score_func)
+    c = s if expert_bias_E is None else s + expert_bias_E
+    top = torch.topk(c, min(spec.top_k + 1, c.shape[-1]), dim=-1).values
+    return (top[:, 1:] == top[:, :-1]).any(-1)
 
 
 def make_params(E, D, F, dtype, seed=0, std=0.02, shared_F=None, El=None):

@@ -1,9 +1,12 @@
 """GPU parity of every kernel, called through the C ABI (torchllmtuner_amd.ops),
 against the CPU oracle on identical seeded inputs.
 
-Bars: routing ids, counts and permutation order bit-exact (on tokens whose decision
-is not a few-ulp near tie, see helpers.stable_tokens); fp32 values within 1e-5
-relative; bf16 values within 2e-2 relative L2.
+Bars: routing ids, counts and permutation order bit-exact -- on EVERY token whose oracle
+scores do not tie exactly where the choice is the plain top-k of the scores (the kernel then
+selects on the logits, which no exp() implementation can reorder), and on every token
+outside the few-ulp near-tie set (helpers.stable_tokens), with the number of differing
+tokens printed and bounded, where a bias or group scores enter the choice; fp32 values
+within 1e-5 relative; bf16 values within 2e-2 relative L2.
 """
 
 import pytest
@@ -11,7 +14,7 @@ import torch
 import torch.nn.functional as F
 
 from oracle import moe_ref as R
-from tests.helpers import rel_l2, rel_max, stable_tokens
+from tests.helpers import exact_score_ties, note, rel_l2, rel_max, stable_tokens
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -82,15 +85,36 @@ def test_router_select_fwd_bwd(ops, case):
     lr = logits.clone().requires_grad_()
     w_ref, ids_ref, _ = R.route(lr, spec, bias)
     mode = 1 if spec.fixed_router else (2 if spec.debug_force_load_balance else 0)
-    w, ids, scores = ops.router_select_fwd(
+    w, ids, scores, rmap = ops.router_select_fwd(
         logits.to(DEV), None if bias is None else bias.to(DEV), K, spec.score_func, spec.route_norm,
-        spec.route_scale, spec.num_expert_groups or 0, spec.num_limited_groups or 0, mode, True)
-    assert ids.dtype == torch.int64
-    ok = torch.ones(T, dtype=torch.bool) if mode else stable_tokens(logits, spec, bias)
-    assert ok.float().mean() > 0.98, "too many near-tie tokens for a meaningful check"
-    assert torch.equal(ids.cpu()[ok], ids_ref[ok]), "routing ids differ on tokens that are not near ties"
+        spec.route_scale, spec.num_expert_groups or 0, spec.num_limited_groups or 0, mode, True, True)
+    assert ids.dtype == torch.int64 and rmap.dtype == torch.bool
+    # the routing map is the one-hot of the kernel's own ids (routing.py:320-324)
+    assert torch.equal(rmap.cpu(), torch.zeros(T, E, dtype=torch.bool).scatter_(-1, ids.cpu(), True))
+    differ = ~(ids.cpu() == ids_ref).all(-1)
+    if mode:
+        assert not differ.any()
+        ok = torch.ones(T, dtype=torch.bool)
+    elif bias is None and not spec.num_expert_groups:
+        # plain top-k of the scores: bit-exact on every token whose scores do not tie exactly
+        # (where the reference's own torch.topk is free to pick either)
+        tied = exact_score_ties(logits, spec)
+        note(f"select {spec.score_func} E={E} K={K}: {int(tied.sum())} of {T} tokens have an exact score tie among "
+             f"the top {K + 1}; {int(differ.sum())} tokens differ from the oracle")
+        assert int(tied.sum()) <= max(1, T // 100)
+        assert not differ[~tied].any(), "routing ids differ although the logits are identical and no score ties"
+        ok = ~tied
+    else:
+        # a bias or group scores enter the choice: two correct exp() implementations may flip a
+        # token whose decision hangs on the last ulps; every difference must be such a token
+        ok = stable_tokens(logits, spec, bias)
+        note(f"select {spec.score_func} E={E} K={K} (bias / groups): {int((~ok).sum())} of {T} tokens are near "
+             f"ties; {int(differ.sum())} tokens differ from the oracle")
+        assert ok.float().mean() > 0.98, "too many near-tie tokens for a meaningful check"
+        assert not differ[ok].any(), "routing ids differ on tokens that are not near ties"
+        assert int(differ.sum()) <= int((~ok).sum())
     assert rel_max(scores, R.score(logits, spec.score_func)) < FP32_TOL
-    assert rel_max(w.cpu()[ok], w_ref[ok]) < FP32_TOL
+    assert rel_max(w.cpu()[~differ], w_ref[~differ]) < FP32_TOL
     # backward given the oracle's ids (same inputs on both sides)
     gw = torch.randn(T, K, generator=g)
     if not spec.fixed_router:
@@ -381,14 +405,14 @@ def test_folded_combine_backward_matches_the_two_call_backward(ops, T, K, E, D, 
     dy, dwt_a = ops.combine_bwd(dd, y, wd, plan)
     drows_a, dw1_a, dw3_a, dw2_a = ops.grouped_swiglu_bwd(dy, xd, w1d, w3d, w2d, gate, up, h, plan, gather=True)
     scale = ops.combine_row_scale(wd, plan)
-    drows_b, dw1_b, dw3_b, dw2_b, dwt_b = ops.grouped_swiglu_combine_bwd(dd, xd, scale, w1d, w3d, w2d, gate, up, plan)
+    dx_b, dw1_b, dw3_b, dw2_b, dwt_b = ops.grouped_swiglu_combine_bwd(dd, xd, wd, w1d, w3d, w2d, gate, up, plan)
 
     # row_scale is the weights read through the plan, zero where a row holds padding
     sor = plan.slot_of_row.cpu()
     want_scale = torch.where(sor >= 0, weights.flatten()[sor.clamp(min=0)], torch.zeros(()))
     assert torch.equal(scale.cpu(), want_scale)
 
-    dx_a, dx_b = ops.permute_rows_bwd(drows_a, plan), ops.permute_rows_bwd(drows_b, plan)
+    dx_a = ops.permute_rows_bwd(drows_a, plan)
     for name, a, b in (("dx", dx_a, dx_b), ("dw1", dw1_a, dw1_b), ("dw3", dw3_a, dw3_b), ("dw2", dw2_a, dw2_b),
                        ("dweights", dwt_a, dwt_b)):
         assert rel_l2(b, a) < BF16_TOL, f"{name}: folded vs two calls {rel_l2(b, a)}"
@@ -414,18 +438,106 @@ def test_folded_combine_backward_matches_the_two_call_backward(ops, T, K, E, D, 
     assert torch.equal(dwt_b.cpu()[~local_slot], torch.zeros_like(dwt_b.cpu()[~local_slot]))
 
 
-def test_wide_row_tile_layout_in_a_child_process():
-    """The 128 x 512 row tile is chosen per process (MI355_ROW_LAYOUT=wide, read when the
-    library first launches a grouped kernel), so its parity cases run in a child."""
-    import os
-    import subprocess
-    import sys
+def test_gathered_experts_combine_autograd_matches_the_explicit_backward(ops):
+    """The differentiable operator (forward + registered autograd formula) gives the gradients of
+    the explicit backward call, bit for bit, and leaves unrequested gradients alone."""
+    print("gather_experts_combine autograd", flush=True)
+    T, K, E, D, Fd = 300, 4, 8, 384, 384
+    g = torch.Generator().manual_seed(3)
+    ids = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(T)]).to(DEV)
+    wts = torch.rand(T, K, generator=g).to(DEV).requires_grad_()
+    x = torch.randn(T, D, generator=g).bfloat16().to(DEV).requires_grad_()
+    dout = torch.randn(T, D, generator=g).bfloat16().to(DEV)
+    mk = lambda *s: (torch.randn(*s, generator=g) * 0.05).bfloat16().to(DEV).requires_grad_()
+    w1, w3, w2 = mk(E, Fd, D), mk(E, Fd, D), mk(E, D, Fd)
+    plan = ops.permute_plan(ids, E)
+    out = ops.gather_experts_combine(x, wts, w1, w3, w2, plan)
+    out.backward(dout)
+    with torch.no_grad():
+        y, gate, up, h = ops.grouped_swiglu_fwd(x, w1, w3, w2, plan, gather=True)
+        assert torch.equal(out, ops.combine_fwd(y, wts, plan))
+        dx, dw1, dw3, dw2, dwt = ops.grouped_swiglu_combine_bwd(dout, x, wts, w1, w3, w2, gate, up, plan)
+    for got, want in ((x.grad, dx), (w1.grad, dw1), (w3.grad, dw3), (w2.grad, dw2), (wts.grad, dwt)):
+        assert torch.equal(got, want)
+    # only dx asked for: the weight-gradient kernels do not run and nothing else gets a gradient
+    x2 = x.detach().clone().requires_grad_()
+    ops.gather_experts_combine(x2, wts.detach(), w1.detach(), w3.detach(), w2.detach(), plan).backward(dout)
+    assert torch.equal(x2.grad, dx)
 
-    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    env = dict(os.environ, MI355_ROW_LAYOUT="wide")
-    child = subprocess.run(
-        [sys.executable, "-m", "pytest", os.path.join(root, "tests", "test_gpu_kernels.py"), "-q", "-x",
-         "-k", "bf16_mfma or plan_is_the_stable", "-p", "no:cacheprovider"],
-        cwd=root, env=env, capture_output=True, text=True, timeout=300)
-    assert child.returncode == 0, child.stdout[-2000:] + child.stderr[-2000:]
-    assert " passed" in child.stdout
+
+@pytest.mark.parametrize("counts", [(2, 0, 3), (0, 5, 0), (0, 0, 0)])
+@pytest.mark.parametrize("dtype,D,Fd", [(torch.float32, 4, 8), (torch.bfloat16, 384, 384)])
+def test_grouped_experts_under_torch_compile(counts, dtype, D, Fd):
+    """GroupedExperts traced whole (aot_eager, fullgraph) equals eager, forward and gradients, for
+    the zero-count segment cases of tests/unit_tests/cpu/test_expert_compile_segments.py:13-40:
+    the operators carry fake kernels and registered autograd formulas, so nothing graph-breaks."""
+    print(f"experts under torch.compile {counts} {dtype}", flush=True)
+    from torchllmtuner_amd import moe
+
+    torch.manual_seed(0)
+    El, Rn = len(counts), sum(counts)
+    experts = moe.GroupedExperts(D, Fd, El).to(DEV).to(dtype)
+    with torch.no_grad():
+        for p in experts.parameters():
+            p.normal_(0, 0.1)
+    x = torch.randn(Rn, D, device=DEV).to(dtype)
+    cnt = torch.tensor(counts, device=DEV)
+    gy = torch.randn(Rn, D, device=DEV).to(dtype)
+
+    def run(fn):
+        experts.zero_grad(set_to_none=True)
+        xin = x.clone().requires_grad_()
+        y = fn(xin, cnt)
+        y.backward(gy)
+        return [y.detach(), xin.grad] + [p.grad.clone() for p in experts.parameters()]
+
+    eager = run(experts)
+    torch._dynamo.reset()
+    compiled = run(torch.compile(experts, backend="aot_eager", fullgraph=True))
+    for a, b in zip(eager, compiled):
+        assert a.shape == b.shape and torch.equal(a, b)
+
+
+def test_rows_not_covered_by_the_counts_come_back_as_zeros(ops):
+    """Counts that add up to fewer rows than were passed (the reference asserts; here the device
+    clamps): the uncovered rows of the output and of the input gradient are zeros, never
+    uninitialised memory."""
+    from torchllmtuner_amd import moe
+
+    torch.manual_seed(1)
+    experts = moe.GroupedExperts(384, 384, 3).to(DEV).to(torch.bfloat16)
+    with torch.no_grad():
+        for p in experts.parameters():
+            p.normal_(0, 0.1)
+    x = torch.randn(40, 384, device=DEV).bfloat16().requires_grad_()
+    # poison the allocator's free blocks so that "uninitialised" cannot happen to be zero
+    junk = torch.full((40, 384), float("nan"), device=DEV, dtype=torch.bfloat16)
+    del junk
+    y = experts(x, torch.tensor([10, 0, 20], device=DEV))
+    assert torch.isfinite(y.float()).all() and not y[30:].any() and y[:30].any()
+    y.backward(torch.ones_like(y))
+    assert torch.isfinite(x.grad.float()).all() and not x.grad[30:].any()
+
+
+def test_plan_edge_cases_largest_expert_count_and_ids_out_of_range(ops):
+    """E = 2048, the largest expert count the plan accepts (its scan keeps 48 KiB in LDS there),
+    is still the stable argsort; one more expert is refused; a slot whose id lies outside [0, E)
+    is not counted and gets no row."""
+    g = torch.Generator().manual_seed(2)
+    T, K, E = 1500, 4, 2048
+    ids = torch.randint(0, E, (T, K), generator=g)
+    plan = ops.permute_plan(ids.to(DEV), E)
+    assert torch.equal(plan.counts_E.cpu().long(), torch.bincount(ids.reshape(-1), minlength=E))
+    assert torch.equal(plan.slot_of_row.cpu().long(), torch.argsort(ids.reshape(-1), stable=True))
+    with pytest.raises(ValueError, match="exceeds 2048"):
+        ops.permute_plan(ids.to(DEV), E + 1)
+    E = 8
+    ids = torch.randint(0, E, (64, 2), generator=g)
+    bad = ids.clone()
+    bad[3, 1], bad[17, 0] = E, -1
+    plan = ops.permute_plan(bad.to(DEV), E)
+    keep = (bad >= 0) & (bad < E)
+    assert torch.equal(plan.counts_E.cpu().long(), torch.bincount(bad[keep], minlength=E))
+    ros = plan.row_of_slot.cpu().view(64, 2)
+    assert ros[3, 1] == -1 and ros[17, 0] == -1 and int((ros >= 0).sum()) == 126
+    assert int(plan.total_rows) == 126

@@ -28,7 +28,7 @@ def test_library_loads_and_exports_every_declared_symbol():
         assert hasattr(raw, name), f"{name} is declared in mi355_moe.h but not exported"
         assert name in _lib.SIGNATURES, f"{name} has no ctypes prototype"
     assert set(_lib.SIGNATURES) == set(names)
-    assert lib.mi355_moe_abi_version() == 1
+    assert lib.mi355_moe_abi_version() == _lib.ABI_VERSION == 2
     assert lib.mi355_grouped_tile_m(1) in (128, 256)  # 256 unless MI355_ROW_LAYOUT=wide
 
 
@@ -37,7 +37,7 @@ def test_argument_validation_reports_errors_without_a_gpu():
 
     lib = _lib.load()
     # E = 0 is rejected before any launch
-    rc = lib.mi355_router_select_fwd(None, None, None, None, None, 4, 0, 1, 0, 0, 1.0, 0, 0, 0, None)
+    rc = lib.mi355_router_select_fwd(None, None, None, None, None, None, 4, 0, 1, 0, 0, 1.0, 0, 0, 0, None)
     assert rc == -1
     assert b"E=0" in lib.mi355_moe_last_error()
     rc = lib.mi355_permute_plan(None, 4, 2, 8, 5, 3, 1, 128, None, None, None, None, None, None, 8, None,
@@ -45,6 +45,35 @@ def test_argument_validation_reports_errors_without_a_gpu():
     assert rc == -1 and b"local range" in lib.mi355_moe_last_error()
     with pytest.raises(ValueError, match="local range"):
         _lib.check(rc, "permute_plan")
+
+
+def test_gather_entry_points_reject_unaddressable_token_matrices_without_launching():
+    """The fused token gather addresses its source with 32-bit byte offsets and clamps the
+    index to [0, num_tokens): a token matrix of 4 GiB or more, or an index with no rows to
+    point at, is MI355_EINVAL from every entry point that takes token_of_row -- checked on
+    the host, before anything is launched (this test runs without a GPU; the pointers are
+    never dereferenced)."""
+    from torchllmtuner_amd import _lib
+
+    lib = _lib.load()
+    p = 0x1000  # any non-null value
+    El, D, F, R, tiles = 4, 2048, 768, 1024, 16
+    too_many = (1 << 32) // (D * 2)  # T * D * 2 == 2^32 bytes
+    for T, needle in ((too_many, b"exceeds the 4 GiB"), (0, b"num_tokens = 0")):
+        rc = lib.mi355_grouped_swiglu_fwd(p, p, T, p, p, p, 1, p, p, p, p, p, tiles, p, p, p, p, El, D, F, R, None)
+        assert rc == -1 and needle in lib.mi355_moe_last_error(), lib.mi355_moe_last_error()
+        rc = lib.mi355_grouped_swiglu_bwd(p, p, p, T, p, p, p, p, p, p, 1, p, p, p, p, p, tiles, p, p, p, p, p, p,
+                                          El, D, F, R, None)
+        assert rc == -1 and needle in lib.mi355_moe_last_error()
+        rc = lib.mi355_grouped_swiglu_stage(1, p, p, p, T, p, p, p, p, p, p, p, p, p, p, p, p, tiles, p, p, p, p, p,
+                                            p, El, D, F, R, None)
+        assert rc == -1 and needle in lib.mi355_moe_last_error()
+        rc = lib.mi355_grouped_swiglu_combine_bwd(p, p, p, T, p, p, p, p, p, p, 1, p, p, p, p, p, tiles, p, p, p, p,
+                                                  p, p, p, p, El, D, F, R, 0, None)
+        assert rc == -1 and needle in lib.mi355_moe_last_error()
+    # fp32 rows cannot be gathered at all
+    rc = lib.mi355_grouped_swiglu_fwd(p, p, 8, p, p, p, 0, p, p, p, p, p, tiles, p, p, p, p, El, D, F, R, None)
+    assert rc == -1 and b"bf16 only" in lib.mi355_moe_last_error()
 
 
 def test_ops_refuse_cpu_tensors():
@@ -137,4 +166,4 @@ def test_header_is_plain_c_and_links_against_the_library(tmp_path):
          "-L", libdir, "-lmi355moe", f"-Wl,-rpath,{libdir}"],
         check=True, capture_output=True)
     out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
-    assert out == [str(len(names)), "1"]
+    assert out == [str(len(names)), str(_lib.ABI_VERSION)]

@@ -152,35 +152,64 @@ __global__ __launch_bounds__(256) void combine_bwd_kernel(
   const float w = lane < K ? weights[s0 + lane] : 0.0f;
   const T* g = dout + static_cast<int64_t>(t) * D;
   float my_dot = 0.0f;  // lane k keeps slot k's dot product
-  for (int k = 0; k < K; ++k) {
-    const int r = __shfl(row, k, kWave);
-    const float ww = __shfl(w, k, kWave);
-    if (r < 0) continue;
-    const T* yr = y + static_cast<int64_t>(r) * D;
-    T* dr = dy + static_cast<int64_t>(r) * D;
-    float dot = 0.0f;
-    if (D % V == 0) {
-      const int nv = D / V;
-      for (int i = lane; i < nv; i += kWave) {
-        float gf[V], yf[V], o[V];
-        Vec<T>::unpack(reinterpret_cast<const uint4*>(g)[i], gf);
-        Vec<T>::unpack(reinterpret_cast<const uint4*>(yr)[i], yf);
+  if (D % V == 0) {
+    // The token's gradient row is read ONCE per pass of G vectors per lane (4 KiB of the row per
+    // wave: all of it at D = 2048 bf16) and kept in registers while the K expert rows stream by;
+    // re-reading it per slot fetched it K times from wherever it had gone meanwhile.
+    const int nv = D / V;
+    constexpr int G = 4;
+    for (int base = 0; base < nv; base += G * kWave) {
+      float gf[G][V];
 #pragma unroll
-        for (int q = 0; q < V; ++q) {
-          dot += yf[q] * gf[q];
-          o[q] = gf[q] * ww;
-        }
-        reinterpret_cast<uint4*>(dr)[i] = Vec<T>::pack(o);
+      for (int q = 0; q < G; ++q) {
+        const int i = base + q * kWave + lane;
+        Vec<T>::unpack(i < nv ? reinterpret_cast<const uint4*>(g)[i] : make_uint4(0, 0, 0, 0), gf[q]);
       }
-    } else {
-      for (int i = lane; i < D; i += kWave) {
-        const float gf = load_as_f32(g + i);
-        dot += load_as_f32(yr + i) * gf;
-        store_from_f32(dr + i, gf * ww);
+      for (int k = 0; k < K; ++k) {
+        const int r = __shfl(row, k, kWave);
+        const float ww = __shfl(w, k, kWave);
+        if (r < 0) continue;
+        const uint4* yr = reinterpret_cast<const uint4*>(y + static_cast<int64_t>(r) * D);
+        uint4* dr = reinterpret_cast<uint4*>(dy + static_cast<int64_t>(r) * D);
+        uint4 yv[G];
+#pragma unroll
+        for (int q = 0; q < G; ++q) {
+          const int i = base + q * kWave + lane;
+          yv[q] = i < nv ? yr[i] : make_uint4(0, 0, 0, 0);
+        }
+        float dot = 0.0f;
+#pragma unroll
+        for (int q = 0; q < G; ++q) {
+          const int i = base + q * kWave + lane;
+          float yf[V], o[V];
+          Vec<T>::unpack(yv[q], yf);
+#pragma unroll
+          for (int c = 0; c < V; ++c) {
+            dot += yf[c] * gf[q][c];
+            o[c] = gf[q][c] * ww;
+          }
+          if (i < nv) dr[i] = Vec<T>::pack(o);
+        }
+        dot = wave_sum(dot);
+        if (lane == k) my_dot += dot;
       }
     }
-    dot = wave_sum(dot);
-    if (lane == k) my_dot = dot;
+  } else {
+    for (int k = 0; k < K; ++k) {
+      const int r = __shfl(row, k, kWave);
+      const float ww = __shfl(w, k, kWave);
+      if (r < 0) continue;
+      const T* yr = y + static_cast<int64_t>(r) * D;
+      T* dr = dy + static_cast<int64_t>(r) * D;
+      float dot = 0.0f;
+      for (int i = lane; i < D; i += kWave) {
+        const float gv = load_as_f32(g + i);
+        dot += load_as_f32(yr + i) * gv;
+        store_from_f32(dr + i, gv * ww);
+      }
+      dot = wave_sum(dot);
+      if (lane == k) my_dot = dot;
+    }
   }
   if (lane < K && dweights) dweights[s0 + lane] = my_dot;
 }

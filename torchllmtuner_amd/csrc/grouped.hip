@@ -15,15 +15,15 @@ int bf16_row_tile_m();
 // every dtype (a plan is built from expert ids alone, before the dtype of its rows is known;
 // the generic kernels walk tiles of any multiple of 64 rows)
 inline int tile_m_for(int dtype) { (void)dtype; return bf16_row_tile_m(); }
-int bf16_grouped_fwd(const void* rows, const int32_t* token_of_row, const void* w1, const void* w3,
-                     const void* w2, const int32_t* seg_offsets, const int32_t* seg_counts,
+int bf16_grouped_fwd(const void* rows, const int32_t* token_of_row, int64_t num_tokens, const void* w1,
+                     const void* w3, const void* w2, const int32_t* seg_offsets, const int32_t* seg_counts,
                      const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* num_tiles,
                      int64_t tile_capacity, void* gate, void* up, void* h, void* y, int64_t D,
                      int64_t F, int stages, hipStream_t s);
 int bf16_fused_dot_slots(int64_t F);
-int bf16_grouped_bwd(const void* dy, const void* rows, const int32_t* token_of_row, const void* w1,
-                     const void* w3, const void* w2, const void* gate, const void* up, const void* h,
-                     const float* row_scale, float* dot_partial,
+int bf16_grouped_bwd(const void* dy, const void* rows, const int32_t* token_of_row, int64_t num_tokens,
+                     const void* w1, const void* w3, const void* w2, const void* gate, const void* up,
+                     const void* h, const float* row_scale, float* dot_partial,
                      const int32_t* seg_offsets, const int32_t* seg_counts,
                      const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* num_tiles,
                      int64_t tile_capacity, void* dgate, void* dup, void* drows, void* dw1,
@@ -114,6 +114,19 @@ int check_common(const char* who, int dtype, int64_t El, int64_t D, int64_t F, i
   return MI355_OK;
 }
 
+// The fused token gather reads rows[token_of_row[r]] with a 32-bit byte offset and clamps the
+// index to [0, num_tokens): the token matrix must hold at least one row and stay below 4 GiB.
+int check_gather(const char* who, const int32_t* token_of_row, int64_t num_tokens, int64_t D, int dtype) {
+  if (!token_of_row) return MI355_OK;
+  MI355_REQUIRE(dtype == MI355_BF16, "%s: the token gather exists for bf16 only", who);
+  MI355_REQUIRE(num_tokens >= 1, "%s: token_of_row given but num_tokens = %lld", who, (long long)num_tokens);
+  MI355_REQUIRE(num_tokens < (1ll << 31) && num_tokens * D * 2 < (1ll << 32),
+                "%s: gathered token matrix of %lld x %lld bf16 exceeds the 4 GiB the fused gather addresses; "
+                "materialise the rows with mi355_permute_rows_fwd instead",
+                who, (long long)num_tokens, (long long)D);
+  return MI355_OK;
+}
+
 }  // namespace
 }  // namespace mi355
 
@@ -123,7 +136,7 @@ extern "C" int64_t mi355_grouped_tile_m(int dtype) {
   return tile_m_for(dtype);
 }
 
-extern "C" int mi355_grouped_swiglu_fwd(const void* rows, const int32_t* token_of_row,
+extern "C" int mi355_grouped_swiglu_fwd(const void* rows, const int32_t* token_of_row, int64_t num_tokens,
                                         const void* w1, const void* w3, const void* w2, int dtype, const int32_t* seg_offsets,
                                         const int32_t* seg_counts, const int32_t* tile_expert,
                                         const int32_t* tile_row0, const int32_t* num_tiles,
@@ -131,15 +144,15 @@ extern "C" int mi355_grouped_swiglu_fwd(const void* rows, const int32_t* token_o
                                         int64_t El, int64_t D, int64_t F, int64_t row_capacity,
                                         void* stream) {
   if (int rc = check_common("grouped_swiglu_fwd", dtype, El, D, F, row_capacity, tile_capacity)) return rc;
+  if (int rc = check_gather("grouped_swiglu_fwd", row_capacity > 0 ? token_of_row : nullptr, num_tokens, D, dtype)) return rc;
   if (row_capacity == 0 || tile_capacity == 0) return MI355_OK;
   MI355_REQUIRE(rows && w1 && w3 && w2 && seg_offsets && seg_counts && tile_expert && tile_row0 &&
                     num_tiles && gate && up && h && y,
                 "grouped_swiglu_fwd: null pointer");
   hipStream_t s = as_stream(stream);
   if (dtype == MI355_BF16 && bf16_fast_path_ok(D, F))
-    return bf16_grouped_fwd(rows, token_of_row, w1, w3, w2, seg_offsets, seg_counts,
-                                                             tile_expert, tile_row0, num_tiles,
-                                                             tile_capacity, gate, up, h, y, D, F, 3, s);
+    return bf16_grouped_fwd(rows, token_of_row, num_tokens, w1, w3, w2, seg_offsets, seg_counts, tile_expert,
+                            tile_row0, num_tiles, tile_capacity, gate, up, h, y, D, F, 3, s);
   if (token_of_row)
     return fail(MI355_EUNSUP, "grouped_swiglu_fwd: the token gather needs bf16 with D and F multiples of 64; "
                               "materialise the rows with mi355_permute_rows_fwd instead");
@@ -160,7 +173,7 @@ extern "C" int mi355_grouped_swiglu_fwd(const void* rows, const int32_t* token_o
 }
 
 extern "C" int mi355_grouped_swiglu_bwd(const void* dy, const void* rows,
-                                        const int32_t* token_of_row, const void* w1,
+                                        const int32_t* token_of_row, int64_t num_tokens, const void* w1,
                                         const void* w3, const void* w2, const void* gate,
                                         const void* up, const void* h, int dtype,
                                         const int32_t* seg_offsets, const int32_t* seg_counts,
@@ -170,6 +183,9 @@ extern "C" int mi355_grouped_swiglu_bwd(const void* dy, const void* rows,
                                         int64_t El, int64_t D, int64_t F, int64_t row_capacity,
                                         void* stream) {
   if (int rc = check_common("grouped_swiglu_bwd", dtype, El, D, F, row_capacity, tile_capacity)) return rc;
+  if (int rc = check_gather("grouped_swiglu_bwd", row_capacity > 0 && tile_capacity > 0 ? token_of_row : nullptr,
+                            num_tokens, D, dtype))
+    return rc;
   MI355_REQUIRE(seg_offsets && seg_counts && num_tiles, "grouped_swiglu_bwd: null plan pointer");
   MI355_REQUIRE(row_capacity == 0 || (dy && rows && w1 && w3 && w2 && gate && up && h && dgate && dup &&
                                       tile_expert && tile_row0),
@@ -177,8 +193,8 @@ extern "C" int mi355_grouped_swiglu_bwd(const void* dy, const void* rows,
   hipStream_t s = as_stream(stream);
   if (dtype == MI355_BF16 && bf16_fast_path_ok(D, F) && row_capacity > 0 && tile_capacity > 0)
     return bf16_grouped_bwd(
-        dy, rows, token_of_row, w1, w3, w2, gate, up, h, nullptr, nullptr, seg_offsets, seg_counts, tile_expert,
-        tile_row0, num_tiles, tile_capacity, dgate, dup, drows, dw1, dw3, dw2, El, D, F, 0x7c, s);
+        dy, rows, token_of_row, num_tokens, w1, w3, w2, gate, up, h, nullptr, nullptr, seg_offsets, seg_counts,
+        tile_expert, tile_row0, num_tiles, tile_capacity, dgate, dup, drows, dw1, dw3, dw2, El, D, F, 0x7c, s);
   // (with no rows at all nothing is gathered: only the zero weight gradients remain to be written)
   if (token_of_row && row_capacity > 0 && tile_capacity > 0)
     return fail(MI355_EUNSUP, "grouped_swiglu_bwd: the token gather needs bf16 with D and F multiples of 64");
@@ -209,7 +225,7 @@ extern "C" int mi355_grouped_swiglu_bwd(const void* dy, const void* rows,
 }
 
 extern "C" int mi355_grouped_swiglu_stage(int stage, const void* dy, const void* rows,
-                                          const int32_t* token_of_row, const void* w1, const void* w3, const void* w2, void* gate, void* up,
+                                          const int32_t* token_of_row, int64_t num_tokens, const void* w1, const void* w3, const void* w2, void* gate, void* up,
                                           void* h, void* y, const int32_t* seg_offsets,
                                           const int32_t* seg_counts, const int32_t* tile_expert,
                                           const int32_t* tile_row0, const int32_t* num_tiles,
@@ -220,14 +236,14 @@ extern "C" int mi355_grouped_swiglu_stage(int stage, const void* dy, const void*
   MI355_REQUIRE(bf16_fast_path_ok(D, F), "grouped_swiglu_stage: needs bf16 with D and F multiples of 64");
   MI355_REQUIRE(stage > 0 && stage < 128 && (stage & (stage - 1)) == 0, "grouped_swiglu_stage: one stage bit expected");
   if (row_capacity == 0 || tile_capacity == 0) return MI355_OK;
+  if (int rc = check_gather("grouped_swiglu_stage", token_of_row, num_tokens, D, MI355_BF16)) return rc;
   hipStream_t s = as_stream(stream);
   if (stage <= 2)
-    return bf16_grouped_fwd(rows, token_of_row, w1, w3, w2, seg_offsets, seg_counts,
-                                                             tile_expert, tile_row0, num_tiles,
-                                                             tile_capacity, gate, up, h, y, D, F, stage, s);
+    return bf16_grouped_fwd(rows, token_of_row, num_tokens, w1, w3, w2, seg_offsets, seg_counts, tile_expert,
+                            tile_row0, num_tiles, tile_capacity, gate, up, h, y, D, F, stage, s);
   return bf16_grouped_bwd(
-      dy, rows, token_of_row, w1, w3, w2, gate, up, h, nullptr, nullptr, seg_offsets, seg_counts, tile_expert,
-      tile_row0, num_tiles, tile_capacity, dgate, dup, drows, dw1, dw3, dw2, El, D, F, stage, s);
+      dy, rows, token_of_row, num_tokens, w1, w3, w2, gate, up, h, nullptr, nullptr, seg_offsets, seg_counts,
+      tile_expert, tile_row0, num_tiles, tile_capacity, dgate, dup, drows, dw1, dw3, dw2, El, D, F, stage, s);
 }
 
 extern "C" int64_t mi355_grouped_combine_bwd_slots(int dtype, int64_t D, int64_t F) {
@@ -236,27 +252,29 @@ extern "C" int64_t mi355_grouped_combine_bwd_slots(int dtype, int64_t D, int64_t
 }
 
 extern "C" int mi355_grouped_swiglu_combine_bwd(
-    const void* dout, const void* x, const int32_t* token_of_row, const float* row_scale, const void* w1,
-    const void* w3, const void* w2, const void* gate, const void* up, int dtype, const int32_t* seg_offsets,
+    const void* dout, const void* x, const int32_t* token_of_row, int64_t num_tokens, const float* row_scale,
+    const void* w1, const void* w3, const void* w2, const void* gate, const void* up, int dtype,
+    const int32_t* seg_offsets,
     const int32_t* seg_counts, const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* num_tiles,
     int64_t tile_capacity, void* dgate, void* dup, void* hs, float* dot_partial, void* drows, void* dw1,
     void* dw3, void* dw2, int64_t El, int64_t D, int64_t F, int64_t row_capacity, int stages, void* stream) {
   if (int rc = check_common("grouped_swiglu_combine_bwd", dtype, El, D, F, row_capacity, tile_capacity)) return rc;
   if (mi355_grouped_combine_bwd_slots(dtype, D, F) == 0)
-    return fail(MI355_EUNSUP, "grouped_swiglu_combine_bwd: needs bf16 with D and F multiples of 64 (>= 384) and the "
-                              "256-row tile layout; use mi355_combine_bwd + mi355_grouped_swiglu_bwd instead");
+    return fail(MI355_EUNSUP, "grouped_swiglu_combine_bwd: needs bf16 with D and F multiples of 64 (>= 384); "
+                              "use mi355_combine_bwd + mi355_grouped_swiglu_bwd instead");
   MI355_REQUIRE(seg_offsets && seg_counts && num_tiles, "grouped_swiglu_combine_bwd: null plan pointer");
   MI355_REQUIRE(stages >= 0 && (stages & ~0x7c) == 0, "grouped_swiglu_combine_bwd: stages must be 0 or a mask of the backward stages");
   if (row_capacity == 0 || tile_capacity == 0) {
     // no rows: the weight gradients are still defined (zeros); the plain entry point writes them
-    return mi355_grouped_swiglu_bwd(dout, x, token_of_row, w1, w3, w2, gate, up, hs, dtype, seg_offsets, seg_counts,
+    return mi355_grouped_swiglu_bwd(dout, x, token_of_row, num_tokens, w1, w3, w2, gate, up, hs, dtype, seg_offsets, seg_counts,
                                     tile_expert, tile_row0, num_tiles, tile_capacity, dgate, dup, drows, dw1, dw3,
                                     dw2, El, D, F, row_capacity, stream);
   }
   MI355_REQUIRE(dout && x && token_of_row && row_scale && w1 && w3 && w2 && gate && up && dgate && dup && hs &&
                     dot_partial && tile_expert && tile_row0,
                 "grouped_swiglu_combine_bwd: null pointer");
-  return bf16_grouped_bwd(dout, x, token_of_row, w1, w3, w2, gate, up, hs, row_scale, dot_partial, seg_offsets,
-                          seg_counts, tile_expert, tile_row0, num_tiles, tile_capacity, dgate, dup, drows, dw1, dw3,
-                          dw2, El, D, F, stages ? stages : 0x7c, as_stream(stream));
+  if (int rc = check_gather("grouped_swiglu_combine_bwd", token_of_row, num_tokens, D, dtype)) return rc;
+  return bf16_grouped_bwd(dout, x, token_of_row, num_tokens, w1, w3, w2, gate, up, hs, row_scale, dot_partial,
+                          seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles, tile_capacity, dgate, dup,
+                          drows, dw1, dw3, dw2, El, D, F, stages ? stages : 0x7c, as_stream(stream));
 }

@@ -11,10 +11,7 @@
 // gradients alike, eight waves per workgroup as 4 (rows) x 2 (columns), two per SIMD, each
 // wave a 64x128 accumulator tile; one workgroup per CU, two 64 KiB LDS stages of operand
 // tiles (overlaid by the eight 17 KiB epilogue regions).  Row tiles come from the
-// permutation plan's tile list (up to 256 rows of one expert each).  A 128x512 shape of the
-// row tile (waves 2 x 4; 384 wide when that divides the width and 512 does not) is kept
-// behind MI355_ROW_LAYOUT=wide: it stages a quarter more operand bytes per flop and fetches
-// an expert's weights twice as often, and measured 2-3 % slower per training step.
+// permutation plan's tile list (up to 256 rows of one expert each).
 //
 // What bounds them, measured on MI355X.  With operands of random bits the card's power
 // management holds the core clock near 1.5-1.9 GHz (2.4 GHz with constant operands): a
@@ -86,6 +83,7 @@ struct RowArgs {
   const uint16_t* gate;  // DH
   const uint16_t* up;    // DH
   const int32_t* a_src;  // GATEUP, DH: row -> row of a0 to read (token gather), or null
+  int a_rows;            // rows of a0 when a_src is given: gathered indices are clamped to [0, a_rows)
   // DH with a_src (the combine's backward folded in): a0 is the layer's output gradient (T, D),
   // row r stands for row_scale[r] * a0[a_src[r]]; o2 receives row_scale * h and dot_partial
   // [row][dot_slots] the pieces of <unscaled dh row, h row>, one per 128 output columns
@@ -104,8 +102,6 @@ struct RowArgs {
 // Row-tiled kernel: 64 WM rows of one expert x 32 NJ (8 / WM) output columns, 8 waves as WM
 // (rows) x 8 / WM (columns), each wave 64 x 32 NJ.  GATEUP's columns are half gate and half
 // up columns of the same f range, so a wave holds gate and up of the same 16 NJ f.
-constexpr int RBM = 128, RBN = 512;
-constexpr int R_STAGE = (RBM + RBN) * BK;  // elements per LDS stage (80 KiB)
 
 struct TileMeta {
   int e, row0, valid, n0, nt;
@@ -251,7 +247,7 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
 #pragma unroll
     for (int i = 0; i < NA; ++i) {
       const int r = max(min(kc_row + 64 * i, m.valid - 1), 0);
-      asrc[i] = GATHER ? p.a_src[m.row0 + r] : r;
+      asrc[i] = GATHER ? min(max(p.a_src[m.row0 + r], 0), p.a_rows - 1) : r;
     }
   };
   auto setup = [&](const TileMeta& m, const int (&asrc)[NA]) {
@@ -259,7 +255,8 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
     ubA0 = reinterpret_cast<const char*>(p.a0 + arow);
     ubA1 = (MODE == RM_DX) ? reinterpret_cast<const char*>(p.a1 + arow) : ubA0;
 #pragma unroll
-    for (int i = 0; i < NA; ++i) voffA[i] = static_cast<uint32_t>(max(asrc[i], 0) * lda + kc_chunk * 8) * 2u;
+    for (int i = 0; i < NA; ++i)
+      voffA[i] = (static_cast<uint32_t>(asrc[i]) * static_cast<uint32_t>(lda) + static_cast<uint32_t>(kc_chunk * 8)) * 2u;
     const uint16_t* B0 = p.b0 + m.e * wsz;
     const uint16_t* B1 = (MODE == RM_GATEUP || MODE == RM_DX) ? p.b1 + m.e * wsz : B0;
     b1_bytes = (B1 - B0) * 2;
@@ -610,6 +607,7 @@ struct WgradArgs {
   uint16_t* c;        // (El, M, N)
   const int32_t* a_src;  // row -> row of a to read, or null (GATHER_A)
   const int32_t* b_src;  // row -> row of b to read (token gather), or null
+  int src_rows;          // rows of the gathered operand: indices are clamped to [0, src_rows)
   const int32_t* seg_offsets;
   const int32_t* seg_counts;  // (2 El): row counts, then the local experts by descending count
   int El;
@@ -698,12 +696,12 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
   // (gather) the source row from the index array.  Needs c > 0.
   auto row_index = [&](int s0, int c, int step, int i) -> int {
     const int k = min(step * BK + ks_k + 16 * i, c - 1);
-    return GATHER ? max(p.b_src[s0 + k], 0) : k;
+    return GATHER ? min(max(p.b_src[s0 + k], 0), p.src_rows - 1) : k;
   };
   // the same for the A row (its own row unless A is gathered too)
   auto a_row_index = [&](int s0, int c, int step, int i) -> int {
     const int k = min(step * BK + ks_k + 16 * i, c - 1);
-    return GATHER_A ? max(p.a_src[s0 + k], 0) : k;
+    return GATHER_A ? min(max(p.a_src[s0 + k], 0), p.src_rows - 1) : k;
   };
   // Loads of one K step, unconditional: rows past the segment re-read its last row and
   // the A side is zeroed when it is parked, so the products vanish.  Needs cnt > 0.
@@ -887,21 +885,7 @@ int set_lds(K kernel, int bytes) {
 
 // The MFMA path needs whole 64-wide K steps, 16-byte aligned rows, and outputs at least
 // one tile wide (a last tile that would overhang is shifted back, never clamped).
-// Two shapes of the row tile: 128 rows x 512 columns (waves 2 x 4) or 256 x 256 (waves 4 x 2).
-// The square one stages a fifth fewer operand bytes per flop and halves how often an
-// expert's weights are fetched, at the price of a coarser last tile per expert.
-// The square one is the default (measured 2-3 % faster per training step on balanced, skewed
-// and few-rows-per-expert routing alike); MI355_ROW_LAYOUT=wide, read once per process,
-// selects the other.
-static bool tall_layout() {
-  static const bool tall = [] {
-    const char* v = std::getenv("MI355_ROW_LAYOUT");
-    return !(v && v[0] == 'w');
-  }();
-  return tall;
-}
-
-int bf16_row_tile_m() { return tall_layout() ? 256 : 128; }
+int bf16_row_tile_m() { return 256; }
 
 bool bf16_fast_path_ok(int64_t D, int64_t F) { return D % 64 == 0 && F % 64 == 0 && D >= 384 && F >= 384; }
 
@@ -922,56 +906,36 @@ static unsigned resident_blocks() {
   return n;
 }
 
-constexpr int R_LDS_BYTES = 2 * R_STAGE * 2;  // 163840
 constexpr int W_LDS_BYTES = 8 * 64 * 136 * 2;  // 139264: the 8 epilogue regions (> 2 stages = 131072)
 
-template <int MODE, int NJ, bool GATHER, int WM>
-static int launch_row_as(RowArgs& a, int64_t tile_capacity, hipStream_t s, const char* what) {
-  constexpr int lds = WM == 4 ? W_LDS_BYTES : R_LDS_BYTES;
-  static PerDeviceOnce configured;  // one per kernel instantiation
-  if (configured.needed()) {
-    if (int rc = set_lds(row_tiled_kernel<MODE, NJ, GATHER, WM>, lds)) return rc;
-    configured.done();
-  }
-  const unsigned blocks = std::min(round8(tile_capacity * a.n_tiles), resident_blocks());
-  hipLaunchKernelGGL((row_tiled_kernel<MODE, NJ, GATHER, WM>), dim3(blocks), dim3(NT), lds, s, a);
-  return check_launch(what);
-}
-
-// 384-column tiles when they divide the width and 512-column tiles do not (F = 768), or
-// when the output is narrower than 512 columns.
-static bool narrow_tiles(int64_t width) { return width < 512 || (width % 512 != 0 && width % 384 == 0); }
-
-// width: output columns; gate/up tiles hold both halves of their column range
+// width: output columns; gate/up tiles hold both halves of their column range.  Tiles are always
+// 256 wide (a 192-wide KS tile would not hold the swizzle: 24 chunks per row are not a multiple
+// of the 16 the key permutes); an overhanging last tile shifts back.
 template <int MODE, bool GATHER = false>
 static int launch_row(RowArgs& a, int64_t width, int64_t tile_capacity, hipStream_t s, const char* what) {
   constexpr int div = MODE == RM_GATEUP ? 2 : 1;
-  if (tall_layout()) {
-    // always 256 wide: a 192-wide KS tile would not hold the swizzle (24 chunks per row are
-    // not a multiple of the 16 the key permutes); an overhanging last tile shifts back
-    a.n_tiles = (int)((width + 256 / div - 1) / (256 / div));
-    return launch_row_as<MODE, 4, GATHER, 4>(a, tile_capacity, s, what);
+  a.n_tiles = (int)((width + 256 / div - 1) / (256 / div));
+  static PerDeviceOnce configured;  // one per kernel instantiation
+  if (configured.needed()) {
+    if (int rc = set_lds(row_tiled_kernel<MODE, 4, GATHER, 4>, W_LDS_BYTES)) return rc;
+    configured.done();
   }
-  if constexpr (MODE != RM_GATEUP) {
-    if (narrow_tiles(width)) {
-      a.n_tiles = (int)((width + 383) / 384);
-      return launch_row_as<MODE, 3, GATHER, 2>(a, tile_capacity, s, what);
-    }
-  }
-  a.n_tiles = (int)((width + RBN / div - 1) / (RBN / div));
-  return launch_row_as<MODE, 4, GATHER, 2>(a, tile_capacity, s, what);
+  const unsigned blocks = std::min(round8(tile_capacity * a.n_tiles), resident_blocks());
+  hipLaunchKernelGGL((row_tiled_kernel<MODE, 4, GATHER, 4>), dim3(blocks), dim3(NT), W_LDS_BYTES, s, a);
+  return check_launch(what);
 }
 
-int bf16_grouped_fwd(const void* rows, const int32_t* token_of_row, const void* w1, const void* w3,
-                       const void* w2, const int32_t* seg_offsets, const int32_t* seg_counts,
-                       const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* num_tiles,
-                       int64_t tile_capacity, void* gate, void* up, void* h, void* y, int64_t D,
-                       int64_t F, int stages, hipStream_t s) {
+int bf16_grouped_fwd(const void* rows, const int32_t* token_of_row, int64_t num_tokens, const void* w1,
+                     const void* w3, const void* w2, const int32_t* seg_offsets, const int32_t* seg_counts,
+                     const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* num_tiles,
+                     int64_t tile_capacity, void* gate, void* up, void* h, void* y, int64_t D,
+                     int64_t F, int stages, hipStream_t s) {
   RowArgs a{};
   a.seg_offsets = seg_offsets; a.seg_counts = seg_counts; a.tile_expert = tile_expert;
   a.tile_row0 = tile_row0; a.num_tiles = num_tiles; a.D = (int)D; a.F = (int)F;
   if (stages & STAGE_GATEUP) {
-    a.a0 = (const uint16_t*)rows; a.a_src = token_of_row; a.b0 = (const uint16_t*)w1; a.b1 = (const uint16_t*)w3;
+    a.a0 = (const uint16_t*)rows; a.a_src = token_of_row; a.a_rows = (int)num_tokens;
+    a.b0 = (const uint16_t*)w1; a.b1 = (const uint16_t*)w3;
     a.o0 = (uint16_t*)gate; a.o1 = (uint16_t*)up; a.o2 = (uint16_t*)h;
     if (token_of_row) {
       if (int rc = launch_row<RM_GATEUP, true>(a, F, tile_capacity, s, "grouped gate/up")) return rc;
@@ -981,6 +945,7 @@ int bf16_grouped_fwd(const void* rows, const int32_t* token_of_row, const void* 
   }
   if (stages & STAGE_DOWN) {
     RowArgs b = a;
+    b.a_src = nullptr;
     b.a0 = (const uint16_t*)h; b.b0 = (const uint16_t*)w2; b.o0 = (uint16_t*)y;
     if (int rc = launch_row<RM_DOWN>(b, D, tile_capacity, s, "grouped down")) return rc;
   }
@@ -989,20 +954,20 @@ int bf16_grouped_fwd(const void* rows, const int32_t* token_of_row, const void* 
 
 int bf16_fused_dot_slots(int64_t F) {
   // one partial per 128 output columns of the dH tile (two waves across its 256 columns)
-  return tall_layout() ? (int)((F + 255) / 256) * 2 : 0;
+  return (int)((F + 255) / 256) * 2;
 }
 
 // row_scale != null: the combine's backward is folded in.  dy is then the layer's output
 // gradient (T, D), read through token_of_row and scaled by row_scale; `h` is written (it
 // receives row_scale * h, the operand of dW2) and dot_partial gets the score-gradient pieces.
-int bf16_grouped_bwd(const void* dy, const void* rows, const int32_t* token_of_row, const void* w1,
-                       const void* w3, const void* w2, const void* gate, const void* up, const void* h,
-                       const float* row_scale, float* dot_partial,
-                       const int32_t* seg_offsets, const int32_t* seg_counts,
-                       const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* num_tiles,
-                       int64_t tile_capacity, void* dgate, void* dup, void* drows, void* dw1,
-                       void* dw3, void* dw2, int64_t El, int64_t D, int64_t F, int stages,
-                       hipStream_t s) {
+int bf16_grouped_bwd(const void* dy, const void* rows, const int32_t* token_of_row, int64_t num_tokens,
+                     const void* w1, const void* w3, const void* w2, const void* gate, const void* up,
+                     const void* h, const float* row_scale, float* dot_partial,
+                     const int32_t* seg_offsets, const int32_t* seg_counts,
+                     const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* num_tiles,
+                     int64_t tile_capacity, void* dgate, void* dup, void* drows, void* dw1,
+                     void* dw3, void* dw2, int64_t El, int64_t D, int64_t F, int stages,
+                     hipStream_t s) {
   RowArgs a{};
   a.seg_offsets = seg_offsets; a.seg_counts = seg_counts; a.tile_expert = tile_expert;
   a.tile_row0 = tile_row0; a.num_tiles = num_tiles; a.D = (int)D; a.F = (int)F;
@@ -1011,12 +976,10 @@ int bf16_grouped_bwd(const void* dy, const void* rows, const int32_t* token_of_r
     a.gate = (const uint16_t*)gate; a.up = (const uint16_t*)up;
     a.o0 = (uint16_t*)dgate; a.o1 = (uint16_t*)dup;
     if (row_scale) {
-      if (!tall_layout()) return fail(MI355_EUNSUP, "grouped dh: the folded combine needs the 256-row tile layout");
-      a.a_src = token_of_row; a.row_scale = row_scale; a.dot_partial = dot_partial;
+      a.a_src = token_of_row; a.a_rows = (int)num_tokens; a.row_scale = row_scale; a.dot_partial = dot_partial;
       a.o2 = (uint16_t*)const_cast<void*>(h);
       a.dot_slots = bf16_fused_dot_slots(F);
-      a.n_tiles = (int)((F + 255) / 256);
-      if (int rc = launch_row_as<RM_DH, 4, true, 4>(a, tile_capacity, s, "grouped dh + combine")) return rc;
+      if (int rc = launch_row<RM_DH, true>(a, F, tile_capacity, s, "grouped dh + combine")) return rc;
       a.a_src = nullptr;
     } else {
       if (int rc = launch_row<RM_DH>(a, F, tile_capacity, s, "grouped dh")) return rc;
@@ -1039,6 +1002,7 @@ int bf16_grouped_bwd(const void* dy, const void* rows, const int32_t* token_of_r
                    const int32_t* a_src = nullptr) {
     WgradArgs w{};
     w.a = (const uint16_t*)A; w.b = (const uint16_t*)B; w.c = (uint16_t*)C; w.b_src = b_src; w.a_src = a_src;
+    w.src_rows = (int)num_tokens;
     w.seg_offsets = seg_offsets; w.seg_counts = seg_counts; w.El = (int)El; w.M = (int)M; w.N = (int)N;
     w.m_tiles = (int)((M + WBM - 1) / WBM); w.n_tiles = (int)((N + WBN - 1) / WBN);
     w.total = (int)(El * w.m_tiles * w.n_tiles);
@@ -1060,4 +1024,3 @@ int bf16_grouped_bwd(const void* dy, const void* rows, const int32_t* token_of_r
 }
 
 }  // namespace mi355
-

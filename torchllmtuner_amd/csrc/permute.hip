@@ -11,7 +11,7 @@
 //                   stable), the padded segment offsets, and the MFMA tile list.
 //   3. plan_rows    row = segment offset + waves-before + rank-in-wave, written both
 //                   ways (row_of_slot, slot_of_row).
-// The row movers are pure bandwidth kernels: one wave per row, 16-byte lanes.
+// The row movers are pure bandwidth kernels: one wave per token, 16-byte lanes.
 #include "common.h"
 
 namespace mi355 {
@@ -37,7 +37,7 @@ __global__ __launch_bounds__(256) void plan_rank_kernel(const int64_t* __restric
     const int slot = begin + c + lane;
     const bool valid = slot < N;
     int e = valid ? static_cast<int>(ids[slot]) : -1;
-    if (e < 0 || e >= E) e = valid ? 0 : -1;  // out-of-range ids are folded, never written OOB
+    if (e < 0 || e >= E) e = -1;  // an id outside [0, E) is not counted and gets no row
     // rank among the chunk's lower lanes with the same expert, and whether a higher lane
     // holds it too: 64 uniform-lane reads, no LDS round trip per distinct expert
     int below = 0, above = 0;
@@ -48,7 +48,7 @@ __global__ __launch_bounds__(256) void plan_rank_kernel(const int64_t* __restric
       below += (j < lane) ? same : 0;
       above += (j > lane) ? same : 0;
     }
-    if (valid) {
+    if (e >= 0) {
       const int base = my[e];
       rank_in_wave[slot] = base + below;
       __builtin_amdgcn_wave_barrier();
@@ -246,8 +246,7 @@ __global__ __launch_bounds__(256) void plan_rows_kernel(
     int32_t* __restrict__ token_of_row, int row_capacity) {
   const int slot = blockIdx.x * blockDim.x + threadIdx.x;
   if (slot >= N) return;
-  int e = static_cast<int>(ids[slot]);
-  if (e < 0 || e >= E) e = 0;
+  const int e = static_cast<int>(ids[slot]);  // outside [0, E): outside [lo, hi) too, no row
   int row = -1;
   if (e >= lo && e < hi) {
     const int gw = slot / kSlotsPerWave;
@@ -263,29 +262,63 @@ __global__ __launch_bounds__(256) void plan_rows_kernel(
 }
 
 // ---- row movers ---------------------------------------------------------------
-// One wave per row; VEC = 16-byte vectors when the row length allows, else scalars.
+// 16-byte vectors when the row length allows, else scalars.
+//
+// rows[row_of_slot[t*K + k]] = x[t]: one wave per token reads the token row ONCE and stores its
+// K copies (walking the rows instead re-fetches every token row K times from wherever it has
+// gone meanwhile: 1.7x the algorithmic traffic at K = 8).  Waves past the tokens zero the
+// padding rows (slot_of_row < 0) below *total_rows.
 template <typename T>
 __global__ __launch_bounds__(256) void permute_rows_fwd_kernel(
-    const T* __restrict__ x, const int32_t* __restrict__ slot_of_row,
-    const int32_t* __restrict__ total_rows, T* __restrict__ rows, int D, int K, int row_capacity) {
+    const T* __restrict__ x, const int32_t* __restrict__ row_of_slot, const int32_t* __restrict__ slot_of_row,
+    const int32_t* __restrict__ total_rows, T* __restrict__ rows, int T_, int D, int K, int token_blocks,
+    int row_capacity) {
   const int lane = threadIdx.x & 63;
-  const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (r >= row_capacity || r >= *total_rows) return;
-  const int slot = slot_of_row[r];
-  T* dst = rows + static_cast<int64_t>(r) * D;
   constexpr int V = 16 / sizeof(T);
-  if (D % V == 0) {
-    uint4* d4 = reinterpret_cast<uint4*>(dst);
-    const int nv = D / V;
-    if (slot < 0) {
-      for (int i = lane; i < nv; i += kWave) d4[i] = make_uint4(0, 0, 0, 0);
+  if (static_cast<int>(blockIdx.x) >= token_blocks) {
+    const int r = (blockIdx.x - token_blocks) * 4 + (threadIdx.x >> 6);
+    if (r >= row_capacity || r >= *total_rows || slot_of_row[r] >= 0) return;
+    T* dst = rows + static_cast<int64_t>(r) * D;
+    if (D % V == 0) {
+      for (int i = lane; i < D / V; i += kWave) reinterpret_cast<uint4*>(dst)[i] = make_uint4(0, 0, 0, 0);
     } else {
-      const uint4* s4 = reinterpret_cast<const uint4*>(x + static_cast<int64_t>(slot / K) * D);
-      for (int i = lane; i < nv; i += kWave) d4[i] = s4[i];
+      for (int i = lane; i < D; i += kWave) dst[i] = T(0);
+    }
+    return;
+  }
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= T_) return;
+  const int64_t s0 = static_cast<int64_t>(t) * K;
+  const T* src = x + static_cast<int64_t>(t) * D;
+  if (D % V == 0) {
+    const int nv = D / V;
+    constexpr int G = 4;  // vectors per lane and pass: 4 KiB of the row in flight per wave
+    for (int base = 0; base < nv; base += G * kWave) {
+      uint4 v[G];
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        const int i = base + g * kWave + lane;
+        v[g] = i < nv ? reinterpret_cast<const uint4*>(src)[i] : make_uint4(0, 0, 0, 0);
+      }
+      for (int k = 0; k < K; ++k) {
+        int row = row_of_slot[s0 + k];  // wave-uniform
+        if (row < 0 || row >= row_capacity) continue;
+        uint4* d4 = reinterpret_cast<uint4*>(rows + static_cast<int64_t>(row) * D);
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+          const int i = base + g * kWave + lane;
+          if (i < nv) d4[i] = v[g];
+        }
+      }
     }
   } else {
-    const T* src = x + static_cast<int64_t>(slot < 0 ? 0 : slot / K) * D;
-    for (int i = lane; i < D; i += kWave) dst[i] = slot < 0 ? T(0) : src[i];
+    for (int i = lane; i < D; i += kWave) {
+      const T v = src[i];
+      for (int k = 0; k < K; ++k) {
+        const int row = row_of_slot[s0 + k];
+        if (row >= 0 && row < row_capacity) rows[static_cast<int64_t>(row) * D + i] = v;
+      }
+    }
   }
 }
 
@@ -382,17 +415,16 @@ extern "C" int64_t mi355_permute_plan_workspace_bytes(int64_t T, int64_t K, int6
   return (N + 2 * plan_num_blocks(N) * kWavesPerBlock * E + 64) * (int64_t)sizeof(int32_t);
 }
 
-extern "C" int mi355_permute_plan(const int64_t* ids, int64_t T, int64_t K, int64_t E,
-                                  int64_t lo, int64_t hi, int64_t align, int64_t tile_m,
-                                  int32_t* counts_E, int32_t* seg_offsets, int32_t* seg_counts,
-                                  int32_t* row_of_slot, int32_t* slot_of_row,
-                                  int32_t* token_of_row, int64_t row_capacity, int32_t* tile_expert, int32_t* tile_row0,
-                                  int32_t* num_tiles, int64_t tile_capacity, void* workspace,
-                                  void* stream) {
+static int plan_impl(const int64_t* ids, int64_t T, int64_t K, int64_t E, int64_t lo, int64_t hi, int64_t align,
+                     int64_t tile_m, int32_t* counts_E, int32_t* seg_offsets, int32_t* seg_counts,
+                     int32_t* row_of_slot, int32_t* slot_of_row, int32_t* token_of_row, int64_t row_capacity,
+                     int32_t* tile_expert, int32_t* tile_row0, int32_t* num_tiles, int64_t tile_capacity,
+                     void* workspace, hipStream_t s) {
   const int64_t N = T * K;
   MI355_REQUIRE(T >= 0 && K >= 1 && E >= 1 && N < (1ll << 30), "permute_plan: bad shape T=%lld K=%lld E=%lld",
                 (long long)T, (long long)K, (long long)E);
-  MI355_REQUIRE(E <= 4096, "permute_plan: E=%lld exceeds 4096", (long long)E);
+  // (the scan workgroup keeps (parts + 1) * E + 4 * El + 2 words in LDS: 48 KiB at E = 2048)
+  MI355_REQUIRE(E <= 2048, "permute_plan: E=%lld exceeds 2048", (long long)E);
   MI355_REQUIRE(0 <= lo && lo < hi && hi <= E, "permute_plan: bad local range [%lld,%lld)", (long long)lo, (long long)hi);
   MI355_REQUIRE(align >= 1 && tile_m >= 1, "permute_plan: align and tile_m must be positive");
   MI355_REQUIRE(row_capacity >= 0 && row_capacity < (1ll << 31) && tile_capacity >= 0,
@@ -401,7 +433,6 @@ extern "C" int mi355_permute_plan(const int64_t* ids, int64_t T, int64_t K, int6
                 "permute_plan: null pointer");
   MI355_REQUIRE(N == 0 || (ids && row_of_slot), "permute_plan: null pointer");
   MI355_REQUIRE(row_capacity == 0 || slot_of_row, "permute_plan: null slot_of_row");
-  hipStream_t s = as_stream(stream);
   int32_t* rank_in_wave = static_cast<int32_t*>(workspace);
   int32_t* wave_hist = rank_in_wave + N;
   const int nblocks = (int)plan_num_blocks(N);
@@ -435,23 +466,39 @@ extern "C" int mi355_permute_plan(const int64_t* ids, int64_t T, int64_t K, int6
   return MI355_OK;
 }
 
-extern "C" int mi355_permute_rows_fwd(const void* x, int dtype, const int32_t* slot_of_row,
-                                      const int32_t* total_rows, void* rows, int64_t T, int64_t D,
-                                      int64_t K, int64_t row_capacity, void* stream) {
-  MI355_REQUIRE(D >= 1 && K >= 1 && T >= 0 && row_capacity >= 0 && row_capacity < (1ll << 31) &&
-                    D < (1ll << 31),
+extern "C" int mi355_permute_plan(const int64_t* ids, int64_t T, int64_t K, int64_t E,
+                                  int64_t lo, int64_t hi, int64_t align, int64_t tile_m,
+                                  int32_t* counts_E, int32_t* seg_offsets, int32_t* seg_counts,
+                                  int32_t* row_of_slot, int32_t* slot_of_row,
+                                  int32_t* token_of_row, int64_t row_capacity, int32_t* tile_expert, int32_t* tile_row0,
+                                  int32_t* num_tiles, int64_t tile_capacity, void* workspace,
+                                  void* stream) {
+  return plan_impl(ids, T, K, E, lo, hi, align, tile_m, counts_E, seg_offsets, seg_counts, row_of_slot, slot_of_row,
+                   token_of_row, row_capacity, tile_expert, tile_row0, num_tiles, tile_capacity, workspace,
+                   as_stream(stream));
+}
+
+extern "C" int mi355_permute_rows_fwd(const void* x, int dtype, const int32_t* row_of_slot,
+                                      const int32_t* slot_of_row, const int32_t* total_rows, void* rows,
+                                      int64_t T, int64_t D, int64_t K, int64_t row_capacity, void* stream) {
+  MI355_REQUIRE(D >= 1 && K >= 1 && T >= 0 && T < (1ll << 31) && T * K < (1ll << 31) && row_capacity >= 0 &&
+                    row_capacity < (1ll << 31) && D < (1ll << 31),
                 "permute_rows_fwd: bad shape");
   if (row_capacity == 0) return MI355_OK;
-  MI355_REQUIRE(slot_of_row && total_rows && rows && (x || T == 0), "permute_rows_fwd: null pointer");
-  const dim3 grid((unsigned)((row_capacity + 3) / 4));
+  MI355_REQUIRE(rows && (T == 0 || (x && row_of_slot)), "permute_rows_fwd: null pointer");
+  MI355_REQUIRE(!slot_of_row || total_rows, "permute_rows_fwd: total_rows required with slot_of_row");
+  const int token_blocks = (int)((T + 3) / 4);
+  const int pad_blocks = slot_of_row ? (int)((row_capacity + 3) / 4) : 0;
+  if (token_blocks + pad_blocks == 0) return MI355_OK;
+  const dim3 grid((unsigned)(token_blocks + pad_blocks));
   if (dtype == MI355_F32)
     hipLaunchKernelGGL(permute_rows_fwd_kernel<float>, grid, dim3(256), 0, as_stream(stream),
-                       static_cast<const float*>(x), slot_of_row, total_rows,
-                       static_cast<float*>(rows), (int)D, (int)K, (int)row_capacity);
+                       static_cast<const float*>(x), row_of_slot, slot_of_row, total_rows,
+                       static_cast<float*>(rows), (int)T, (int)D, (int)K, token_blocks, (int)row_capacity);
   else if (dtype == MI355_BF16)
     hipLaunchKernelGGL(permute_rows_fwd_kernel<uint16_t>, grid, dim3(256), 0, as_stream(stream),
-                       static_cast<const uint16_t*>(x), slot_of_row, total_rows,
-                       static_cast<uint16_t*>(rows), (int)D, (int)K, (int)row_capacity);
+                       static_cast<const uint16_t*>(x), row_of_slot, slot_of_row, total_rows,
+                       static_cast<uint16_t*>(rows), (int)T, (int)D, (int)K, token_blocks, (int)row_capacity);
   else
     return fail(MI355_EINVAL, "permute_rows_fwd: unknown dtype %d", dtype);
   return check_launch("permute_rows_fwd");

@@ -37,8 +37,7 @@ __device__ __forceinline__ float pick(const float (&a)[VPL], int j) {
 
 template <int VPL>
 __device__ __forceinline__ void compute_scores(const float* __restrict__ row, int E, int lane,
-                                               int score_func, float (&s)[VPL]) {
-  float x[VPL];
+                                               int score_func, float (&s)[VPL], float (&x)[VPL]) {
 #pragma unroll
   for (int j = 0; j < VPL; ++j) {
     const int e = lane + j * kWave;
@@ -71,14 +70,15 @@ template <int VPL>
 __global__ __launch_bounds__(256) void select_fwd_kernel(
     const float* __restrict__ logits, const float* __restrict__ expert_bias,
     float* __restrict__ weights, int64_t* __restrict__ ids, float* __restrict__ scores_out,
-    float* __restrict__ cutoff_out, int T, int E, int K, int score_func, int route_norm,
+    uint8_t* __restrict__ map_out, float* __restrict__ cutoff_out, int T, int E, int K, int score_func,
+    int route_norm,
     float route_scale, int num_groups, int num_limited, int mode) {
   const int lane = threadIdx.x & 63;
   const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= T) return;
 
-  float s[VPL];
-  compute_scores<VPL>(logits + static_cast<int64_t>(t) * E, E, lane, score_func, s);
+  float s[VPL], x[VPL];
+  compute_scores<VPL>(logits + static_cast<int64_t>(t) * E, E, lane, score_func, s, x);
   if (scores_out) {
 #pragma unroll
     for (int j = 0; j < VPL; ++j)
@@ -89,11 +89,16 @@ __global__ __launch_bounds__(256) void select_fwd_kernel(
   int my_id = 0;
 
   if (mode == MI355_SELECT_TOPK) {
+    // Choice values.  Without a bias and without groups the choice is the plain top-k of the
+    // scores, and every score function here is non-decreasing in the logit: the experts are
+    // then chosen by LOGIT, which is exact -- two implementations of exp() that differ in the
+    // last ulp can order two nearly equal scores differently, but never two logits.
+    const bool by_logit = !expert_bias && num_groups == 0;
     float c[VPL];
 #pragma unroll
     for (int j = 0; j < VPL; ++j) {
       const int e = lane + j * kWave;
-      c[j] = e < E ? (expert_bias ? s[j] + expert_bias[e] : s[j]) : -INFINITY;
+      c[j] = e < E ? (by_logit ? x[j] : (expert_bias ? s[j] + expert_bias[e] : s[j])) : -INFINITY;
     }
     unsigned taken = 0;
 #pragma unroll
@@ -197,6 +202,17 @@ __global__ __launch_bounds__(256) void select_fwd_kernel(
     weights[static_cast<int64_t>(t) * K + lane] = my_w;
     ids[static_cast<int64_t>(t) * K + lane] = my_id;
   }
+  if (map_out) {
+    // one-hot routing map of the token, one byte per expert
+    unsigned chosen = 0;
+    for (int k = 0; k < K; ++k) {
+      const int idk = __shfl(my_id, k, kWave);
+      if ((idk & 63) == lane) chosen |= 1u << (idk >> 6);
+    }
+#pragma unroll
+    for (int j = 0; j < VPL; ++j)
+      if (lane + j * kWave < E) map_out[static_cast<int64_t>(t) * E + lane + j * kWave] = (chosen >> j) & 1u;
+  }
 }
 
 template <int VPL>
@@ -215,7 +231,8 @@ __global__ __launch_bounds__(256) void select_bwd_kernel(
 
   const float* row = logits + static_cast<int64_t>(t) * E;
   float s[VPL];
-  compute_scores<VPL>(row, E, lane, score_func, s);
+  float xs[VPL];
+  compute_scores<VPL>(row, E, lane, score_func, s, xs);
 #pragma unroll
   for (int j = 0; j < VPL; ++j) {
     const int e = lane + j * kWave;
@@ -387,10 +404,10 @@ extern "C" int mi355_router_gate_bwd(const float* dlogits, const void* x, int x_
   } while (0)
 
 extern "C" int mi355_router_select_fwd(const float* logits, const float* expert_bias,
-                                       float* weights, int64_t* ids, float* scores_TE, int64_t T,
-                                       int64_t E, int64_t K, int score_func, int route_norm,
-                                       float route_scale, int num_groups, int num_limited,
-                                       int select_mode, void* stream) {
+                                       float* weights, int64_t* ids, float* scores_TE,
+                                       uint8_t* routing_map_TE, int64_t T, int64_t E, int64_t K,
+                                       int score_func, int route_norm, float route_scale, int num_groups,
+                                       int num_limited, int select_mode, void* stream) {
   if (int rc = check_router_args(T, E, K)) return rc;
   MI355_REQUIRE(score_func >= 0 && score_func <= 2, "router_select_fwd: unknown score_func %d", score_func);
   MI355_REQUIRE(select_mode >= 0 && select_mode <= 2, "router_select_fwd: unknown select_mode %d", select_mode);
@@ -405,7 +422,7 @@ extern "C" int mi355_router_select_fwd(const float* logits, const float* expert_
   MI355_REQUIRE(logits && weights && ids, "router_select_fwd: null pointer");
   const dim3 grid((unsigned)((T + 3) / 4));
   DISPATCH_VPL(E, hipLaunchKernelGGL(select_fwd_kernel<VPL>, grid, dim3(256), 0, as_stream(stream),
-                                     logits, expert_bias, weights, ids, scores_TE,
+                                     logits, expert_bias, weights, ids, scores_TE, routing_map_TE,
                                      static_cast<float*>(nullptr), (int)T, (int)E, (int)K, score_func,
                                      route_norm, route_scale, num_groups, num_limited, select_mode));
   return check_launch("router_select_fwd");
@@ -425,7 +442,8 @@ extern "C" int mi355_router_select_cutoff_fwd(const float* logits, const float* 
   MI355_REQUIRE(logits && weights && ids && cutoff_T, "router_select_cutoff_fwd: null pointer");
   const dim3 grid((unsigned)((T + 3) / 4));
   DISPATCH_VPL(E, hipLaunchKernelGGL(select_fwd_kernel<VPL>, grid, dim3(256), 0, as_stream(stream),
-                                     logits, expert_bias, weights, ids, scores_TE, cutoff_T, (int)T,
+                                     logits, expert_bias, weights, ids, scores_TE,
+                                     static_cast<uint8_t*>(nullptr), cutoff_T, (int)T,
                                      (int)E, (int)K, score_func, route_norm, route_scale, 0, 0,
                                      MI355_SELECT_TOPK));
   return check_launch("router_select_cutoff_fwd");

@@ -95,21 +95,6 @@ class AuxLoss(nn.Module):
         return AuxLossInjection.apply(carrier, injected)
 
 
-class _BalanceLossFunction(torch.autograd.Function):
-    @staticmethod
-    def forward(ctx, scores_TE, routing_map_TE, padding_mask_T):
-        loss, f_E = ops.balance_loss_fwd(scores_TE, routing_map_TE, padding_mask_T)
-        ctx.save_for_backward(scores_TE, f_E)
-        ctx.padding = padding_mask_T
-        return loss
-
-    @staticmethod
-    @once_differentiable
-    def backward(ctx, grad_loss):
-        scores_TE, f_E = ctx.saved_tensors
-        return ops.balance_loss_bwd(scores_TE, f_E, grad_loss, ctx.padding), None, None
-
-
 class MicrobatchWiseLoadBalanceLoss(AuxLoss):
     """``sum_i f_i p_i`` over one forward's tokens (auxiliary_loss.py:30-168):
     ``f_i = E * counts_i / sum_j counts_j``, ``p_i = sum_t s_ti / sum_j s_tj``."""
@@ -127,7 +112,7 @@ class MicrobatchWiseLoadBalanceLoss(AuxLoss):
 
     def forward(self, scores_TE: torch.Tensor, routing_map_TE: torch.Tensor, *, carrier: torch.Tensor,
                 padding_mask_T: torch.Tensor | None = None) -> torch.Tensor:
-        loss = _BalanceLossFunction.apply(scores_TE, routing_map_TE, padding_mask_T)
+        loss, _f_E = ops.balance_loss_fwd(scores_TE, routing_map_TE, padding_mask_T)
         if self.token_replication_size > 1:
             loss = loss.detach() + (loss - loss.detach()) / self.token_replication_size
         return self.inject(loss, carrier=carrier)

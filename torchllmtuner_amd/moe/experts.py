@@ -7,9 +7,11 @@ stacked parameters keep their names and layouts -- ``w1_EFD`` and ``w3_EFD`` of
 shape ``(E, F, D)``, ``w2_EDF`` of shape ``(E, D, F)`` -- so a reference state
 dict loads key for key.
 
-``RoutedExperts.forward`` keeps the reference signature; ``forward_planned`` is the
-same computation for a caller that already holds the permutation plan (the MoE
-block does), and never synchronises the host with the device.
+``RoutedExperts.forward`` keeps the reference signature and chooses the device path
+itself: where the fused kernels apply (bf16, MFMA-sized widths) the row gather rides in
+the expert GEMMs' operand loads and the combine's backward in their backward; otherwise
+dispatch, experts and combine run as separate stages.  Nothing here synchronises the
+host with the device.
 """
 
 from __future__ import annotations
@@ -117,19 +119,15 @@ class GroupedExperts(nn.Module):
             torch.uint8, torch.int8, torch.int16, torch.int32, torch.int64,
         ):
             raise TypeError("Expert token counts must use an integer dtype")
-        # Counts are clamped on the device (negatives to zero, segments to the rows
-        # that exist), so malformed counts cannot make a kernel read out of bounds.
+        # Counts are clamped on the device (negatives to zero, segments to the rows that
+        # exist), so malformed counts cannot make a kernel read out of bounds; rows that the
+        # counts do not cover come back as zeros (and get zero gradients).
         plan = ops.segments_from_counts(num_tokens_per_expert_E, x_RD.shape[0])
-        return self.compute_planned(x_RD, plan)
+        return self.compute_planned(x_RD, plan, zero_fill=True)
 
-    def compute_planned(self, x_RD, plan: ops.PermutePlan):
+    def compute_planned(self, x_RD, plan: ops.PermutePlan, zero_fill: bool = False):
         w1, w3, w2 = self._weights_as(x_RD.dtype)
-        return Fn.grouped_swiglu(x_RD, w1, w3, w2, plan)
-
-    def compute_gathered(self, x_TD, plan: ops.PermutePlan):
-        """Expert outputs for every planned row, reading the tokens through the plan."""
-        w1, w3, w2 = self._weights_as(x_TD.dtype)
-        return Fn.gather_grouped_swiglu(x_TD, w1, w3, w2, plan)
+        return Fn.grouped_swiglu(x_RD, w1, w3, w2, plan, zero_fill=zero_fill)
 
 
 class RoutedExperts(nn.Module):
@@ -143,32 +141,53 @@ class RoutedExperts(nn.Module):
 
     def forward(self, x_TD, topk_scores_TK, topk_expert_ids_TK, num_local_tokens_per_expert_E):
         """Dispatch tokens to experts, run them, and combine the results."""
-        del num_local_tokens_per_expert_E  # the plan recounts on the device
-        self.token_dispatcher._check_routing(x_TD, topk_scores_TK, topk_expert_ids_TK)
-        plan = self.token_dispatcher.plan(topk_expert_ids_TK)
-        return self.forward_planned(x_TD, topk_scores_TK, plan)
-
-    def forward_planned(self, x_TD, topk_scores_TK, plan: ops.PermutePlan):
+        del num_local_tokens_per_expert_E  # the plan counts on the device
+        dispatcher = self.token_dispatcher
+        dispatcher._check_routing(x_TD, topk_scores_TK, topk_expert_ids_TK)
         experts = self.inner_experts
-        round_terms = not self.token_dispatcher.accumulate_in_fp32
-        if ops.gather_supported(x_TD, experts.hidden_dim) and x_TD.is_contiguous():
-            if ops.combine_bwd_slots(x_TD.dtype, x_TD.shape[-1], experts.hidden_dim) > 0:
-                # ... and the combine's backward inside the expert kernels' backward
-                w1, w3, w2 = experts._weights_as(x_TD.dtype)
-                out = Fn.gather_experts_combine(x_TD, topk_scores_TK, w1, w3, w2, plan, round_terms)
-                return out.to(x_TD.dtype)
-            # the dispatch gather rides inside the expert kernels' operand loads
-            y = experts.compute_gathered(x_TD, plan)
-        else:
-            with (
-                self.dispatch_observation.measure(x_TD.device)
-                if self.dispatch_observation is not None
-                else nullcontext()
-            ):
-                rows = Fn.permute_rows(x_TD, plan)
-            y = experts.compute_planned(rows, plan)
+        round_terms = not dispatcher.accumulate_in_fp32
+        observe = (
+            self.dispatch_observation.measure(x_TD.device)
+            if self.dispatch_observation is not None
+            else nullcontext()
+        )
+        fused = (
+            _is_plain_grouped_experts(experts)  # hooks on, or a subclass of, the inner module must run
+            and ops.gather_supported(x_TD, experts.hidden_dim)
+            and x_TD.is_contiguous()
+            and ops.combine_bwd_slots(x_TD.dtype, x_TD.shape[-1], experts.hidden_dim) > 0
+        )
+        if fused:
+            # the dispatch is the plan alone: the row gather rides inside the expert kernels'
+            # operand loads, and the combine's backward inside their backward
+            with observe:
+                plan = dispatcher.plan(topk_expert_ids_TK)
+            w1, w3, w2 = experts._weights_as(x_TD.dtype)
+            out = Fn.gather_experts_combine(x_TD, topk_scores_TK, w1, w3, w2, plan, round_terms)
+            return out.to(x_TD.dtype)
+        with observe:
+            plan = dispatcher.plan(topk_expert_ids_TK)
+            rows = Fn.permute_rows(x_TD, plan)
+        # rows per local expert as laid out (padding included), the counts the reference hands
+        # to its inner module; rows past the last segment are not covered and come back as zeros
+        covered = plan.seg_offsets[1:] - plan.seg_offsets[:-1]
+        y = experts(rows, covered)
         out = Fn.combine(y, topk_scores_TK, plan, round_terms)
         return out.to(x_TD.dtype)
+
+
+def _is_plain_grouped_experts(module: nn.Module) -> bool:
+    """True when calling the module is exactly GroupedExperts._compute: no subclass override
+    and no hook anywhere that a caller could be relying on."""
+    from torch.nn.modules import module as _m
+
+    cls = type(module)
+    if cls.forward is not GroupedExperts.forward or cls._compute is not GroupedExperts._compute:
+        return False
+    own = (module._forward_hooks, module._forward_pre_hooks, module._backward_hooks, module._backward_pre_hooks)
+    shared = (_m._global_forward_hooks, _m._global_forward_pre_hooks, _m._global_backward_hooks,
+              _m._global_backward_pre_hooks)
+    return not any(own) and not any(shared)
 
 
 class DenseSwiGLU(nn.Module):

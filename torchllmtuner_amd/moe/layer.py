@@ -135,19 +135,16 @@ class MoE(nn.Module):
                     f"got {tuple(padding_mask.shape)} for {tokens.shape[0]} tokens."
                 )
 
-        router = self.router
-        if router.training and router.aux_loss is not None:
-            # the aux-loss hook needs the full score map and the routing map
-            topk_scores_TK, topk_expert_ids_TK, _ = router(
-                tokens, self.expert_bias_E, padding_mask_T=padding_mask
-            )
-        else:
-            topk_scores_TK, topk_expert_ids_TK = router.route(
-                tokens, self.expert_bias_E, padding_mask_T=padding_mask
-            )
-
-        plan = self.routed_experts.token_dispatcher.plan(topk_expert_ids_TK)
-        out_TD = self.routed_experts.forward_planned(tokens, topk_scores_TK, plan)
+        topk_scores_TK, topk_expert_ids_TK, _routing_map_TE = self.router(
+            tokens, self.expert_bias_E, padding_mask_T=padding_mask
+        )
+        # The reference counts by summing the routing map (layer.py:278); the permutation plan
+        # counts the same slots on the device as a by-product, and the dispatcher hands that
+        # very plan to the experts a moment later, so neither the sum nor a second plan is run.
+        dispatcher = self.routed_experts.token_dispatcher
+        plan = dispatcher.plan(topk_expert_ids_TK)
+        num_tokens_per_expert_E = plan.counts_E
+        out_TD = self.routed_experts(tokens, topk_scores_TK, topk_expert_ids_TK, num_tokens_per_expert_E)
 
         if self.shared_experts is not None:
             out_TD = out_TD + self.shared_experts(tokens)
@@ -155,7 +152,7 @@ class MoE(nn.Module):
         if self.training and not in_checkpoint_recompute.get():
             with torch.no_grad():
                 if padding_mask is None:
-                    valid_counts_E = plan.counts_E  # int32; add_ promotes inside its one kernel
+                    valid_counts_E = num_tokens_per_expert_E  # int32; add_ promotes inside its one kernel
                 else:
                     keep = (~padding_mask).to(torch.float32).repeat_interleave(plan.top_k)
                     valid_counts_E = torch.zeros_like(self.tokens_per_expert_E).scatter_add_(

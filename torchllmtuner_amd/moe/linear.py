@@ -11,9 +11,9 @@ from __future__ import annotations
 import torch
 import torch.nn as nn
 
-from ..functional import RouterGateLinearFunction
+from .. import functional as Fn
 
-__all__ = ["RouterGateLinear", "RouterGateLinearFunction"]
+__all__ = ["RouterGateLinear"]
 
 
 class RouterGateLinear(nn.Linear):
@@ -23,5 +23,5 @@ class RouterGateLinear(nn.Linear):
     def forward(self, input: torch.Tensor) -> torch.Tensor:
         lead = input.shape[:-1]
         x = input.reshape(-1, input.shape[-1]) if input.dim() != 2 else input
-        out = RouterGateLinearFunction.apply(x, self.weight, self.bias)
+        out = Fn.router_gate(x, self.weight, self.bias)
         return out.reshape(*lead, out.shape[-1]) if input.dim() != 2 else out

@@ -4,8 +4,8 @@ Constructor surface, validation messages, return contract and hook points of
 llmtuner/models/common/moe/routing.py:31-345 (``TokenChoiceTopKRouter``).  The
 gate GEMM and the score / top-k / gather / norm / scale chain each run as one
 device kernel; ``forward`` returns ``(topk_scores_TK, topk_expert_ids_TK,
-routing_map_TE)`` like the reference, ``route`` skips the (T, E) map for callers
-that only need ids and weights.
+routing_map_TE)`` like the reference (the select kernel writes the bool map itself);
+``route`` skips the (T, E) map for callers that only need ids and weights.
 
 Selection order is "higher choice score first, ties to the lower expert id"; the
 reference's ``torch.topk(sorted=False)`` leaves both unspecified.
@@ -115,9 +115,10 @@ class TokenChoiceTopKRouter(nn.Module):
             return ops.SELECT_BALANCED
         return ops.SELECT_TOPK
 
-    def _select(self, logits_TE, expert_bias_E, want_scores, padding_mask_T=None):
+    def _select(self, logits_TE, expert_bias_E, want_scores, padding_mask_T=None, want_map=False):
+        """``(scores_TK, ids_TK, scores_TE or None, routing_map_TE or None)``."""
         # padding_mask_T is for subclasses that keep statistics (the quantile router)
-        return Fn.route_select(
+        out = Fn.route_select(
             logits_TE,
             expert_bias_E,
             self.top_k,
@@ -128,14 +129,16 @@ class TokenChoiceTopKRouter(nn.Module):
             self.num_limited_groups,
             self._mode(),
             want_scores,
+            want_map,
         )
+        return out if want_map else (*out, None)
 
     def route(self, x_TD: torch.Tensor, expert_bias_E: torch.Tensor | None = None, *,
               padding_mask_T: torch.Tensor | None = None):
         """Scores and ids only: ``(topk_scores_TK fp32, topk_expert_ids_TK int64)``.
         ``padding_mask_T`` only matters to routers that keep statistics."""
         logits_TE = self.gate(x_TD)
-        scores_TK, ids_TK, _ = self._select(logits_TE, expert_bias_E, False)
+        scores_TK, ids_TK, _, _ = self._select(logits_TE, expert_bias_E, False)
         return scores_TK, ids_TK
 
     def forward(
@@ -156,14 +159,14 @@ class TokenChoiceTopKRouter(nn.Module):
                 )
         logits_TE = self.gate(x_TD)
         want_scores = self.training and self.aux_loss is not None
-        topk_scores_TK, topk_expert_ids_TK, scores_TE = self._select(
-            logits_TE, expert_bias_E, want_scores, padding_mask_T
+        topk_scores_TK, topk_expert_ids_TK, scores_TE, routing_map_TE = self._select(
+            logits_TE, expert_bias_E, want_scores, padding_mask_T, want_map=True
         )
-        # One-hot map of each token's chosen experts; (T, E) bool is index glue, not
-        # arithmetic, and is built with a scatter like the reference's.
-        routing_map_TE = torch.zeros(
-            x_TD.shape[0], self.num_experts, dtype=torch.bool, device=x_TD.device
-        ).scatter_(-1, topk_expert_ids_TK, True)
+        if routing_map_TE is None:
+            # a selection path without the map output: the reference's scatter (index glue)
+            routing_map_TE = torch.zeros(
+                x_TD.shape[0], self.num_experts, dtype=torch.bool, device=x_TD.device
+            ).scatter_(-1, topk_expert_ids_TK, True)
 
         if want_scores:
             masked_map = (
@@ -268,7 +271,7 @@ class QuantileBalancedTopKRouter(TokenChoiceTopKRouter):
         self.quantile_balancer.observe(
             scores_TE.detach(), cutoff_T, expert_bias_E, padding_mask_T=padding_mask_T
         )
-        return scores_TK, ids_TK, scores_TE
+        return scores_TK, ids_TK, scores_TE, None
 
     def forward(self, x_TD, expert_bias_E=None, *, padding_mask_T=None):
         self._require_bias(expert_bias_E)
@@ -280,11 +283,11 @@ class QuantileBalancedTopKRouter(TokenChoiceTopKRouter):
             return super().route(x_TD, expert_bias_E)
         if padding_mask_T is not None:
             padding_mask_T = padding_mask_T.reshape(-1)
-        scores_TK, ids_TK, _ = self._select_observing(self.gate(x_TD), expert_bias_E, padding_mask_T)
+        scores_TK, ids_TK, _, _ = self._select_observing(self.gate(x_TD), expert_bias_E, padding_mask_T)
         return scores_TK, ids_TK
 
-    def _select(self, logits_TE, expert_bias_E, want_scores, padding_mask_T=None):
+    def _select(self, logits_TE, expert_bias_E, want_scores, padding_mask_T=None, want_map=False):
         self._require_bias(expert_bias_E)
         if not self.training:
-            return super()._select(logits_TE, expert_bias_E, want_scores)
+            return super()._select(logits_TE, expert_bias_E, want_scores, want_map=want_map)
         return self._select_observing(logits_TE, expert_bias_E, padding_mask_T)

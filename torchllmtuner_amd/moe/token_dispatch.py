@@ -22,7 +22,7 @@ The rows are ordered exactly like ``argsort(ids.flatten(), stable=True)``.
 
 from __future__ import annotations
 
-from dataclasses import dataclass
+import weakref
 
 import torch
 
@@ -37,25 +37,51 @@ __all__ = [
 ]
 
 
-@dataclass(frozen=True, kw_only=True)
 class LocalDispatchMetadata:
-    """What ``dispatch()`` hands to ``combine()``: the plan and the (T, K) scores."""
+    """What ``dispatch()`` hands to ``combine()``.
 
-    plan: ops.PermutePlan
-    topk_scores_TK: torch.Tensor
+    The reference's record has two fields (token_dispatch.py:84-89):
+    ``token_indices_experts_sorted_N`` (token of each expert-sorted row) and
+    ``topk_scores_experts_sorted_N`` (score of each row); both are accepted as keywords and
+    readable here.  Records made by this package's dispatchers also carry the permutation
+    ``plan`` and the unsorted ``(T, K)`` scores, which is what the device kernels consume;
+    the two reference fields are then derived from the plan on first access (-1 / 0 for
+    padding rows).
+    """
+
+    __slots__ = ("plan", "topk_scores_TK", "_token_indices", "_scores_sorted")
+
+    def __init__(self, *, token_indices_experts_sorted_N: torch.Tensor | None = None,
+                 topk_scores_experts_sorted_N: torch.Tensor | None = None,
+                 plan: ops.PermutePlan | None = None, topk_scores_TK: torch.Tensor | None = None) -> None:
+        if plan is None and (token_indices_experts_sorted_N is None or topk_scores_experts_sorted_N is None):
+            raise TypeError(
+                "LocalDispatchMetadata needs token_indices_experts_sorted_N and "
+                "topk_scores_experts_sorted_N (or a plan with the (T, K) scores)"
+            )
+        if plan is not None and topk_scores_TK is None:
+            raise TypeError("LocalDispatchMetadata: a plan needs the (T, K) scores it was made for")
+        self.plan = plan
+        self.topk_scores_TK = topk_scores_TK
+        self._token_indices = token_indices_experts_sorted_N
+        self._scores_sorted = topk_scores_experts_sorted_N
 
     @property
     def token_indices_experts_sorted_N(self) -> torch.Tensor:  # noqa: N802
-        """Token of each row, int64 (-1 for padding rows); the reference's field."""
-        slot = self.plan.slot_of_row.to(torch.int64)
-        return torch.where(slot >= 0, slot // self.plan.top_k, slot)
+        """Token of each row, int64 (-1 for padding rows)."""
+        if self._token_indices is None:
+            slot = self.plan.slot_of_row.to(torch.int64)
+            self._token_indices = torch.where(slot >= 0, slot // self.plan.top_k, slot)
+        return self._token_indices
 
     @property
     def topk_scores_experts_sorted_N(self) -> torch.Tensor:  # noqa: N802
-        """Score of each row (0 for padding rows); the reference's field."""
-        slot = self.plan.slot_of_row.to(torch.int64)
-        flat = self.topk_scores_TK.reshape(-1)
-        return torch.where(slot >= 0, flat[slot.clamp_min(0)], flat.new_zeros(()))
+        """Score of each row (0 for padding rows)."""
+        if self._scores_sorted is None:
+            slot = self.plan.slot_of_row.to(torch.int64)
+            flat = self.topk_scores_TK.reshape(-1)
+            self._scores_sorted = torch.where(slot >= 0, flat[slot.clamp_min(0)], flat.new_zeros(()))
+        return self._scores_sorted
 
 
 class LocalTokenDispatcher:
@@ -65,6 +91,7 @@ class LocalTokenDispatcher:
         self.num_experts = num_experts
         self.top_k = top_k
         self.accumulate_in_fp32 = False
+        self._last_plan = None  # (weakref to the ids tensor, its version, the plan made for it)
 
     def set_ep_group(self, *, ep_group=None) -> None:
         """No-op: there is no expert-parallel group on one GPU."""
@@ -88,8 +115,41 @@ class LocalTokenDispatcher:
             )
 
     def plan(self, topk_expert_ids_TK: torch.Tensor) -> ops.PermutePlan:
+        """The expert-major layout for these ids.  The plan of the most recent call is kept
+        and returned again for the very same tensor object (unchanged since): the block asks
+        for the counts first and the experts for the layout right after."""
+        ids = topk_expert_ids_TK
+        last = self._last_plan
+        if last is not None and last[0]() is ids and last[1] == ids._version:
+            return last[2]
         lo, hi = self._local_range()
-        return ops.permute_plan(topk_expert_ids_TK, self.num_experts, lo, hi, self._align())
+        plan = ops.permute_plan(ids, self.num_experts, lo, hi, self._align())
+        try:
+            self._last_plan = (weakref.ref(ids), ids._version, plan)
+        except TypeError:  # tensor subclasses without weak references: no memo
+            self._last_plan = None
+        return plan
+
+    def _rows_for_combine(self, routed_output_RD, metadata: "LocalDispatchMetadata"):
+        """(plan, scores_TK) for a record that only carries the reference's two fields: with
+        K rows per token the stable order of the token indices IS the slot -> row map."""
+        tok = metadata.token_indices_experts_sorted_N
+        K = self.top_k
+        if tok.numel() % K != 0:
+            raise ValueError("combine: the dispatch record does not hold top_k rows per token")
+        T = tok.numel() // K
+        order = torch.argsort(tok, stable=True)
+        if T > 0 and not bool((tok[order].view(T, K) == torch.arange(T, device=tok.device)[:, None]).all()):
+            raise ValueError("combine: the dispatch record does not hold top_k rows per token")
+        row_of_slot = order.to(torch.int32)
+        inv = torch.empty_like(row_of_slot)
+        inv[order] = torch.arange(tok.numel(), device=tok.device, dtype=torch.int32)
+        counts = torch.tensor([tok.numel()], dtype=torch.int32, device=tok.device)
+        seg = ops.segments_from_counts(counts, tok.numel())
+        plan = ops.PermutePlan(T, K, 1, 0, 1, 1, seg.tile_m, tok.numel(), seg.tile_capacity, None, seg.seg_offsets,
+                               seg.seg_counts, row_of_slot, inv, None, seg.tile_expert, seg.tile_row0,
+                               seg.num_tiles, seg.expert_order)
+        return plan, metadata.topk_scores_experts_sorted_N[order].view(T, K)
 
     def dispatch(self, x_TD, topk_scores_TK, topk_expert_ids_TK, num_local_tokens_per_expert_E):
         self._check_routing(x_TD, topk_scores_TK, topk_expert_ids_TK)
@@ -99,9 +159,11 @@ class LocalTokenDispatcher:
         return rows, num_local_tokens_per_expert_E, metadata
 
     def combine(self, routed_output_RD, metadata: LocalDispatchMetadata, x_TD):
-        out = Fn.combine(
-            routed_output_RD, metadata.topk_scores_TK, metadata.plan, not self.accumulate_in_fp32
-        )
+        if metadata.plan is not None:
+            plan, scores_TK = metadata.plan, metadata.topk_scores_TK
+        else:
+            plan, scores_TK = self._rows_for_combine(routed_output_RD, metadata)
+        out = Fn.combine(routed_output_RD, scores_TK, plan, not self.accumulate_in_fp32)
         return out.to(x_TD.dtype)
 
 

@@ -1,22 +1,33 @@
-"""Tensor-level wrappers over the C ABI: allocate outputs, pass pointers, check codes.
+"""Tensor-level entry points of the MoE kernels: the ``mi355_moe`` torch.library operators.
 
-PyTorch is used here for device memory and the current stream only.  Every function
-requires device tensors and raises if given CPU tensors -- the kernels are the only
-implementation.
+``libmi355moe_torch.so`` registers one operator per stage (``torch.ops.mi355_moe.*``): a
+thin C++ layer that allocates outputs with PyTorch's allocator and calls the C ABI of
+``include/mi355_moe.h`` on the current HIP stream.  This module adds what the dispatcher
+needs around them -- shape propagation for fake / meta tensors (so the operators trace
+under ``torch.compile``) and the autograd formulas, whose backward passes are again
+operators of the same library -- plus Python wrappers that validate arguments the way the
+reference's modules do and carry the permutation plan as one object.
+
+Every function requires device tensors and raises if given CPU tensors: the kernels are the
+only implementation.  The profiling hooks at the end (one MFMA kernel per call on
+pre-allocated buffers) go straight to the C ABI through ``ctypes``.
 """
 
 from __future__ import annotations
 
-import os
 from dataclasses import dataclass
 
 import torch
 
 from . import _lib
 
+_lib.load_torch_ops()  # fails loudly when the library is not built
+_O = torch.ops.mi355_moe
+
 _DT = {torch.float32: 0, torch.bfloat16: 1}
 SCORE_FUNCS = {"sigmoid": 0, "softmax": 1, "sqrtsoftplus": 2}
 SELECT_TOPK, SELECT_FIXED, SELECT_BALANCED = 0, 1, 2
+TILE_M = 256  # rows per entry of a plan's tile list (mi355_grouped_tile_m)
 
 
 def _dt(t: torch.Tensor) -> int:
@@ -51,234 +62,472 @@ def _stream(dev: torch.device):
     return torch.cuda.current_stream(dev).cuda_stream
 
 
-def _c(t: torch.Tensor) -> torch.Tensor:
-    return t if t.is_contiguous() else t.contiguous()
-
-
 def tile_m(dtype: torch.dtype = torch.bfloat16) -> int:
-    return int(_lib.load().mi355_grouped_tile_m(_DT[dtype]))
+    return TILE_M
 
 
-# ------------------------------------------------------------------ router
-def router_gate_fwd(x_TD, w_ED, logit_bias_E=None):
-    dev = _dev(x_TD, w_ED, logit_bias_E)
-    x_TD, w_ED = _c(x_TD), _c(w_ED)
-    T, D = x_TD.shape
-    E = w_ED.shape[0]
-    if w_ED.shape[1] != D:
-        raise ValueError(f"gate weight {tuple(w_ED.shape)} does not match input dim {D}")
-    bias = None if logit_bias_E is None else _c(logit_bias_E.float())
-    out = torch.empty(T, E, dtype=torch.float32, device=dev)
-    lib = _lib.load()
-    nbytes = lib.mi355_router_gate_fwd_workspace_bytes(T, D, E)
-    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev) if nbytes else None
-    with torch.cuda.device(dev):
-        rc = lib.mi355_router_gate_fwd(
-            _p(x_TD), _dt(x_TD), _p(w_ED), _dt(w_ED), _p(bias), _p(out), _p(ws), T, D, E, _stream(dev)
+def _opt(t: torch.Tensor, wanted: bool):
+    """Operators return an empty (0,) tensor for an output that was not asked for."""
+    return t if wanted else None
+
+
+# ====================================================================== fake kernels
+# Shape / dtype propagation for tracing.  Skipped outputs are empty (0,) tensors.
+def _fake(name):
+    return torch.library.register_fake(f"mi355_moe::{name}")
+
+
+def _e0(like, dtype=None):
+    return like.new_empty((0,), dtype=dtype or like.dtype)
+
+
+@_fake("router_gate_fwd")
+def _(x, w, logit_bias):
+    return x.new_empty((x.shape[0], w.shape[0]), dtype=torch.float32)
+
+
+@_fake("router_gate_bwd")
+def _(dlogits, x, w, need_dx, need_dw):
+    return (torch.empty_like(x) if need_dx else _e0(x)), (torch.empty_like(w) if need_dw else _e0(w))
+
+
+@_fake("router_select_fwd")
+def _(logits, expert_bias, top_k, score_func, route_norm, route_scale, num_groups, num_limited, mode,
+      want_scores, want_map):
+    T, E = logits.shape
+    return (logits.new_empty((T, top_k)), logits.new_empty((T, top_k), dtype=torch.int64),
+            logits.new_empty((T, E)) if want_scores else _e0(logits),
+            logits.new_empty((T, E) if want_map else (0, 0), dtype=torch.bool))
+
+
+@_fake("router_select_cutoff_fwd")
+def _(logits, expert_bias, top_k, score_func, route_norm, route_scale):
+    T, E = logits.shape
+    return (logits.new_empty((T, top_k)), logits.new_empty((T, top_k), dtype=torch.int64),
+            logits.new_empty((T, E)), logits.new_empty((T,)))
+
+
+@_fake("router_select_bwd")
+def _(logits, ids, dweights, dscores, score_func, route_norm, route_scale, mode):
+    return torch.empty_like(logits)
+
+
+@_fake("quantile_observe")
+def _(histogram, scores, cutoff, expert_bias, padding_mask):
+    return None
+
+
+@_fake("quantile_estimate")
+def _(histogram, expert_bias, top_k):
+    return expert_bias.new_empty((histogram.shape[0],), dtype=torch.float32)
+
+
+@_fake("rms_norm_fwd")
+def _(x, weight, epsilon):
+    rows = x.numel() // max(weight.numel(), 1)
+    return torch.empty_like(x), x.new_empty((rows,), dtype=torch.float32)
+
+
+@_fake("rms_norm_bwd")
+def _(dy, x, weight, rstd, need_dx, need_dw):
+    return (torch.empty_like(x) if need_dx else _e0(x)), (torch.empty_like(weight) if need_dw else _e0(weight))
+
+
+@_fake("balance_loss_fwd")
+def _(scores, routing_map, padding_mask):
+    return scores.new_empty((1 + scores.shape[1],))
+
+
+@_fake("balance_loss_bwd")
+def _(scores, f, padding_mask, grad_loss):
+    return torch.empty_like(scores)
+
+
+def _plan_sizes(N, El, align):
+    row_cap = N + (El * (align - 1) if align > 1 else 0)
+    tile_cap = N // TILE_M + El + 1
+    return row_cap, tile_cap
+
+
+@_fake("permute_plan")
+def _(ids, num_experts, local_lo, local_hi, align):
+    T, K = ids.shape
+    El = local_hi - local_lo
+    row_cap, tile_cap = _plan_sizes(T * K, El, align)
+    i32 = dict(dtype=torch.int32)
+    return (ids.new_empty((num_experts + (El + 1) + 2 * El + 2 * tile_cap + 1,), **i32),
+            ids.new_empty((T * K,), **i32), ids.new_empty((2, row_cap), **i32))
+
+
+@_fake("segments_from_counts")
+def _(counts, total_rows):
+    El = counts.shape[0]
+    tile_cap = total_rows // TILE_M + El + 1
+    return counts.new_empty(((El + 1) + 2 * El + 2 * tile_cap + 1,), dtype=torch.int32)
+
+
+@_fake("permute_rows_fwd")
+def _(x, row_of_slot, slot_of_row, total_rows, top_k, row_capacity):
+    return x.new_empty((row_capacity, x.shape[1]))
+
+
+@_fake("permute_rows_bwd")
+def _(drows, row_of_slot, num_tokens, top_k):
+    return drows.new_empty((num_tokens, drows.shape[1]))
+
+
+@_fake("combine_fwd")
+def _(y, weights, row_of_slot, slot_of_row, total_rows, num_tokens, top_k, round_terms):
+    return y.new_empty((num_tokens, y.shape[1]))
+
+
+@_fake("combine_bwd")
+def _(dout, y, weights, row_of_slot, slot_of_row, total_rows, top_k):
+    return torch.empty_like(y), y.new_empty((dout.shape[0], top_k), dtype=torch.float32)
+
+
+@_fake("combine_row_scale")
+def _(weights, slot_of_row, row_capacity):
+    return weights.new_empty((row_capacity,), dtype=torch.float32)
+
+
+@_fake("combine_scores_bwd")
+def _(dot_partial, row_of_slot, num_tokens, top_k):
+    return dot_partial.new_empty((num_tokens, top_k))
+
+
+@_fake("grouped_swiglu_fwd")
+def _(rows, token_of_row, w1, w3, w2, seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles,
+      row_capacity, zero_fill):
+    F, D = w1.shape[1], rows.shape[1]
+    mk = lambda n: rows.new_empty((row_capacity, n))
+    return mk(D), mk(F), mk(F), mk(F)
+
+
+@_fake("grouped_swiglu_bwd")
+def _(dy, rows, token_of_row, w1, w3, w2, gate, up, h, seg_offsets, seg_counts, tile_expert, tile_row0,
+      num_tiles, need_drows, need_dw, zero_fill):
+    drows = rows.new_empty((dy.shape[0], rows.shape[1])) if need_drows else _e0(rows)
+    g = lambda w: torch.empty_like(w) if need_dw else _e0(w)
+    return drows, g(w1), g(w3), g(w2)
+
+
+@_fake("gather_experts_combine_fwd")
+def _(x, weights, w1, w3, w2, token_of_row, slot_of_row, row_of_slot, seg_offsets, seg_counts, tile_expert,
+      tile_row0, num_tiles, top_k, row_capacity, round_terms):
+    F = w1.shape[1]
+    return torch.empty_like(x), x.new_empty((row_capacity, F)), x.new_empty((row_capacity, F))
+
+
+@_fake("gather_experts_combine_bwd")
+def _(dout, x, weights, w1, w3, w2, gate, up, token_of_row, slot_of_row, row_of_slot, seg_offsets, seg_counts,
+      tile_expert, tile_row0, num_tiles, top_k, need_dx, need_dw):
+    g = lambda w: torch.empty_like(w) if need_dw else _e0(w)
+    return ((torch.empty_like(x) if need_dx else _e0(x)), g(w1), g(w3), g(w2),
+            x.new_empty((x.shape[0], top_k), dtype=torch.float32))
+
+
+# ====================================================================== autograd formulas
+# Each differentiable operator's backward is the hand-written kernel for that stage.
+def _autograd(name, backward, setup):
+    torch.library.register_autograd(f"mi355_moe::{name}", backward, setup_context=setup)
+
+
+# -- router gate: dX in the input dtype, dW in the weight dtype (linear.py:133-151)
+def _rg_setup(ctx, inputs, output):
+    x, w, bias = inputs
+    ctx.save_for_backward(x, w)
+    ctx.bias_dtype = None if bias is None else bias.dtype
+
+
+def _rg_backward(ctx, grad_TE):
+    x, w = ctx.saved_tensors
+    need = ctx.needs_input_grad
+    dx = dw = None
+    if need[0] or need[1]:
+        dx, dw = _O.router_gate_bwd(grad_TE, x, w, need[0], need[1])
+    db = grad_TE.float().sum(dim=0).to(ctx.bias_dtype) if (ctx.bias_dtype is not None and need[2]) else None
+    return (dx if need[0] else None), (dw if need[1] else None), db
+
+
+_autograd("router_gate_fwd", _rg_backward, _rg_setup)
+
+
+# -- select: gather / norm / scale / score VJP per token; ids and the map are not differentiable
+def _rs_setup(ctx, inputs, output):
+    logits, _bias, _k, score_func, route_norm, route_scale, _g, _l, mode, want_scores, _m = inputs
+    ctx.save_for_backward(logits, output[1])
+    ctx.cfg = (score_func, route_norm, route_scale, mode, want_scores)
+    ctx.set_materialize_grads(False)
+
+
+def _rs_backward(ctx, dweights, _dids, dscores, _dmap):
+    logits, ids = ctx.saved_tensors
+    score_func, route_norm, route_scale, mode, want_scores = ctx.cfg
+    dlogits = None
+    if ctx.needs_input_grad[0]:
+        dlogits = _O.router_select_bwd(logits, ids, dweights, dscores if want_scores else None, score_func,
+                                       route_norm, route_scale, mode)
+    return (dlogits,) + (None,) * 10
+
+
+_autograd("router_select_fwd", _rs_backward, _rs_setup)
+
+
+def _rsc_setup(ctx, inputs, output):
+    logits, _bias, _k, score_func, route_norm, route_scale = inputs
+    ctx.save_for_backward(logits, output[1])
+    ctx.cfg = (score_func, route_norm, route_scale)
+    ctx.set_materialize_grads(False)  # no dense zero gradient for an unused score map
+
+
+def _rsc_backward(ctx, dweights, _dids, dscores, _dcutoff):
+    logits, ids = ctx.saved_tensors
+    score_func, route_norm, route_scale = ctx.cfg
+    dlogits = None
+    if ctx.needs_input_grad[0]:
+        dlogits = _O.router_select_bwd(logits, ids, dweights, dscores, score_func, route_norm, route_scale,
+                                       SELECT_TOPK)
+    return (dlogits,) + (None,) * 5
+
+
+_autograd("router_select_cutoff_fwd", _rsc_backward, _rsc_setup)
+
+
+def _rms_setup(ctx, inputs, output):
+    x, weight, _eps = inputs
+    ctx.save_for_backward(x, weight, output[1])
+    ctx.set_materialize_grads(False)
+
+
+def _rms_backward(ctx, dy, _drstd):
+    x, weight, rstd = ctx.saved_tensors
+    need = ctx.needs_input_grad
+    if dy is None or not (need[0] or need[1]):
+        return None, None, None
+    dx, dw = _O.rms_norm_bwd(dy, x, weight, rstd, need[0], need[1])
+    return (dx if need[0] else None), (dw if need[1] else None), None
+
+
+_autograd("rms_norm_fwd", _rms_backward, _rms_setup)
+
+
+def _bl_setup(ctx, inputs, output):
+    scores, _map, pad = inputs
+    ctx.save_for_backward(scores, output, pad)
+
+
+def _bl_backward(ctx, grad):
+    scores, out, pad = ctx.saved_tensors
+    ds = _O.balance_loss_bwd(scores, out[1:], pad, grad[0:1]) if ctx.needs_input_grad[0] else None
+    return ds, None, None
+
+
+_autograd("balance_loss_fwd", _bl_backward, _bl_setup)
+
+
+# -- row gather: backward sums the K row gradients of every token
+def _pr_setup(ctx, inputs, output):
+    x, row_of_slot, _sor, _total, top_k, _cap = inputs
+    ctx.save_for_backward(row_of_slot)
+    ctx.shape = (x.shape[0], top_k)
+
+
+def _pr_backward(ctx, drows):
+    (row_of_slot,) = ctx.saved_tensors
+    dx = _O.permute_rows_bwd(drows, row_of_slot, ctx.shape[0], ctx.shape[1]) if ctx.needs_input_grad[0] else None
+    return dx, None, None, None, None, None
+
+
+_autograd("permute_rows_fwd", _pr_backward, _pr_setup)
+
+
+# -- combine: dY = weights * dout per row, dWeights = <y row, dout row>
+def _cb_setup(ctx, inputs, output):
+    y, weights, row_of_slot, slot_of_row, total_rows, _T, top_k, _round = inputs
+    ctx.save_for_backward(y, weights, row_of_slot, slot_of_row, total_rows)
+    ctx.top_k = top_k
+
+
+def _cb_backward(ctx, dout):
+    y, weights, row_of_slot, slot_of_row, total_rows = ctx.saved_tensors
+    dy, dw = _O.combine_bwd(dout, y, weights, row_of_slot, slot_of_row, total_rows, ctx.top_k)
+    need = ctx.needs_input_grad
+    return ((dy if need[0] else None), (dw.to(weights.dtype) if need[1] else None)) + (None,) * 6
+
+
+_autograd("combine_fwd", _cb_backward, _cb_setup)
+
+
+# -- grouped experts
+def _gs_setup(ctx, inputs, output):
+    rows, tok, w1, w3, w2, so, sc, te, tr, nt, _cap, zero_fill = inputs
+    _y, gate, up, h = output
+    ctx.gathered = tok is not None
+    ctx.save_for_backward(rows, w1, w3, w2, gate, up, h, so, sc, te, tr, nt)
+    ctx.zero_fill = zero_fill
+    ctx.set_materialize_grads(False)
+
+
+def _gs_backward(ctx, dy, _dgate, _dup, _dh):
+    if ctx.gathered:
+        raise NotImplementedError(
+            "grouped_swiglu_fwd with a token gather is differentiated through gather_experts_combine_fwd"
         )
-    _lib.check(rc, "router_gate_fwd")
-    return out
+    rows, w1, w3, w2, gate, up, h, so, sc, te, tr, nt = ctx.saved_tensors
+    need = ctx.needs_input_grad
+    if dy is None:
+        return (None,) * 12
+    need_dw = need[2] or need[3] or need[4]
+    drows, dw1, dw3, dw2 = _O.grouped_swiglu_bwd(dy, rows, None, w1, w3, w2, gate, up, h, so, sc, te, tr, nt,
+                                                 need[0], need_dw, ctx.zero_fill)
+    return ((drows if need[0] else None), None, (dw1 if need[2] else None), (dw3 if need[3] else None),
+            (dw2 if need[4] else None)) + (None,) * 7
+
+
+_autograd("grouped_swiglu_fwd", _gs_backward, _gs_setup)
+
+
+# -- gathered experts + combine: one backward for both halves
+def _gec_setup(ctx, inputs, output):
+    x, weights, w1, w3, w2, tok, sor, ros, so, sc, te, tr, nt, top_k, _cap, _round = inputs
+    _out, gate, up = output
+    ctx.save_for_backward(x, weights, w1, w3, w2, gate, up, tok, sor, ros, so, sc, te, tr, nt)
+    ctx.top_k = top_k
+    ctx.set_materialize_grads(False)
+
+
+def _gec_backward(ctx, dout, _dgate, _dup):
+    x, weights, w1, w3, w2, gate, up, tok, sor, ros, so, sc, te, tr, nt = ctx.saved_tensors
+    need = ctx.needs_input_grad
+    if dout is None:
+        return (None,) * 16
+    need_dw = need[2] or need[3] or need[4]
+    dx, dw1, dw3, dw2, dweights = _O.gather_experts_combine_bwd(
+        dout, x, weights, w1, w3, w2, gate, up, tok, sor, ros, so, sc, te, tr, nt, ctx.top_k, need[0], need_dw)
+    return ((dx if need[0] else None), (dweights.to(weights.dtype) if need[1] else None),
+            (dw1 if need[2] else None), (dw3 if need[3] else None), (dw2 if need[4] else None)) + (None,) * 11
+
+
+_autograd("gather_experts_combine_fwd", _gec_backward, _gec_setup)
+
+
+# ====================================================================== router
+def router_gate_fwd(x_TD, w_ED, logit_bias_E=None):
+    """fp32 logits (differentiable: dX in the input dtype, dW in the weight dtype)."""
+    _dev(x_TD, w_ED, logit_bias_E)
+    if w_ED.shape[1] != x_TD.shape[1]:
+        raise ValueError(f"gate weight {tuple(w_ED.shape)} does not match input dim {x_TD.shape[1]}")
+    _dt(x_TD), _dt(w_ED)
+    return _O.router_gate_fwd(x_TD, w_ED, logit_bias_E)
 
 
 def router_gate_bwd(dlogits_TE, x_TD, w_ED, need_dx=True, need_dw=True):
-    dev = _dev(dlogits_TE, x_TD, w_ED)
-    dlogits_TE, x_TD, w_ED = _c(dlogits_TE.float()), _c(x_TD), _c(w_ED)
-    T, D = x_TD.shape
-    E = w_ED.shape[0]
-    lib = _lib.load()
-    dx = torch.empty_like(x_TD) if need_dx else None
-    dw = torch.empty_like(w_ED) if need_dw else None
-    nbytes = lib.mi355_router_gate_bwd_workspace_bytes(T, D, E)
-    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev) if nbytes else None
-    with torch.cuda.device(dev):
-        rc = lib.mi355_router_gate_bwd(
-            _p(dlogits_TE), _p(x_TD), _dt(x_TD), _p(w_ED), _dt(w_ED), _p(dx), _p(dw), _p(ws),
-            T, D, E, _stream(dev),
-        )
-    _lib.check(rc, "router_gate_bwd")
-    return dx, dw
+    _dev(dlogits_TE, x_TD, w_ED)
+    dx, dw = _O.router_gate_bwd(dlogits_TE, x_TD, w_ED, bool(need_dx), bool(need_dw))
+    return _opt(dx, need_dx), _opt(dw, need_dw)
 
 
 def router_select_fwd(logits_TE, expert_bias_E, top_k, score_func, route_norm, route_scale,
-                      num_groups=0, num_limited=0, mode=SELECT_TOPK, want_scores=False):
-    dev = _dev(logits_TE, expert_bias_E)
+                      num_groups=0, num_limited=0, mode=SELECT_TOPK, want_scores=False, want_map=False):
+    """Returns ``(weights_TK, ids_TK, scores_TE or None)`` -- and the bool routing map as a
+    fourth item when ``want_map`` is set.  Differentiable in the logits through the weights
+    and (when materialised) the dense scores."""
+    _dev(logits_TE, expert_bias_E)
     if logits_TE.dtype != torch.float32:
         raise TypeError("router logits must be float32")
-    logits_TE = _c(logits_TE)
-    T, E = logits_TE.shape
-    bias = None if expert_bias_E is None else _c(expert_bias_E.float())
-    weights = torch.empty(T, top_k, dtype=torch.float32, device=dev)
-    ids = torch.empty(T, top_k, dtype=torch.int64, device=dev)
-    scores = torch.empty(T, E, dtype=torch.float32, device=dev) if want_scores else None
-    with torch.cuda.device(dev):
-        rc = _lib.load().mi355_router_select_fwd(
-            _p(logits_TE), _p(bias), _p(weights), _p(ids), _p(scores), T, E, top_k,
-            SCORE_FUNCS[score_func], int(route_norm), float(route_scale), int(num_groups or 0),
-            int(num_limited or 0), mode, _stream(dev),
-        )
-    _lib.check(rc, "router_select_fwd")
-    return weights, ids, scores
+    weights, ids, scores, rmap = _O.router_select_fwd(
+        logits_TE, expert_bias_E, int(top_k), SCORE_FUNCS[score_func], bool(route_norm), float(route_scale),
+        int(num_groups or 0), int(num_limited or 0), int(mode), bool(want_scores), bool(want_map))
+    scores = scores if want_scores else None
+    return (weights, ids, scores, rmap) if want_map else (weights, ids, scores)
 
 
 def router_select_cutoff_fwd(logits_TE, expert_bias_E, top_k, score_func, route_norm, route_scale):
     """Biased top-k plus the (K+1)-th biased score of every token: returns
     ``(weights_TK, ids_TK, scores_TE, cutoff_T)``."""
-    dev = _dev(logits_TE, expert_bias_E)
+    _dev(logits_TE, expert_bias_E)
     if logits_TE.dtype != torch.float32:
         raise TypeError("router logits must be float32")
-    logits_TE = _c(logits_TE)
-    T, E = logits_TE.shape
-    bias = None if expert_bias_E is None else _c(expert_bias_E.float())
-    weights = torch.empty(T, top_k, dtype=torch.float32, device=dev)
-    ids = torch.empty(T, top_k, dtype=torch.int64, device=dev)
-    scores = torch.empty(T, E, dtype=torch.float32, device=dev)
-    cutoff = torch.empty(T, dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
-        rc = _lib.load().mi355_router_select_cutoff_fwd(
-            _p(logits_TE), _p(bias), _p(weights), _p(ids), _p(scores), _p(cutoff), T, E, top_k,
-            SCORE_FUNCS[score_func], int(route_norm), float(route_scale), _stream(dev),
-        )
-    _lib.check(rc, "router_select_cutoff_fwd")
-    return weights, ids, scores, cutoff
+    return _O.router_select_cutoff_fwd(logits_TE, expert_bias_E, int(top_k), SCORE_FUNCS[score_func],
+                                       bool(route_norm), float(route_scale))
+
+
+def router_select_bwd(logits_TE, ids_TK, dweights_TK, dscores_TE, score_func, route_norm,
+                      route_scale, mode=SELECT_TOPK):
+    _dev(logits_TE, ids_TK, dweights_TK, dscores_TE)
+    return _O.router_select_bwd(logits_TE, ids_TK, dweights_TK, dscores_TE, SCORE_FUNCS[score_func],
+                                bool(route_norm), float(route_scale), int(mode))
 
 
 def quantile_observe(histogram_EB, scores_TE, cutoff_T, expert_bias_E, padding_mask_T=None):
     """Accumulates the required-bias histogram in place (int64 ``(E, B)``)."""
-    dev = _dev(histogram_EB, scores_TE, cutoff_T, expert_bias_E, padding_mask_T)
+    _dev(histogram_EB, scores_TE, cutoff_T, expert_bias_E, padding_mask_T)
     if histogram_EB.dtype != torch.int64 or not histogram_EB.is_contiguous():
         raise TypeError("histogram_EB must be a contiguous int64 tensor")
-    scores_TE = _c(scores_TE.float())
     T, E = scores_TE.shape
     if histogram_EB.shape[0] != E or cutoff_T.numel() != T or expert_bias_E.numel() != E:
         raise ValueError(
             f"quantile_observe: histogram {tuple(histogram_EB.shape)}, scores {(T, E)}, "
             f"cutoff {tuple(cutoff_T.shape)} and bias {tuple(expert_bias_E.shape)} do not agree"
         )
-    cutoff_T = _c(cutoff_T.float().reshape(-1))
-    bias = _c(expert_bias_E.float())
     pad = None
     if padding_mask_T is not None:
         if padding_mask_T.dtype != torch.bool or padding_mask_T.numel() != T:
             raise ValueError("padding_mask_T must be a bool tensor with one entry per token")
-        pad = _c(padding_mask_T.reshape(-1)).view(torch.uint8)
-    with torch.cuda.device(dev):
-        rc = _lib.load().mi355_quantile_observe(
-            _p(scores_TE), _p(cutoff_T), _p(bias), _p(pad), _p(histogram_EB), T, E,
-            histogram_EB.shape[1], _stream(dev),
-        )
-    _lib.check(rc, "quantile_observe")
+        pad = padding_mask_T.reshape(-1)
+    _O.quantile_observe(histogram_EB, scores_TE, cutoff_T, expert_bias_E, pad)
 
 
 def quantile_estimate(histogram_EB, expert_bias_E, top_k):
     """The next mean-centred expert bias (new tensor, dtype of ``expert_bias_E``)."""
-    dev = _dev(histogram_EB, expert_bias_E)
+    _dev(histogram_EB, expert_bias_E)
     if histogram_EB.dtype != torch.int64:
         raise TypeError("histogram_EB must be int64")
-    histogram_EB = _c(histogram_EB)
-    E, B = histogram_EB.shape
-    bias = _c(expert_bias_E.float())
-    out = torch.empty(E, dtype=torch.float32, device=dev)
-    ws = torch.empty(2 * E, dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
-        rc = _lib.load().mi355_quantile_estimate(
-            _p(histogram_EB), _p(bias), _p(out), _p(ws), E, top_k, B, _stream(dev)
-        )
-    _lib.check(rc, "quantile_estimate")
-    return out.to(expert_bias_E.dtype)
+    return _O.quantile_estimate(histogram_EB, expert_bias_E, int(top_k)).to(expert_bias_E.dtype)
 
 
 def rms_norm_fwd(x, weight, epsilon):
-    """Returns ``(y, rstd)``; ``x`` is ``(..., D)``, ``weight`` ``(D,)`` of the same dtype."""
-    dev = _dev(x, weight)
+    """Returns ``(y, rstd)``; ``x`` is ``(..., D)``, ``weight`` ``(D,)`` of the same dtype.
+    Differentiable through ``y``."""
+    _dev(x, weight)
     if x.dtype != weight.dtype:
         raise TypeError(f"rms_norm: input ({x.dtype}) and weight ({weight.dtype}) must share a dtype")
-    x, weight = _c(x), _c(weight)
-    D = weight.numel()
-    rows = x.numel() // D
-    y = torch.empty_like(x)
-    rstd = torch.empty(rows, dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
-        rc = _lib.load().mi355_rms_norm_fwd(_p(x), _p(weight), _dt(x), _p(y), _p(rstd), rows, D,
-                                            float(epsilon), _stream(dev))
-    _lib.check(rc, "rms_norm_fwd")
-    return y, rstd
+    _dt(x)
+    return _O.rms_norm_fwd(x, weight, float(epsilon))
 
 
 def rms_norm_bwd(dy, x, weight, rstd, need_dx=True, need_dw=True):
     """Returns ``(dx or None, dweight or None)``."""
-    dev = _dev(dy, x, weight, rstd)
-    dy, x, weight = _c(dy), _c(x), _c(weight)
-    if dy.dtype != x.dtype:
-        dy = dy.to(x.dtype)
-    D = weight.numel()
-    rows = x.numel() // D
-    lib = _lib.load()
-    dx = torch.empty_like(x) if need_dx else None
-    dw = torch.empty_like(weight) if need_dw else None
-    ws = torch.empty(max(lib.mi355_rms_norm_bwd_workspace_bytes(rows, D), 4), dtype=torch.uint8,
-                     device=dev) if need_dw else None
-    with torch.cuda.device(dev):
-        rc = lib.mi355_rms_norm_bwd(_p(dy), _p(x), _p(weight), _p(rstd), _dt(x), _p(dx), _p(dw), _p(ws),
-                                    rows, D, _stream(dev))
-    _lib.check(rc, "rms_norm_bwd")
-    return dx, dw
+    _dev(dy, x, weight, rstd)
+    dx, dw = _O.rms_norm_bwd(dy, x, weight, rstd, bool(need_dx), bool(need_dw))
+    return _opt(dx, need_dx), _opt(dw, need_dw)
 
 
-def router_select_bwd(logits_TE, ids_TK, dweights_TK, dscores_TE, score_func, route_norm,
-                      route_scale, mode=SELECT_TOPK):
-    dev = _dev(logits_TE, ids_TK, dweights_TK, dscores_TE)
-    logits_TE, ids_TK = _c(logits_TE), _c(ids_TK)
-    T, E = logits_TE.shape
-    K = ids_TK.shape[1]
-    dweights_TK = None if dweights_TK is None else _c(dweights_TK.float())
-    dscores_TE = None if dscores_TE is None else _c(dscores_TE.float())
-    out = torch.empty_like(logits_TE)
-    with torch.cuda.device(dev):
-        rc = _lib.load().mi355_router_select_bwd(
-            _p(logits_TE), _p(ids_TK), _p(dweights_TK), _p(dscores_TE), _p(out), T, E, K,
-            SCORE_FUNCS[score_func], int(route_norm), float(route_scale), mode, _stream(dev),
-        )
-    _lib.check(rc, "router_select_bwd")
-    return out
+def _as_bool(m):
+    return m if m.dtype == torch.bool else m.ne(0)
 
 
 def balance_loss_fwd(scores_TE, routing_map_TE, padding_mask_T=None):
-    """Returns (loss 0-d fp32, f_E) of the per-forward load-balance loss."""
-    dev = _dev(scores_TE, routing_map_TE, padding_mask_T)
+    """Returns (loss 0-d fp32, f_E) of the per-forward load-balance loss; the loss is
+    differentiable in the scores."""
+    _dev(scores_TE, routing_map_TE, padding_mask_T)
     if scores_TE.dtype != torch.float32:
         raise TypeError("router scores must be float32")
-    scores_TE = _c(scores_TE)
-    T, E = scores_TE.shape
     if routing_map_TE.shape != scores_TE.shape:
         raise ValueError(f"routing map {tuple(routing_map_TE.shape)} does not match scores {tuple(scores_TE.shape)}")
-    as_bytes = lambda m: _c(m).view(torch.uint8) if m.dtype == torch.bool else _c(m.ne(0)).view(torch.uint8)
-    rmap = as_bytes(routing_map_TE)
-    pad = None if padding_mask_T is None else as_bytes(padding_mask_T)
-    lib = _lib.load()
-    out = torch.empty(1 + E, dtype=torch.float32, device=dev)
-    ws = torch.empty(max(lib.mi355_balance_loss_workspace_bytes(T, E), 4), dtype=torch.uint8, device=dev)
-    with torch.cuda.device(dev):
-        rc = lib.mi355_balance_loss_fwd(_p(scores_TE), _p(rmap), _p(pad), _p(out), out[1:].data_ptr(), _p(ws),
-                                        T, E, _stream(dev))
-    _lib.check(rc, "balance_loss_fwd")
+    out = _O.balance_loss_fwd(scores_TE, _as_bool(routing_map_TE),
+                              None if padding_mask_T is None else _as_bool(padding_mask_T))
     return out[0], out[1:]
 
 
 def balance_loss_bwd(scores_TE, f_E, grad_loss, padding_mask_T=None):
-    dev = _dev(scores_TE, f_E, grad_loss, padding_mask_T)
-    scores_TE = _c(scores_TE)
-    T, E = scores_TE.shape
-    pad = None if padding_mask_T is None else _c(padding_mask_T).view(torch.uint8)
-    g = _c(grad_loss.float().reshape(1))
-    out = torch.empty_like(scores_TE)
-    with torch.cuda.device(dev):
-        rc = _lib.load().mi355_balance_loss_bwd(_p(scores_TE), _p(_c(f_E)), _p(pad), _p(g), _p(out), T, E,
-                                                _stream(dev))
-    _lib.check(rc, "balance_loss_bwd")
-    return out
+    _dev(scores_TE, f_E, grad_loss, padding_mask_T)
+    pad = None if padding_mask_T is None else _as_bool(padding_mask_T)
+    return _O.balance_loss_bwd(scores_TE, f_E, pad, grad_loss)
 
 
-# ------------------------------------------------------------------ plan
+# ====================================================================== plan
 @dataclass
 class PermutePlan:
     """Device-resident description of the expert-major row layout (all int32)."""
@@ -314,272 +563,194 @@ class PermutePlan:
         """0-d device view of the number of rows in use (padding included)."""
         return self.seg_offsets[self.num_local_experts]
 
+    def total_rows_1(self) -> torch.Tensor:
+        """The same as a 1-element view (what the operators take)."""
+        El = self.num_local_experts
+        return self.seg_offsets[El:El + 1]
+
+    def pad_index(self):
+        """slot_of_row when the plan has padding rows (they must read as zeros), else None."""
+        return self.slot_of_row if self.align > 1 else None
+
+    def segments(self):
+        return self.seg_offsets, self.seg_counts, self.tile_expert, self.tile_row0, self.num_tiles
+
+
+def _split_small(small, E, El, tile_cap):
+    o = 0
+    counts_E = None
+    if E:
+        counts_E = small[o:o + E]; o += E
+    seg_offsets = small[o:o + El + 1]; o += El + 1
+    # 2*El ints: the counts, then the experts by descending count
+    seg_counts = small[o:o + El]; expert_order = small[o + El:o + 2 * El]; o += 2 * El
+    tile_expert = small[o:o + tile_cap]; o += tile_cap
+    tile_row0 = small[o:o + tile_cap]; o += tile_cap
+    num_tiles = small[o:o + 1]
+    return counts_E, seg_offsets, seg_counts, expert_order, tile_expert, tile_row0, num_tiles
+
 
 def permute_plan(ids_TK, num_experts, local_lo=0, local_hi=None, align=1) -> PermutePlan:
-    dev = _dev(ids_TK)
-    if ids_TK.dtype != torch.int64:
-        ids_TK = ids_TK.to(torch.int64)
-    ids_TK = _c(ids_TK)
+    _dev(ids_TK)
     T, K = ids_TK.shape
     E = int(num_experts)
     hi = E if local_hi is None else int(local_hi)
     lo = int(local_lo)
     El = hi - lo
-    N = T * K
-    tm = tile_m()
-    row_cap = N + (El * (align - 1) if align > 1 else 0)
-    tile_cap = N // tm + El + 1
-    lib = _lib.load()
-    i32 = dict(dtype=torch.int32, device=dev)
-    # one allocation for the small arrays, one for the per-slot / per-row ones
-    small = torch.empty(E + (El + 1) + 2 * El + 2 * tile_cap + 1, **i32)
-    o = 0
-    counts_E = small[o:o + E]; o += E
-    seg_offsets = small[o:o + El + 1]; o += El + 1
-    # the library writes 2*El ints here: the counts, then the experts by descending count
-    seg_counts = small[o:o + El]; expert_order = small[o + El:o + 2 * El]; o += 2 * El
-    tile_expert = small[o:o + tile_cap]; o += tile_cap
-    tile_row0 = small[o:o + tile_cap]; o += tile_cap
-    num_tiles = small[o:o + 1]
-    row_of_slot = torch.empty(N, **i32)
-    rows2 = torch.empty(2, row_cap, **i32)
-    slot_of_row, token_of_row = rows2[0], rows2[1]
-    ws = torch.empty(lib.mi355_permute_plan_workspace_bytes(T, K, E), dtype=torch.uint8, device=dev)
-    with torch.cuda.device(dev):
-        rc = lib.mi355_permute_plan(
-            _p(ids_TK), T, K, E, lo, hi, align, tm, _p(counts_E), _p(seg_offsets), _p(seg_counts),
-            _p(row_of_slot), _p(slot_of_row), _p(token_of_row), row_cap, _p(tile_expert), _p(tile_row0),
-            _p(num_tiles), tile_cap, _p(ws), _stream(dev),
-        )
-    _lib.check(rc, "permute_plan")
-    return PermutePlan(T, K, E, lo, hi, align, tm, row_cap, tile_cap, counts_E, seg_offsets,
-                       seg_counts, row_of_slot, slot_of_row, token_of_row, tile_expert, tile_row0, num_tiles,
+    align = int(align)
+    row_cap, tile_cap = _plan_sizes(T * K, El, align)
+    small, row_of_slot, rows2 = _O.permute_plan(ids_TK, E, lo, hi, align)
+    counts_E, seg_offsets, seg_counts, expert_order, tile_expert, tile_row0, num_tiles = _split_small(
+        small, E, El, tile_cap)
+    return PermutePlan(T, K, E, lo, hi, align, TILE_M, row_cap, tile_cap, counts_E, seg_offsets,
+                       seg_counts, row_of_slot, rows2[0], rows2[1], tile_expert, tile_row0, num_tiles,
                        expert_order)
 
 
 def segments_from_counts(counts_e, total_rows: int) -> PermutePlan:
     """Plan for rows that are already expert-major with ``counts_e`` rows each."""
-    dev = _dev(counts_e)
-    counts = _c(counts_e.to(torch.int32))
-    El = counts.shape[0]
-    tm = tile_m()
-    tile_cap = total_rows // tm + El + 1
-    i32 = dict(dtype=torch.int32, device=dev)
-    small = torch.empty((El + 1) + 2 * El + 2 * tile_cap + 1, **i32)
-    o = 0
-    seg_offsets = small[o:o + El + 1]; o += El + 1
-    seg_counts = small[o:o + El]; expert_order = small[o + El:o + 2 * El]; o += 2 * El
-    tile_expert = small[o:o + tile_cap]; o += tile_cap
-    tile_row0 = small[o:o + tile_cap]; o += tile_cap
-    num_tiles = small[o:o + 1]
-    with torch.cuda.device(dev):
-        rc = _lib.load().mi355_segments_from_counts(
-            _p(counts), El, tm, total_rows, _p(seg_offsets), _p(seg_counts), _p(tile_expert), _p(tile_row0),
-            _p(num_tiles), tile_cap, _stream(dev),
-        )
-    _lib.check(rc, "segments_from_counts")
-    return PermutePlan(0, 1, El, 0, El, 1, tm, total_rows, tile_cap, None, seg_offsets, seg_counts,
+    _dev(counts_e)
+    El = counts_e.shape[0]
+    tile_cap = total_rows // TILE_M + El + 1
+    small = _O.segments_from_counts(counts_e, total_rows)
+    _, seg_offsets, seg_counts, expert_order, tile_expert, tile_row0, num_tiles = _split_small(small, 0, El, tile_cap)
+    return PermutePlan(0, 1, El, 0, El, 1, TILE_M, total_rows, tile_cap, None, seg_offsets, seg_counts,
                        None, None, None, tile_expert, tile_row0, num_tiles, expert_order)
 
 
-# ------------------------------------------------------------------ row movers
+# ====================================================================== row movers
 def permute_rows_fwd(x_TD, plan: PermutePlan):
-    dev = _dev(x_TD, plan.slot_of_row)
-    x_TD = _c(x_TD)
-    T, D = x_TD.shape
-    rows = torch.empty(plan.row_capacity, D, dtype=x_TD.dtype, device=dev)
-    with torch.cuda.device(dev):
-        rc = _lib.load().mi355_permute_rows_fwd(
-            _p(x_TD), _dt(x_TD), _p(plan.slot_of_row), _p(plan.total_rows), _p(rows), T, D,
-            plan.top_k, plan.row_capacity, _stream(dev),
-        )
-    _lib.check(rc, "permute_rows_fwd")
-    return rows
+    """rows[r] = x[token of row r], zeros in padding rows.  Differentiable in ``x`` (the
+    backward sums each token's K row gradients)."""
+    _dev(x_TD, plan.row_of_slot)
+    _dt(x_TD)
+    return _O.permute_rows_fwd(x_TD, plan.row_of_slot, plan.pad_index(), plan.total_rows_1(), plan.top_k,
+                               plan.row_capacity)
 
 
 def permute_rows_bwd(drows_RD, plan: PermutePlan):
-    dev = _dev(drows_RD, plan.row_of_slot)
-    drows_RD = _c(drows_RD)
-    D = drows_RD.shape[1]
-    dx = torch.empty(plan.num_tokens, D, dtype=drows_RD.dtype, device=dev)
-    with torch.cuda.device(dev):
-        rc = _lib.load().mi355_permute_rows_bwd(
-            _p(drows_RD), _dt(drows_RD), _p(plan.row_of_slot), _p(dx), plan.num_tokens, D,
-            plan.top_k, _stream(dev),
-        )
-    _lib.check(rc, "permute_rows_bwd")
-    return dx
+    _dev(drows_RD, plan.row_of_slot)
+    return _O.permute_rows_bwd(drows_RD, plan.row_of_slot, plan.num_tokens, plan.top_k)
 
 
-def combine_fwd(y_RD, weights_TK, plan: PermutePlan, round_terms=True, out_dtype=None):
-    dev = _dev(y_RD, weights_TK, plan.row_of_slot)
-    y_RD, weights_TK = _c(y_RD), _c(weights_TK.float())
-    D = y_RD.shape[1]
-    out = torch.empty(plan.num_tokens, D, dtype=y_RD.dtype, device=dev)
-    with torch.cuda.device(dev):
-        rc = _lib.load().mi355_combine_fwd(
-            _p(y_RD), _dt(y_RD), _p(weights_TK), _p(plan.row_of_slot), _p(out), plan.num_tokens, D,
-            plan.top_k, int(round_terms), _stream(dev),
-        )
-    _lib.check(rc, "combine_fwd")
-    return out
+def combine_fwd(y_RD, weights_TK, plan: PermutePlan, round_terms=True):
+    """out[t] = sum_k weights[t,k] * y[row(t,k)].  Differentiable in ``y`` and ``weights``."""
+    _dev(y_RD, weights_TK, plan.row_of_slot)
+    _dt(y_RD)
+    return _O.combine_fwd(y_RD, weights_TK, plan.row_of_slot, plan.pad_index(), plan.total_rows_1(),
+                          plan.num_tokens, plan.top_k, bool(round_terms))
 
 
 def combine_bwd(dout_TD, y_RD, weights_TK, plan: PermutePlan, zero_padding=True):
-    dev = _dev(dout_TD, y_RD, weights_TK)
-    dout_TD, y_RD, weights_TK = _c(dout_TD), _c(y_RD), _c(weights_TK.float())
-    if dout_TD.dtype != y_RD.dtype:
-        dout_TD = dout_TD.to(y_RD.dtype)
-    D = y_RD.shape[1]
-    dy = torch.empty_like(y_RD)
-    dw = torch.empty(plan.num_tokens, plan.top_k, dtype=torch.float32, device=dev)
-    pad = plan.slot_of_row if (zero_padding and plan.align > 1) else None
-    with torch.cuda.device(dev):
-        rc = _lib.load().mi355_combine_bwd(
-            _p(dout_TD), _p(y_RD), _dt(y_RD), _p(weights_TK), _p(plan.row_of_slot), _p(pad),
-            _p(plan.total_rows), _p(dy), _p(dw), plan.num_tokens, D, plan.top_k,
-            y_RD.shape[0], _stream(dev),
-        )
-    _lib.check(rc, "combine_bwd")
-    return dy, dw
+    _dev(dout_TD, y_RD, weights_TK)
+    pad = plan.pad_index() if zero_padding else None
+    return _O.combine_bwd(dout_TD, y_RD, weights_TK, plan.row_of_slot, pad, plan.total_rows_1(), plan.top_k)
 
 
-# ------------------------------------------------------------------ experts
+# ====================================================================== experts
 def gather_supported(x_TD, hidden_dim: int) -> bool:
     """The fused token gather exists for the bf16 MFMA kernels (D, F multiples of 64, at
-    least 384: the library's own condition for that path)."""
+    least 384: the library's own condition for that path) and addresses its source with
+    32-bit byte offsets."""
     D = x_TD.shape[-1]
     return (x_TD.dtype == torch.bfloat16 and D % 64 == 0 and hidden_dim % 64 == 0
-            and D >= 384 and hidden_dim >= 384 and x_TD.shape[0] * D < 2**31)
+            and D >= 384 and hidden_dim >= 384 and 1 <= x_TD.shape[0] and x_TD.shape[0] * D * 2 < 2**32)
 
 
-def grouped_swiglu_fwd(rows_RD, w1_EFD, w3_EFD, w2_EDF, plan: PermutePlan, gather=False):
-    """``gather=True``: ``rows_RD`` is the (T, D) token matrix, read through ``plan.token_of_row``."""
-    dev = _dev(rows_RD, w1_EFD, w3_EFD, w2_EDF)
-    rows_RD, w1_EFD, w3_EFD, w2_EDF = _c(rows_RD), _c(w1_EFD), _c(w3_EFD), _c(w2_EDF)
+def _check_experts(rows_RD, w1_EFD, w3_EFD, w2_EDF, plan):
     D = rows_RD.shape[1]
-    R = plan.row_capacity if gather else rows_RD.shape[0]
-    tok = plan.token_of_row if gather else None
     El, F, D2 = w1_EFD.shape
-    if D2 != D or w3_EFD.shape != w1_EFD.shape or w2_EDF.shape != (El, D, F):
+    if D2 != D or w3_EFD.shape != w1_EFD.shape or tuple(w2_EDF.shape) != (El, D, F):
         raise ValueError("expert weight shapes do not match (E,F,D)/(E,F,D)/(E,D,F)")
     if not (w1_EFD.dtype == w3_EFD.dtype == w2_EDF.dtype == rows_RD.dtype):
         raise TypeError("expert weights and rows must share one dtype")
     if El != plan.num_local_experts:
         raise ValueError(f"plan covers {plan.num_local_experts} experts, weights hold {El}")
-    mk = lambda n: torch.empty(R, n, dtype=rows_RD.dtype, device=dev)
-    gate, up, h, y = mk(F), mk(F), mk(F), mk(D)
-    with torch.cuda.device(dev):
-        rc = _lib.load().mi355_grouped_swiglu_fwd(
-            _p(rows_RD), _p(tok), _p(w1_EFD), _p(w3_EFD), _p(w2_EDF), _dt(rows_RD),
-            _p(plan.seg_offsets), _p(plan.seg_counts), _p(plan.tile_expert), _p(plan.tile_row0),
-            _p(plan.num_tiles), plan.tile_capacity, _p(gate), _p(up), _p(h), _p(y), El, D, F, R,
-            _stream(dev),
+    _dt(rows_RD)
+
+
+def grouped_swiglu_fwd(rows_RD, w1_EFD, w3_EFD, w2_EDF, plan: PermutePlan, gather=False, zero_fill=False):
+    """Returns ``(y, gate, up, h)``; ``y`` is differentiable in the rows and the weights
+    (not with ``gather``: that case is differentiated through ``gather_experts_combine``).
+
+    ``gather=True``: ``rows_RD`` is the (T, D) token matrix, read through ``plan.token_of_row``.
+    ``zero_fill``: rows the plan does not cover come back as zeros, not uninitialised."""
+    _dev(rows_RD, w1_EFD, w3_EFD, w2_EDF)
+    _check_experts(rows_RD, w1_EFD, w3_EFD, w2_EDF, plan)
+    if gather and plan.row_capacity > 0 and not gather_supported(rows_RD, w1_EFD.shape[1]):
+        raise ValueError(
+            "the fused token gather needs bf16, D and F multiples of 64 (>= 384), at least one token and a "
+            "token matrix below 4 GiB; materialise the rows with permute_rows_fwd instead"
         )
-    _lib.check(rc, "grouped_swiglu_fwd")
-    return y, gate, up, h
+    R = plan.row_capacity if gather else rows_RD.shape[0]
+    tok = plan.token_of_row if gather else None
+    return _O.grouped_swiglu_fwd(rows_RD, tok, w1_EFD, w3_EFD, w2_EDF, *plan.segments(), R, bool(zero_fill))
 
 
 def grouped_swiglu_bwd(dy_RD, rows_RD, w1_EFD, w3_EFD, w2_EDF, gate, up, h, plan: PermutePlan,
-                       need_drows=True, need_dw=True, gather=False):
-    dev = _dev(dy_RD, rows_RD)
-    dy_RD = _c(dy_RD)
-    w1_EFD, w3_EFD, w2_EDF = _c(w1_EFD), _c(w3_EFD), _c(w2_EDF)
-    D = rows_RD.shape[1]
-    R = dy_RD.shape[0]
+                       need_drows=True, need_dw=True, gather=False, zero_fill=False):
+    _dev(dy_RD, rows_RD)
+    if gather and dy_RD.shape[0] > 0 and not gather_supported(rows_RD, w1_EFD.shape[1]):
+        raise ValueError("the fused token gather does not cover this dtype / shape")
     tok = plan.token_of_row if gather else None
-    El, F, _ = w1_EFD.shape
-    dgate, dup = torch.empty_like(gate), torch.empty_like(up)
-    drows = torch.empty(R, D, dtype=rows_RD.dtype, device=dev) if need_drows else None
-    dw1 = torch.empty_like(w1_EFD) if need_dw else None
-    dw3 = torch.empty_like(w3_EFD) if need_dw else None
-    dw2 = torch.empty_like(w2_EDF) if need_dw else None
-    with torch.cuda.device(dev):
-        rc = _lib.load().mi355_grouped_swiglu_bwd(
-            _p(dy_RD), _p(rows_RD), _p(tok), _p(w1_EFD), _p(w3_EFD), _p(w2_EDF), _p(gate), _p(up),
-            _p(h), _dt(rows_RD), _p(plan.seg_offsets), _p(plan.seg_counts), _p(plan.tile_expert),
-            _p(plan.tile_row0), _p(plan.num_tiles), plan.tile_capacity, _p(dgate), _p(dup),
-            _p(drows), _p(dw1), _p(dw3), _p(dw2), El, D, F, R, _stream(dev),
-        )
-    _lib.check(rc, "grouped_swiglu_bwd")
-    return drows, dw1, dw3, dw2
-
-
-# False sends RoutedExperts through the two-call backward (combine, then experts) also where
-# the folded one applies (MI355_FOLD_COMBINE=0 in the environment does the same).
-FOLD_COMBINE = os.environ.get("MI355_FOLD_COMBINE", "1") != "0"
+    drows, dw1, dw3, dw2 = _O.grouped_swiglu_bwd(dy_RD, rows_RD, tok, w1_EFD, w3_EFD, w2_EDF, gate, up, h,
+                                                 *plan.segments(), bool(need_drows), bool(need_dw), bool(zero_fill))
+    return _opt(drows, need_drows), _opt(dw1, need_dw), _opt(dw3, need_dw), _opt(dw2, need_dw)
 
 
 def combine_bwd_slots(dtype, D, F):
     """Partials per row of the folded experts+combine backward; 0 when it does not apply."""
-    if dtype != torch.bfloat16 or not FOLD_COMBINE:
+    if dtype != torch.bfloat16:
         return 0
     return int(_lib.load().mi355_grouped_combine_bwd_slots(_DT[dtype], int(D), int(F)))
 
 
-def combine_row_scale(weights_TK, plan: PermutePlan):
-    """row_scale[r] = weights[slot_of_row[r]] (0 for padding rows), fp32."""
-    dev = _dev(weights_TK, plan.slot_of_row)
-    weights_TK = _c(weights_TK.float())
-    R = plan.row_capacity
-    out = torch.empty(R, dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
-        rc = _lib.load().mi355_combine_row_scale(
-            _p(weights_TK), _p(plan.slot_of_row), _p(out), plan.num_tokens, plan.top_k, R, _stream(dev),
-        )
-    _lib.check(rc, "combine_row_scale")
+def gather_experts_combine(x_TD, weights_TK, w1_EFD, w3_EFD, w2_EDF, plan: PermutePlan, round_terms=True):
+    """out[t] = sum_k weights[t,k] * experts(x)[row(t,k)], with one backward for both halves.
+
+    The forward is the gathered expert product followed by the combine.  The backward never
+    forms the expert-major output gradient ``weights * dout`` and never re-reads the expert
+    outputs: the dH kernel reads ``dout`` through the plan's token index and scales each row
+    in its epilogue, where the same pass yields the gradient of the routing weights (the row's
+    unscaled dh times its h, summed over the hidden columns); dW2 contracts the gathered
+    ``dout`` rows with ``weights * h``.  Nothing of size (R, D) is kept between forward and
+    backward, and of the (R, F) tensors only gate and up."""
+    _dev(x_TD, weights_TK, w1_EFD, w3_EFD, w2_EDF)
+    _check_experts(x_TD, w1_EFD, w3_EFD, w2_EDF, plan)
+    if not gather_supported(x_TD, w1_EFD.shape[1]):
+        raise ValueError("gather_experts_combine needs bf16 with D and F multiples of 64 (>= 384)")
+    out, _gate, _up = _O.gather_experts_combine_fwd(
+        x_TD, weights_TK, w1_EFD, w3_EFD, w2_EDF, plan.token_of_row, plan.slot_of_row, plan.row_of_slot,
+        *plan.segments(), plan.top_k, plan.row_capacity, bool(round_terms))
     return out
 
 
-def grouped_swiglu_combine_bwd(dout_TD, x_TD, row_scale_R, w1_EFD, w3_EFD, w2_EDF, gate, up, plan: PermutePlan,
-                               need_drows=True, need_dw=True, sum_rows=False):
-    """Backward of gathered experts + combine in one pass; returns (drows, dw1, dw3, dw2, dweights_TK).
-
-    ``sum_rows``: return ``dx`` (T, D), the K-way row sum of ``drows``, in its place.  The sum
-    then runs right behind the kernel that wrote ``drows``, while those rows are still in the
-    memory-side cache, and the weight-gradient kernels follow; summed after them it finds its
-    input gone to HBM.
-    """
-    dev = _dev(dout_TD, x_TD)
-    dout_TD, x_TD = _c(dout_TD), _c(x_TD)
-    if dout_TD.dtype != x_TD.dtype:
-        dout_TD = dout_TD.to(x_TD.dtype)
-    w1_EFD, w3_EFD, w2_EDF = _c(w1_EFD), _c(w3_EFD), _c(w2_EDF)
-    D = x_TD.shape[1]
-    R = gate.shape[0]
-    El, F, _ = w1_EFD.shape
-    lib = _lib.load()
-    slots = combine_bwd_slots(x_TD.dtype, D, F)
-    if slots <= 0:
-        raise _lib.MI355LibraryError("grouped_swiglu_combine_bwd does not cover this dtype/shape/layout")
-    dgate, dup, hs = torch.empty_like(gate), torch.empty_like(up), torch.empty_like(gate)
-    partial = torch.empty(R, slots, dtype=torch.float32, device=dev)
-    drows = torch.empty(R, D, dtype=x_TD.dtype, device=dev) if need_drows else None
-    dw1 = torch.empty_like(w1_EFD) if need_dw else None
-    dw3 = torch.empty_like(w3_EFD) if need_dw else None
-    dw2 = torch.empty_like(w2_EDF) if need_dw else None
-    def run(stages):
-        with torch.cuda.device(dev):
-            rc = lib.mi355_grouped_swiglu_combine_bwd(
-                _p(dout_TD), _p(x_TD), _p(plan.token_of_row), _p(row_scale_R), _p(w1_EFD), _p(w3_EFD), _p(w2_EDF),
-                _p(gate), _p(up), _dt(x_TD), _p(plan.seg_offsets), _p(plan.seg_counts), _p(plan.tile_expert),
-                _p(plan.tile_row0), _p(plan.num_tiles), plan.tile_capacity, _p(dgate), _p(dup), _p(hs), _p(partial),
-                _p(drows), _p(dw1), _p(dw3), _p(dw2), El, D, F, R, stages, _stream(dev),
-            )
-        _lib.check(rc, "grouped_swiglu_combine_bwd")
-
-    if not (sum_rows and need_drows and need_dw and R > 0):
-        run(0)
-        if sum_rows and drows is not None:
-            drows = permute_rows_bwd(drows, plan)
-        return drows, dw1, dw3, dw2, combine_scores_bwd(partial, plan)
-    run(STAGES["dh"] | STAGES["drows"])
-    dx = permute_rows_bwd(drows, plan)
-    dweights = combine_scores_bwd(partial, plan)
-    run(STAGES["dw2"] | STAGES["dw1"] | STAGES["dw3"])
-    return dx, dw1, dw3, dw2, dweights
+def combine_row_scale(weights_TK, plan: PermutePlan):
+    """row_scale[r] = weights[slot_of_row[r]] (0 for padding rows), fp32."""
+    _dev(weights_TK, plan.slot_of_row)
+    return _O.combine_row_scale(weights_TK, plan.slot_of_row, plan.row_capacity)
 
 
+def combine_scores_bwd(dot_partial, plan: PermutePlan):
+    _dev(dot_partial)
+    return _O.combine_scores_bwd(dot_partial, plan.row_of_slot, plan.num_tokens, plan.top_k)
+
+
+def grouped_swiglu_combine_bwd(dout_TD, x_TD, weights_TK, w1_EFD, w3_EFD, w2_EDF, gate, up, plan: PermutePlan,
+                               need_dx=True, need_dw=True):
+    """Backward of gathered experts + combine in one pass; returns (dx, dw1, dw3, dw2, dweights_TK)."""
+    _dev(dout_TD, x_TD)
+    if combine_bwd_slots(x_TD.dtype, x_TD.shape[1], w1_EFD.shape[1]) <= 0:
+        raise _lib.MI355LibraryError("grouped_swiglu_combine_bwd does not cover this dtype/shape")
+    dx, dw1, dw3, dw2, dweights = _O.gather_experts_combine_bwd(
+        dout_TD, x_TD, weights_TK, w1_EFD, w3_EFD, w2_EDF, gate, up, plan.token_of_row, plan.slot_of_row,
+        plan.row_of_slot, *plan.segments(), plan.top_k, bool(need_dx), bool(need_dw))
+    return _opt(dx, need_dx), _opt(dw1, need_dw), _opt(dw3, need_dw), _opt(dw2, need_dw), dweights
+
+
+# ====================================================================== profiling hooks
+# One MFMA kernel per call on pre-allocated buffers, straight through the C ABI: for
+# profilers and per-kernel timing.  Not operators: they write into caller-owned buffers.
 STAGES = {"gate_up": 1, "down": 2, "dh": 4, "drows": 8, "dw2": 16, "dw1": 32, "dw3": 64}
 
 
@@ -598,24 +769,12 @@ def grouped_swiglu_combine_stage(stage: str, buf: dict, plan: PermutePlan):
     g = lambda k: _p(buf.get(k))
     with torch.cuda.device(dev):
         rc = _lib.load().mi355_grouped_swiglu_combine_bwd(
-            g("dout"), g("rows"), _p(plan.token_of_row), g("row_scale"), g("w1"), g("w3"), g("w2"), g("gate"),
-            g("up"), _dt(x), _p(plan.seg_offsets), _p(plan.seg_counts), _p(plan.tile_expert), _p(plan.tile_row0),
-            _p(plan.num_tiles), plan.tile_capacity, g("dgate"), g("dup"), g("hs"), g("dot_partial"), g("drows"),
-            g("dw1"), g("dw3"), g("dw2"), El, D, F, R, STAGES[stage], _stream(dev),
+            g("dout"), g("rows"), _p(plan.token_of_row), x.shape[0], g("row_scale"), g("w1"), g("w3"), g("w2"),
+            g("gate"), g("up"), _dt(x), _p(plan.seg_offsets), _p(plan.seg_counts), _p(plan.tile_expert),
+            _p(plan.tile_row0), _p(plan.num_tiles), plan.tile_capacity, g("dgate"), g("dup"), g("hs"),
+            g("dot_partial"), g("drows"), g("dw1"), g("dw3"), g("dw2"), El, D, F, R, STAGES[stage], _stream(dev),
         )
     _lib.check(rc, f"grouped_swiglu_combine_bwd[{stage}]")
-
-
-def combine_scores_bwd(dot_partial, plan: PermutePlan):
-    dev = _dev(dot_partial)
-    dweights = torch.empty(plan.num_tokens, plan.top_k, dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
-        rc = _lib.load().mi355_combine_scores_bwd(
-            _p(dot_partial), dot_partial.shape[1], _p(plan.row_of_slot), _p(dweights), plan.num_tokens, plan.top_k,
-            dot_partial.shape[0], _stream(dev),
-        )
-    _lib.check(rc, "combine_scores_bwd")
-    return dweights
 
 
 def grouped_swiglu_stage(stage: str, buf: dict, plan: PermutePlan):
@@ -632,8 +791,8 @@ def grouped_swiglu_stage(stage: str, buf: dict, plan: PermutePlan):
     g = lambda k: _p(buf.get(k))
     with torch.cuda.device(dev):
         rc = _lib.load().mi355_grouped_swiglu_stage(
-            STAGES[stage], g("dy"), g("rows"), g("token_of_row"), g("w1"), g("w3"), g("w2"), g("gate"), g("up"), g("h"),
-            g("y"), _p(plan.seg_offsets), _p(plan.seg_counts), _p(plan.tile_expert),
+            STAGES[stage], g("dy"), g("rows"), g("token_of_row"), rows.shape[0], g("w1"), g("w3"), g("w2"),
+            g("gate"), g("up"), g("h"), g("y"), _p(plan.seg_offsets), _p(plan.seg_counts), _p(plan.tile_expert),
             _p(plan.tile_row0), _p(plan.num_tiles), plan.tile_capacity, g("dgate"), g("dup"),
             g("drows"), g("dw1"), g("dw3"), g("dw2"), El, D, F, R, _stream(dev),
         )
