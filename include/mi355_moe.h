@@ -236,6 +236,28 @@ int mi355_permute_plan(const int64_t* ids_TK, int64_t T, int64_t K, int64_t E,
                        int64_t tile_capacity, void* workspace, void* stream);
 
 /*
+ * mi355_permute_plan without a workspace argument, for callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that forbid it).  No
+ * counterpart in the reference.  Same arguments, outputs and results as mi355_permute_plan;
+ * the scratch (slot ranks, per-wave histograms) lives in an array inside the library,
+ * mi355_permute_plan_static_max_bytes() = 8 MiB per GPU, held until the process ends.
+ * Returns MI355_EINVAL without launching when mi355_permute_plan_workspace_bytes(T,K,E)
+ * exceeds that (e.g. N = T*K = 2^20 slots with E <= 128 fits; N = 131072, E = 256 fits).
+ * Calls no hipMalloc / hipFree and no allocating library routine.  All calls on one GPU share
+ * that GPU's array: calls that overlap on one GPU (two streams or threads) race -- serialise
+ * them, or use mi355_permute_plan with separate workspaces.
+ */
+int64_t mi355_permute_plan_static_max_bytes(void);
+int mi355_permute_plan_static(const int64_t* ids_TK, int64_t T, int64_t K, int64_t E,
+                              int64_t local_lo, int64_t local_hi, int64_t align,
+                              int64_t tile_m, int32_t* counts_E, int32_t* seg_offsets,
+                              int32_t* seg_counts, int32_t* row_of_slot,
+                              int32_t* slot_of_row, int32_t* token_of_row,
+                              int64_t row_capacity, int32_t* tile_expert,
+                              int32_t* tile_row0, int32_t* num_tiles,
+                              int64_t tile_capacity, void* stream);
+
+/*
  * Segment offsets, counts and the tile list for rows that are ALREADY expert-major
  * with `counts[e]` rows per local expert (no padding): the layout
  * GroupedExperts.forward receives, llmtuner/models/common/moe/experts.py:152-204

@@ -45,6 +45,8 @@ SIGNATURES = {
     "mi355_permute_plan_workspace_bytes": (L, [L, L, L]),
     "mi355_permute_plan": (I, [P, L, L, L, L, L, L, L, P, P, P, P, P, P, L, P, P, P, L, P, P]),
     "mi355_segments_from_counts": (I, [P, L, L, L, P, P, P, P, P, L, P]),
+    "mi355_permute_plan_static_max_bytes": (L, []),
+    "mi355_permute_plan_static": (I, [P, L, L, L, L, L, L, L, P, P, P, P, P, P, L, P, P, P, L, P]),
     "mi355_permute_rows_fwd": (I, [P, I, P, P, P, P, L, L, L, L, P]),
     "mi355_permute_rows_bwd": (I, [P, I, P, P, L, L, L, P]),
     "mi355_combine_fwd": (I, [P, I, P, P, P, L, L, L, I, P]),

@@ -478,6 +478,49 @@ extern "C" int mi355_permute_plan(const int64_t* ids, int64_t T, int64_t K, int6
                    as_stream(stream));
 }
 
+// ---- the same plan without a caller-provided workspace -------------------------------------
+// For callers that cannot allocate (under HIP graph capture, in a tight serving loop): the
+// ranks and per-wave histograms live in a file-scope device array, 8 MiB per GPU, held until
+// the process ends.  The array's name is a host-side stand-in, not a device address: its
+// address on each device is asked for once, with that device current, and only that pointer
+// is ever handed to kernels.  Every call on a GPU shares that GPU's array: calls that overlap
+// on one GPU (two streams, two threads) race.  Nothing in it must start at zero -- every word
+// a kernel of the plan reads was written by an earlier kernel of the same call.
+constexpr int64_t kStaticPlanBytes = 8ll << 20;
+static __device__ __align__(256) unsigned char plan_scratch[kStaticPlanBytes];
+constexpr int kMaxDevices = 64;
+static std::atomic<void*> plan_scratch_ptr[kMaxDevices];
+
+extern "C" int64_t mi355_permute_plan_static_max_bytes(void) { return kStaticPlanBytes; }
+
+extern "C" int mi355_permute_plan_static(const int64_t* ids, int64_t T, int64_t K, int64_t E, int64_t lo,
+                                         int64_t hi, int64_t align, int64_t tile_m, int32_t* counts_E,
+                                         int32_t* seg_offsets, int32_t* seg_counts, int32_t* row_of_slot,
+                                         int32_t* slot_of_row, int32_t* token_of_row, int64_t row_capacity,
+                                         int32_t* tile_expert, int32_t* tile_row0, int32_t* num_tiles,
+                                         int64_t tile_capacity, void* stream) {
+  MI355_REQUIRE(T >= 0 && K >= 1 && E >= 1 && T * K < (1ll << 30) && E <= 2048,
+                "permute_plan_static: bad shape T=%lld K=%lld E=%lld", (long long)T, (long long)K, (long long)E);
+  const int64_t need = mi355_permute_plan_workspace_bytes(T, K, E);
+  MI355_REQUIRE(need <= kStaticPlanBytes,
+                "permute_plan_static: T=%lld K=%lld E=%lld needs %lld bytes of scratch, the built-in array holds %lld; "
+                "use mi355_permute_plan with a workspace of your own",
+                (long long)T, (long long)K, (long long)E, (long long)need, (long long)kStaticPlanBytes);
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    return fail(MI355_ELAUNCH, "permute_plan_static: no current device");
+  void* ptr = plan_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!ptr) {
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(plan_scratch));
+    if (e != hipSuccess || !ptr)
+      return fail(MI355_ELAUNCH, "permute_plan_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    plan_scratch_ptr[dev].store(ptr, std::memory_order_release);
+  }
+  return plan_impl(ids, T, K, E, lo, hi, align, tile_m, counts_E, seg_offsets, seg_counts, row_of_slot, slot_of_row,
+                   token_of_row, row_capacity, tile_expert, tile_row0, num_tiles, tile_capacity, ptr,
+                   as_stream(stream));
+}
+
 extern "C" int mi355_permute_rows_fwd(const void* x, int dtype, const int32_t* row_of_slot,
                                       const int32_t* slot_of_row, const int32_t* total_rows, void* rows,
                                       int64_t T, int64_t D, int64_t K, int64_t row_capacity, void* stream) {
