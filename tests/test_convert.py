@@ -117,3 +117,76 @@ def test_converted_block_computes_the_hf_expert_math():
             gate, up = bf(gu[e, :Fg].float() @ x[t].float()), bf(gu[e, Fg:].float() @ x[t].float())
             ref[t] += float(w[t, k]) * bf(dn[e].float() @ bf(bf(torch.nn.functional.silu(gate)) * up))
     assert (out - ref).norm() / ref.norm() < 2e-2
+
+
+# ---- convert_block: the reference's own entry, fed with objects that merely LOOK like its bindings
+class _Gate(torch.nn.Module):
+    """An HF-style router gate: ``weight (E, D)`` and the aux-loss-free correction bias."""
+
+    def __init__(self, weight, bias=None):
+        super().__init__()
+        self.weight = torch.nn.Parameter(weight.clone())
+        if bias is not None:
+            self.register_buffer("e_score_correction_bias", bias.clone())
+
+
+def _bindings(dtype=torch.bfloat16, bias=None, shared=None, **routing):
+    """Plain stand-ins with the fields of MoERoutingBinding / PackedExpertBinding /
+    PackedExpertViews (llmtuner/parallel/expert_parallel/bindings.py:36-170); none of the
+    reference's classes is imported."""
+    from collections import namedtuple
+    from types import SimpleNamespace
+
+    rw, gu, dn = _packed(dtype)
+    fields = dict(top_k=K, score_func="sigmoid", route_norm=True, route_scale=2.5, num_expert_groups=None,
+                  num_limited_groups=None)
+    fields.update(routing)
+    routing_binding = SimpleNamespace(source=None, router=_Gate(rw, bias), shared=shared, shared_gate=None, **fields)
+    views = namedtuple("PackedExpertViews", "gate_EFD up_EFD down_EDF num_experts")(gu[:, :F], gu[:, F:], dn, E)
+    binding = SimpleNamespace(gate_up=torch.nn.Parameter(gu.clone()), down=torch.nn.Parameter(dn.clone()),
+                              shape=tuple(gu.shape))
+    return routing_binding, views, binding, (rw, gu, dn)
+
+
+def test_convert_block_accepts_the_reference_binding_objects_by_their_fields():
+    bias = torch.linspace(-1, 1, E)
+    shared = moe.DenseSwiGLU(D, F)
+    routing, views, binding, (rw, gu, dn) = _bindings(bias=bias, shared=shared)
+    source = torch.nn.Module().eval()  # the HF block being replaced: supplies the mode
+    for packed in (views, binding):
+        block = moe.convert_block(source, routing=routing, packed_experts=packed, ep_group=None,
+                                  aux_loss_coeff=0.01, load_balance_coeff=1e-3, quantile_balancing=False,
+                                  token_dispatcher="alltoall", torchao_pad_multiple=16)
+        ie = block.routed_experts.inner_experts
+        assert torch.equal(ie.w1_EFD, gu[:, :F]) and torch.equal(ie.w3_EFD, gu[:, F:]) and torch.equal(ie.w2_EDF, dn)
+        assert ie.w1_EFD.dtype == torch.bfloat16
+        assert torch.equal(block.router.gate.weight, rw) and block.router.gate.weight.dtype == torch.float32
+        assert torch.equal(block.expert_bias_E, bias) and block.expert_bias_E.dtype == torch.float32
+        assert block.shared_experts is shared and not block.training
+        r = block.router
+        assert (r.top_k, r.score_func, r.route_norm, r.route_scale) == (K, "sigmoid", True, 2.5)
+        assert isinstance(r.aux_loss, moe.MicrobatchWiseLoadBalanceLoss) and r.aux_loss.coeff == 0.01
+        assert isinstance(block.routed_experts.token_dispatcher, moe.LocalTokenDispatcher)
+    # a binding that can validate itself is asked to
+    calls = []
+    routing.validate = lambda blk: calls.append(blk)
+    padded = moe.convert_block(source, routing=routing, packed_experts=views, token_dispatcher="torchao",
+                               torchao_pad_multiple=32, load_balance_coeff=None)
+    assert calls == [source] and padded.expert_bias_E is None
+    assert padded.routed_experts.token_dispatcher.pad_multiple == 32
+
+
+def test_convert_block_quantile_balancing_and_what_one_gpu_refuses():
+    routing, views, _, _ = _bindings()
+    q = moe.convert_block(None, routing=routing, packed_experts=views, quantile_balancing=True)
+    assert isinstance(q.router, moe.QuantileBalancedTopKRouter) and q.load_balance_coeff is None
+    assert q.expert_bias_E is not None and q.training
+    soft, views2, _, _ = _bindings(score_func="softmax")
+    with pytest.raises(ValueError, match="sigmoid"):
+        moe.convert_block(None, routing=soft, packed_experts=views2, quantile_balancing=True)
+    for kw, needle in ((dict(ep_group=object()), "one GPU"), (dict(tp_enabled=True), "tensor parallelism"),
+                       (dict(token_dispatcher="domino"), "peers")):
+        with pytest.raises(NotImplementedError, match=needle):
+            moe.convert_block(None, routing=routing, packed_experts=views, **kw)
+    with pytest.raises(TypeError, match="packed_experts"):
+        moe.convert_block(None, routing=routing, packed_experts=object())

@@ -11,6 +11,7 @@ from .bias_update import (
     update_quantile_expert_bias,
 )
 from .convert import (
+    convert_block,
     hf_expert_state_to_native,
     moe_from_packed_experts,
     native_ep_expert_key,
@@ -46,6 +47,7 @@ __all__ = [
     "SwiGLU",
     "TokenChoiceTopKRouter",
     "collect_moe_layers",
+    "convert_block",
     "collect_routing_load_metrics",
     "hf_expert_state_to_native",
     "moe_from_packed_experts",

@@ -22,12 +22,13 @@ import torch.nn as nn
 from .auxiliary_loss import MicrobatchWiseLoadBalanceLoss
 from .experts import GroupedExperts, RoutedExperts
 from .layer import MoE
-from .routing import TokenChoiceTopKRouter
+from .routing import QuantileBalancedTopKRouter, TokenChoiceTopKRouter
 from .token_dispatch import LocalShareTokenDispatcher, LocalTokenDispatcher, PaddedTokenDispatcher
 
 __all__ = [
     "HF_PROJECTIONS",
     "NATIVE_PROJECTIONS",
+    "convert_block",
     "hf_expert_state_to_native",
     "moe_from_packed_experts",
     "native_ep_expert_key",
@@ -163,4 +164,109 @@ def moe_from_packed_experts(
         target.requires_grad_(source.requires_grad)
     moe.shared_experts = shared_experts
     moe.train(training)
+    return moe
+
+
+def _expert_views(packed_experts, block):
+    """(gate_EFD, up_EFD, down_EDF, num_experts) from whatever describes the packed experts: the
+    reference's ``PackedExpertBinding`` (``projections(block)``, or its ``gate_up`` / ``down`` /
+    ``shape`` fields) or its ``PackedExpertViews`` tuple (bindings.py:101-170), by their fields."""
+    if hasattr(packed_experts, "gate_EFD"):
+        views = packed_experts
+    elif callable(getattr(packed_experts, "projections", None)):
+        views = packed_experts.projections(block)
+    elif hasattr(packed_experts, "gate_up") and hasattr(packed_experts, "down"):
+        gate_up, down = packed_experts.gate_up, packed_experts.down
+        hidden = gate_up.shape[1] // 2
+        return gate_up[:, :hidden], gate_up[:, hidden:], down, gate_up.shape[0]
+    else:
+        raise TypeError(
+            "packed_experts must provide gate_EFD / up_EFD / down_EDF / num_experts, a projections(block) "
+            "method, or gate_up / down parameters"
+        )
+    return views.gate_EFD, views.up_EFD, views.down_EDF, int(views.num_experts)
+
+
+def convert_block(
+    block: nn.Module | None,
+    *,
+    routing,
+    packed_experts,
+    ep_group=None,
+    aux_loss_coeff: float | None = None,
+    load_balance_coeff: float | None = 1e-3,
+    quantile_balancing: bool = False,
+    token_dispatcher: str = "alltoall",
+    torchao_pad_multiple: int = 16,
+    tp_enabled: bool = False,
+) -> MoE:
+    """The reference's ``convert_block`` for one GPU, with its own keyword surface
+    (llmtuner/parallel/expert_parallel/block_conversion.py:123-300): one native block built
+    from already resolved bindings.
+
+    ``routing`` is read by its fields (``router`` -- the HF gate module with ``weight (E, D)``
+    and optionally ``e_score_correction_bias`` --, ``shared``, ``top_k``, ``score_func``,
+    ``route_norm``, ``route_scale``, ``num_expert_groups``, ``num_limited_groups``; the reference's
+    ``MoERoutingBinding``, bindings.py:36-98), ``packed_experts`` as described in
+    ``_expert_views``; both are validated against ``block`` when they offer ``validate``.  No
+    reference class is imported: any object with those fields will do.  One process owns every
+    expert: an expert-parallel group, tensor parallelism and the dispatchers that need peers are
+    refused.  ``block`` only supplies the training / eval mode (``None``: training).
+    """
+    if ep_group is not None:
+        raise NotImplementedError("convert_block: this build runs on one GPU; ep_group must be None")
+    if tp_enabled:
+        raise NotImplementedError("convert_block: tensor parallelism needs more than one GPU")
+    if token_dispatcher not in ("alltoall", "torchao"):
+        raise NotImplementedError(
+            f"convert_block: the {token_dispatcher!r} dispatcher needs expert-parallel peers; one GPU runs "
+            "'alltoall' (local reordering at EP=1) or 'torchao' (padded segments)"
+        )
+    for binding in (routing, packed_experts):
+        validate = getattr(binding, "validate", None)
+        if callable(validate) and block is not None:
+            validate(block)
+    gate_EFD, up_EFD, down_EDF, num_experts = _expert_views(packed_experts, block)
+    router_gate = routing.router
+    weight = router_gate.weight
+    if tuple(weight.shape) != (num_experts, gate_EFD.shape[2]):
+        raise ValueError(
+            f"router weight {tuple(weight.shape)} does not match {num_experts} experts of width {gate_EFD.shape[2]}"
+        )
+    dim, hidden, top_k = weight.shape[1], gate_EFD.shape[1], routing.top_k
+    aux = MicrobatchWiseLoadBalanceLoss(coeff=aux_loss_coeff) if aux_loss_coeff else None
+    if quantile_balancing:
+        if routing.score_func != "sigmoid" or routing.num_expert_groups is not None:
+            raise ValueError("quantile balancing is defined over sigmoid scores without expert groups")
+        router = QuantileBalancedTopKRouter(num_experts, dim, top_k, route_norm=routing.route_norm,
+                                            route_scale=routing.route_scale, aux_loss=aux)
+        load_balance_coeff = None  # the quantile update owns expert_bias_E
+    else:
+        router = TokenChoiceTopKRouter(
+            num_experts, dim, top_k, score_func=routing.score_func, route_norm=routing.route_norm,
+            route_scale=routing.route_scale, num_expert_groups=routing.num_expert_groups,
+            num_limited_groups=routing.num_limited_groups, aux_loss=aux)
+    if token_dispatcher == "torchao":
+        dispatcher = PaddedTokenDispatcher(num_experts, top_k, pad_multiple=torchao_pad_multiple)
+    else:
+        dispatcher = LocalTokenDispatcher(num_experts, top_k)
+    grouped = GroupedExperts(dim, hidden, num_experts)
+    moe = MoE(num_experts, RoutedExperts(grouped, dispatcher), router, load_balance_coeff=load_balance_coeff)
+    # the expert subtree in its source dtype, the router in its own (fp32 under bf16 experts)
+    moe.to(dtype=gate_EFD.dtype, device=weight.device)
+    router.to(dtype=weight.dtype, device=weight.device)
+    moe.train(True if block is None else block.training)
+    projections = ((grouped.w1_EFD, gate_EFD), (grouped.w3_EFD, up_EFD), (grouped.w2_EDF, down_EDF))
+    router.gate.weight.requires_grad_(weight.requires_grad)
+    for target, source in projections:
+        target.requires_grad_(source.requires_grad)
+    with torch.no_grad():
+        router.gate.weight.copy_(weight)
+        for target, source in projections:
+            target.copy_(source)
+        bias = getattr(router_gate, "e_score_correction_bias", None)
+        if bias is not None and moe.expert_bias_E is not None:
+            moe.expert_bias_E.copy_(bias.float())
+    # the HF shared expert is reused as it is, after the new subtree was cast and moved
+    moe.shared_experts = getattr(routing, "shared", None)
     return moe
