@@ -44,7 +44,8 @@ __device__ __forceinline__ float round_to<float>(float v) { return v; }
 template <>
 __device__ __forceinline__ float round_to<uint16_t>(float v) { return round_bf16(v); }
 
-template <typename T>
+// SMALL_K: K <= 8, the eight-row chunk below is the only one
+template <typename T, bool SMALL_K>
 __global__ __launch_bounds__(256) void combine_fwd_kernel(
     const T* __restrict__ y, const float* __restrict__ weights,
     const int32_t* __restrict__ row_of_slot, T* __restrict__ out, int T_, int D, int K,
@@ -62,55 +63,87 @@ __global__ __launch_bounds__(256) void combine_fwd_kernel(
     pos += (rj >= 0 && (rj < row || (rj == row && j < lane))) ? 1 : 0;
   }
   const int nvalid = __popcll(__ballot(row >= 0));
-  int o_row = -1;
-  float o_w = 0.0f;  // lane p holds the p-th visited slot
-  for (int p = 0; p < nvalid; ++p) {
-    const unsigned long long m = __ballot(row >= 0 && pos == p);
-    const int src = __ffsll(static_cast<long long>(m)) - 1;
-    const int r = __shfl(row, src, kWave);
-    const float ww = __shfl(w, src, kWave);
-    if (lane == p) { o_row = r; o_w = ww; }
-  }
+  // lane p receives the p-th visited slot: every valid lane sends its (row, weight) to lane
+  // `pos` (one cross-lane permute each); the others send to lane 63, which is past the last
+  // valid position whenever such a lane exists and is not read then
+  const int to = (row >= 0 ? pos : 63) << 2;
+  int o_row = __builtin_amdgcn_ds_permute(to, row);
+  float o_w = __int_as_float(__builtin_amdgcn_ds_permute(to, __float_as_int(w)));
+  if (lane >= nvalid) { o_row = -1; o_w = 0.0f; }
 
   constexpr int V = Vec<T>::N;
   T* dst = out + static_cast<int64_t>(t) * D;
   // Loops are uniform across the wave (shuffles need every lane).
   if (D % V == 0) {
     const int nv = D / V;
-    for (int base = 0; base < nv; base += kWave) {
-      const int i = base + lane;
-      const bool on = i < nv;
-      float a[V];
+    // G vectors per lane and pass (4 KiB of every row per wave) from eight rows at a time, all
+    // requested before the first is used: 32 KiB in flight per wave.  Rows and weights are
+    // wave-uniform; the terms are still added in visiting order.
+    constexpr int G = 4, B = 8;
+    auto request = [&](int base, int p0, uint4 (&v)[B][G], float (&ww)[B]) {
 #pragma unroll
-      for (int q = 0; q < V; ++q) a[q] = 0.0f;
-      // eight rows requested before the first is used (one load at a time leaves a wave with
-      // 1 KiB in flight); the terms are still added in visiting order
-      constexpr int B = 8;
-      for (int p0 = 0; p0 < nvalid; p0 += B) {
-        uint4 v[B];
-        float ww[B];
+      for (int j = 0; j < B; ++j) {
+        const int p = min(p0 + j, nvalid - 1);  // past the end: not loaded, not used
+        const int r = __builtin_amdgcn_readfirstlane(__shfl(o_row, p, kWave));
+        ww[j] = __shfl(o_w, p, kWave);
+        const uint4* src = reinterpret_cast<const uint4*>(y + static_cast<int64_t>(max(r, 0)) * D);
 #pragma unroll
-        for (int j = 0; j < B; ++j) {
-          const int p = min(p0 + j, nvalid - 1);  // past the end: the last row again, not used
-          const int r = __shfl(o_row, p, kWave);
-          ww[j] = __shfl(o_w, p, kWave);
-          v[j] = make_uint4(0, 0, 0, 0);
-          if (on && p0 + j < nvalid) v[j] = reinterpret_cast<const uint4*>(y + static_cast<int64_t>(r) * D)[i];
-        }
-#pragma unroll
-        for (int j = 0; j < B; ++j) {
-          if (p0 + j < nvalid) {
-            float f[V];
-            Vec<T>::unpack(v[j], f);
-#pragma unroll
-            for (int q = 0; q < V; ++q) {
-              const float term = f[q] * ww[j];
-              a[q] += round_terms ? round_to<T>(term) : term;
-            }
-          }
+        for (int g = 0; g < G; ++g) {
+          const int i = base + g * kWave + lane;
+          v[j][g] = (p0 + j < nvalid && i < nv) ? load_stream(src + i) : make_uint4(0, 0, 0, 0);
         }
       }
-      if (on) reinterpret_cast<uint4*>(dst)[i] = Vec<T>::pack(a);
+    };
+    auto add_terms = [&](float (&a)[V], const uint4& v, float w) {
+      float f[V];
+      Vec<T>::unpack(v, f);
+#pragma unroll
+      for (int q = 0; q < V; ++q) {
+        const float term = f[q] * w;
+        a[q] += round_terms ? round_to<T>(term) : term;
+      }
+    };
+    for (int base = 0; base < nv; base += G * kWave) {
+      if constexpr (SMALL_K) {
+        // one chunk: each vector is summed and stored on its own (8 live accumulators, not 32,
+        // which is what lets three waves share a SIMD)
+        uint4 v[B][G];
+        float ww[B];
+        request(base, 0, v, ww);
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+          float a[V];
+#pragma unroll
+          for (int q = 0; q < V; ++q) a[q] = 0.0f;
+#pragma unroll
+          for (int j = 0; j < B; ++j)
+            if (j < nvalid) add_terms(a, v[j][g], ww[j]);
+          const int i = base + g * kWave + lane;
+          if (i < nv) reinterpret_cast<uint4*>(dst)[i] = Vec<T>::pack(a);
+        }
+      } else {
+        float a[G][V];
+#pragma unroll
+        for (int g = 0; g < G; ++g)
+#pragma unroll
+          for (int q = 0; q < V; ++q) a[g][q] = 0.0f;
+        for (int p0 = 0; p0 < nvalid; p0 += B) {
+          uint4 v[B][G];
+          float ww[B];
+          request(base, p0, v, ww);
+#pragma unroll
+          for (int j = 0; j < B; ++j)
+            if (p0 + j < nvalid) {
+#pragma unroll
+              for (int g = 0; g < G; ++g) add_terms(a[g], v[j][g], ww[j]);
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+          const int i = base + g * kWave + lane;
+          if (i < nv) reinterpret_cast<uint4*>(dst)[i] = Vec<T>::pack(a[g]);
+        }
+      }
     }
   } else {
     for (int base = 0; base < D; base += kWave) {
@@ -134,7 +167,7 @@ __global__ __launch_bounds__(256) void combine_bwd_kernel(
     const T* __restrict__ dout, const T* __restrict__ y, const float* __restrict__ weights,
     const int32_t* __restrict__ row_of_slot, const int32_t* __restrict__ slot_of_row,
     const int32_t* __restrict__ total_rows, T* __restrict__ dy, float* __restrict__ dweights,
-    int T_, int D, int K, int token_blocks, int row_capacity) {
+    int T_, int D, int K, int token_blocks, int row_capacity, int stream_stores) {
   const int lane = threadIdx.x & 63;
   constexpr int V = Vec<T>::N;
   if (static_cast<int>(blockIdx.x) >= token_blocks) {
@@ -175,7 +208,7 @@ __global__ __launch_bounds__(256) void combine_bwd_kernel(
 #pragma unroll
         for (int q = 0; q < G; ++q) {
           const int i = base + q * kWave + lane;
-          yv[q] = i < nv ? yr[i] : make_uint4(0, 0, 0, 0);
+          yv[q] = i < nv ? load_stream(yr + i) : make_uint4(0, 0, 0, 0);
         }
         float dot = 0.0f;
 #pragma unroll
@@ -188,7 +221,10 @@ __global__ __launch_bounds__(256) void combine_bwd_kernel(
             dot += yf[c] * gf[q][c];
             o[c] = gf[q][c] * ww;
           }
-          if (i < nv) dr[i] = Vec<T>::pack(o);
+          if (i < nv) {
+            if (stream_stores) store_stream(dr + i, Vec<T>::pack(o));
+            else dr[i] = Vec<T>::pack(o);
+          }
         }
         dot = wave_sum(dot);
         if (lane == k) my_dot += dot;
@@ -227,15 +263,17 @@ extern "C" int mi355_combine_fwd(const void* y, int dtype, const float* weights,
   if (T == 0) return MI355_OK;
   MI355_REQUIRE(weights && row_of_slot && out, "combine_fwd: null pointer");
   const dim3 grid((unsigned)((T + 3) / 4));
-  if (dtype == MI355_F32)
-    hipLaunchKernelGGL(combine_fwd_kernel<float>, grid, dim3(256), 0, as_stream(stream),
-                       static_cast<const float*>(y), weights, row_of_slot, static_cast<float*>(out),
-                       (int)T, (int)D, (int)K, round_terms);
-  else if (dtype == MI355_BF16)
-    hipLaunchKernelGGL(combine_fwd_kernel<uint16_t>, grid, dim3(256), 0, as_stream(stream),
-                       static_cast<const uint16_t*>(y), weights, row_of_slot,
-                       static_cast<uint16_t*>(out), (int)T, (int)D, (int)K, round_terms);
-  else
+  auto launch = [&](auto kernel, auto* yp, auto* op) {
+    hipLaunchKernelGGL(kernel, grid, dim3(256), 0, as_stream(stream), yp, weights, row_of_slot, op, (int)T, (int)D,
+                       (int)K, round_terms);
+  };
+  if (dtype == MI355_F32) {
+    if (K <= 8) launch(combine_fwd_kernel<float, true>, static_cast<const float*>(y), static_cast<float*>(out));
+    else launch(combine_fwd_kernel<float, false>, static_cast<const float*>(y), static_cast<float*>(out));
+  } else if (dtype == MI355_BF16) {
+    if (K <= 8) launch(combine_fwd_kernel<uint16_t, true>, static_cast<const uint16_t*>(y), static_cast<uint16_t*>(out));
+    else launch(combine_fwd_kernel<uint16_t, false>, static_cast<const uint16_t*>(y), static_cast<uint16_t*>(out));
+  } else
     return fail(MI355_EINVAL, "combine_fwd: unknown dtype %d", dtype);
   return check_launch("combine_fwd");
 }
@@ -253,16 +291,19 @@ extern "C" int mi355_combine_bwd(const void* dout, const void* y, int dtype, con
   MI355_REQUIRE(T == 0 || (dout && weights && row_of_slot && dy), "combine_bwd: null pointer");
   MI355_REQUIRE(!slot_of_row || total_rows, "combine_bwd: total_rows required with slot_of_row");
   const dim3 grid((unsigned)(token_blocks + pad_blocks));
+  // dy larger than the 256 MiB memory-side cache is written with non-temporal stores (as the
+  // row scatter of the forward permutation does)
+  const int stream_stores = row_capacity * D * (dtype == MI355_F32 ? 4 : 2) > (256ll << 20);
   if (dtype == MI355_F32)
     hipLaunchKernelGGL(combine_bwd_kernel<float>, grid, dim3(256), 0, as_stream(stream),
                        static_cast<const float*>(dout), static_cast<const float*>(y), weights,
                        row_of_slot, slot_of_row, total_rows, static_cast<float*>(dy), dweights,
-                       (int)T, (int)D, (int)K, token_blocks, (int)row_capacity);
+                       (int)T, (int)D, (int)K, token_blocks, (int)row_capacity, stream_stores);
   else if (dtype == MI355_BF16)
     hipLaunchKernelGGL(combine_bwd_kernel<uint16_t>, grid, dim3(256), 0, as_stream(stream),
                        static_cast<const uint16_t*>(dout), static_cast<const uint16_t*>(y), weights,
                        row_of_slot, slot_of_row, total_rows, static_cast<uint16_t*>(dy), dweights,
-                       (int)T, (int)D, (int)K, token_blocks, (int)row_capacity);
+                       (int)T, (int)D, (int)K, token_blocks, (int)row_capacity, stream_stores);
   else
     return fail(MI355_EINVAL, "combine_bwd: unknown dtype %d", dtype);
   return check_launch("combine_bwd");

@@ -272,7 +272,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void permute_rows_fwd_kernel(
     const T* __restrict__ x, const int32_t* __restrict__ row_of_slot, const int32_t* __restrict__ slot_of_row,
     const int32_t* __restrict__ total_rows, T* __restrict__ rows, int T_, int D, int K, int token_blocks,
-    int row_capacity) {
+    int row_capacity, int stream_stores) {
   const int lane = threadIdx.x & 63;
   constexpr int V = 16 / sizeof(T);
   if (static_cast<int>(blockIdx.x) >= token_blocks) {
@@ -307,7 +307,10 @@ __global__ __launch_bounds__(256) void permute_rows_fwd_kernel(
 #pragma unroll
         for (int g = 0; g < G; ++g) {
           const int i = base + g * kWave + lane;
-          if (i < nv) d4[i] = v[g];
+          if (i < nv) {
+            if (stream_stores) store_stream(d4 + i, v[g]);
+            else d4[i] = v[g];
+          }
         }
       }
     }
@@ -363,29 +366,39 @@ __global__ __launch_bounds__(256) void permute_rows_bwd_kernel(
   // end of the row just skip their loads and stores.
   if (D % V == 0) {
     const int nv = D / V;
-    for (int base = 0; base < nv; base += kWave) {
-      const int i = base + lane;
-      const bool on = i < nv;
-      float a[V];
+    // G vectors per lane and pass (4 KiB of every row per wave) from eight rows at a time, all
+    // requested before the first is summed: 32 KiB in flight per wave.  The row numbers are
+    // wave-uniform (scalar address arithmetic); the sum still runs in ascending k.
+    constexpr int G = 4, B = 8;
+    for (int base = 0; base < nv; base += G * kWave) {
+      float a[G][V];
 #pragma unroll
-      for (int q = 0; q < V; ++q) a[q] = 0.0f;
-      // eight rows requested before the first is summed: one load at a time leaves a wave
-      // with 1 KiB in flight, too little to keep HBM busy; the sum still runs in ascending k
-      constexpr int B = 8;
+      for (int g = 0; g < G; ++g)
+#pragma unroll
+        for (int q = 0; q < V; ++q) a[g][q] = 0.0f;
       for (int k0 = 0; k0 < K; k0 += B) {
-        uint4 v[B];
+        uint4 v[B][G];
 #pragma unroll
         for (int j = 0; j < B; ++j) {
           const int k = k0 + j;
-          const int row = __shfl(my_row, k < K ? k : 0, kWave);
-          v[j] = make_uint4(0, 0, 0, 0);
-          if (k < K && row >= 0 && on)
-            v[j] = reinterpret_cast<const uint4*>(drows + static_cast<int64_t>(row) * D)[i];
+          const int row = k < K ? __builtin_amdgcn_readfirstlane(__shfl(my_row, k, kWave)) : -1;
+          const uint4* src = reinterpret_cast<const uint4*>(drows + static_cast<int64_t>(max(row, 0)) * D);
+#pragma unroll
+          for (int g = 0; g < G; ++g) {
+            const int i = base + g * kWave + lane;
+            v[j][g] = (row >= 0 && i < nv) ? load_stream(src + i) : make_uint4(0, 0, 0, 0);
+          }
         }
 #pragma unroll
-        for (int j = 0; j < B; ++j) acc_vec<T>(a, v[j]);  // absent rows add zeros
+        for (int j = 0; j < B; ++j)
+#pragma unroll
+          for (int g = 0; g < G; ++g) acc_vec<T>(a[g], v[j][g]);  // absent rows add zeros
       }
-      if (on) reinterpret_cast<uint4*>(dst)[i] = pack_vec<T>(a);
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        const int i = base + g * kWave + lane;
+        if (i < nv) reinterpret_cast<uint4*>(dst)[i] = pack_vec<T>(a[g]);
+      }
     }
   } else {
     for (int base = 0; base < D; base += kWave) {
@@ -534,14 +547,19 @@ extern "C" int mi355_permute_rows_fwd(const void* x, int dtype, const int32_t* r
   const int pad_blocks = slot_of_row ? (int)((row_capacity + 3) / 4) : 0;
   if (token_blocks + pad_blocks == 0) return MI355_OK;
   const dim3 grid((unsigned)(token_blocks + pad_blocks));
+  // Rows that the 256 MiB memory-side cache can hold are written with plain stores and wait
+  // there for the kernel that reads them (6.5 against 5.5 TB/s with non-temporal stores at
+  // exactly 256 MiB); beyond that size they only displace each other, and non-temporal stores
+  // are the faster ones (5.5 against 5.0 TB/s at 512 MiB).
+  const int stream_stores = row_capacity * D * (dtype == MI355_F32 ? 4 : 2) > (256ll << 20);
   if (dtype == MI355_F32)
     hipLaunchKernelGGL(permute_rows_fwd_kernel<float>, grid, dim3(256), 0, as_stream(stream),
                        static_cast<const float*>(x), row_of_slot, slot_of_row, total_rows,
-                       static_cast<float*>(rows), (int)T, (int)D, (int)K, token_blocks, (int)row_capacity);
+                       static_cast<float*>(rows), (int)T, (int)D, (int)K, token_blocks, (int)row_capacity, stream_stores);
   else if (dtype == MI355_BF16)
     hipLaunchKernelGGL(permute_rows_fwd_kernel<uint16_t>, grid, dim3(256), 0, as_stream(stream),
                        static_cast<const uint16_t*>(x), row_of_slot, slot_of_row, total_rows,
-                       static_cast<uint16_t*>(rows), (int)T, (int)D, (int)K, token_blocks, (int)row_capacity);
+                       static_cast<uint16_t*>(rows), (int)T, (int)D, (int)K, token_blocks, (int)row_capacity, stream_stores);
   else
     return fail(MI355_EINVAL, "permute_rows_fwd: unknown dtype %d", dtype);
   return check_launch("permute_rows_fwd");
