@@ -75,6 +75,30 @@ def time_events(fn, iters, warmup=2):
     return start.elapsed_time(stop) / iters
 
 
+def time_sequence(fns, iters, warmup=2):
+    """Average milliseconds of each launch in ``fns`` (name -> callable), launched round after
+    round in the given order -- the order of a training step -- with HIP events around every
+    launch.  A kernel timed back to back with itself runs under a different power and cache
+    state than in the step (the matrix-core kernels measure up to a fifth slower that way on
+    this card); timed in sequence, the averages agree with a profiler's view of the step."""
+    import torch
+
+    for _ in range(warmup):
+        for fn in fns.values():
+            fn()
+    events = {name: [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+                     for _ in range(iters)] for name in fns}
+    torch.cuda.synchronize()
+    for i in range(iters):
+        for name, fn in fns.items():
+            start, stop = events[name][i]
+            start.record()
+            fn()
+            stop.record()
+    torch.cuda.synchronize()
+    return {name: sum(a.elapsed_time(b) for a, b in pairs) / iters for name, pairs in events.items()}
+
+
 def sustained_mfma(dev):
     """What the matrix cores hold on the two MFMA shapes the grouped GEMMs use, with
     register-resident operands of random bits (bench_probe/libmi355probe.so): rate and core
@@ -233,51 +257,23 @@ def per_kernel_times(args, wl, block, x, gout, dev):
                 else:
                     ops.grouped_swiglu_stage(s, buf, plan)
 
-            stage_ms = {s: time_events(lambda s=s: run_stage(s), it) for s in stage_flops}
+            stage_fns = {s: (lambda s=s: run_stage(s)) for s in stage_flops}
             drows = buf["drows"]
         else:
             # fp32 / odd shapes: the generic kernels, timed per call (forward: gate, up, SwiGLU, down;
             # backward: dh, SwiGLU', drows, three weight gradients)
             stage_flops = {"experts_fwd": 3 * proj}
-            stage_ms["experts_fwd"] = time_events(lambda: ops.grouped_swiglu_fwd(rows, w1, w3, w2, plan), it)
+            stage_fns = {"experts_fwd": lambda: ops.grouped_swiglu_fwd(rows, w1, w3, w2, plan)}
             if wl.backward:
                 stage_flops["experts_bwd"] = 6 * proj
-                stage_ms["experts_bwd"] = time_events(
-                    lambda: ops.grouped_swiglu_bwd(dy, rows, w1, w3, w2, gate, up, h, plan), it)
+                stage_fns["experts_bwd"] = lambda: ops.grouped_swiglu_bwd(dy, rows, w1, w3, w2, gate, up, h, plan)
             drows = torch.empty_like(rows)
         gw, gb = block.router.gate.weight, block.router.gate.bias
         sel = lambda: ops.router_select_fwd(logits, block.expert_bias_E, K, wl.score_func, wl.route_norm,
                                             wl.route_scale, wl.num_expert_groups or 0, wl.num_limited_groups or 0,
                                             want_map=True)
         lo, hi = wl.local_experts or (0, E)
-        other_ms = {
-            "router_gate_fwd": time_events(lambda: ops.router_gate_fwd(x, gw, gb), it),
-            "router_select_fwd": time_events(sel, it),
-            "permute_plan": time_events(lambda: ops.permute_plan(ids, E, lo, hi, wl.pad_multiple or 1), it),
-            "permute_rows_fwd": time_events(lambda: ops.permute_rows_fwd(x, plan), it),
-            "combine_fwd": time_events(lambda: ops.combine_fwd(y, scores, plan), it),
-        }
-        in_step = {"router_gate_fwd", "router_select_fwd", "permute_plan", "combine_fwd"}
-        if not folded:
-            in_step.add("permute_rows_fwd")
-        if wl.backward:
-            other_ms.update({
-                "combine_bwd": time_events(lambda: ops.combine_bwd(gout, y, scores, plan), it),
-                "permute_rows_bwd": time_events(lambda: ops.permute_rows_bwd(drows, plan), it),
-                "router_gate_bwd": time_events(lambda: ops.router_gate_bwd(logits, x, gw), it),
-                "router_select_bwd": time_events(
-                    lambda: ops.router_select_bwd(logits, ids, scores, None, wl.score_func, wl.route_norm,
-                                                  wl.route_scale), it),
-            })
-            in_step |= {"permute_rows_bwd", "router_gate_bwd", "router_select_bwd"}
-            if folded:
-                other_ms["combine_row_scale"] = time_events(lambda: ops.combine_row_scale(scores, plan), it)
-                other_ms["combine_scores_bwd"] = time_events(
-                    lambda: ops.combine_scores_bwd(buf["dot_partial"], plan), it)
-                in_step |= {"combine_row_scale", "combine_scores_bwd"}
-            else:
-                in_step.add("combine_bwd")
-        shared_ms, shared_flops = {}, {}
+        shared_fns, shared_flops = {}, {}
         if wl.shared_hidden_dim and ops.gather_supported(x, wl.shared_hidden_dim):
             # the shared expert: a dense SwiGLU over all tokens on the same kernels (one segment)
             sh = block.shared_experts
@@ -293,7 +289,43 @@ def per_kernel_times(args, wl, block, x, gout, dev):
                             "dw1": sproj, "dw3": sproj}
             if not wl.backward:
                 shared_flops = {k: shared_flops[k] for k in ("gate_up", "down")}
-            shared_ms = {s: time_events(lambda s=s: ops.grouped_swiglu_stage(s, sbuf, sp), it) for s in shared_flops}
+            shared_fns = {s: (lambda s=s: ops.grouped_swiglu_stage(s, sbuf, sp)) for s in shared_flops}
+        # ---- the launches of one step, in the step's order
+        fwd_stages = [s for s in stage_fns if s in ("gate_up", "down", "experts_fwd")]
+        bwd_stages = [s for s in stage_fns if s not in fwd_stages]
+        seq = {"router_gate_fwd": lambda: ops.router_gate_fwd(x, gw, gb), "router_select_fwd": sel,
+               "permute_plan": lambda: ops.permute_plan(ids, E, lo, hi, wl.pad_multiple or 1)}
+        if not folded:
+            seq["permute_rows_fwd"] = lambda: ops.permute_rows_fwd(x, plan)
+        seq.update({f"grouped_{s}": stage_fns[s] for s in fwd_stages})
+        seq["combine_fwd"] = lambda: ops.combine_fwd(y, scores, plan)
+        seq.update({f"shared_{s}": shared_fns[s] for s in shared_fns if s in ("gate_up", "down")})
+        if wl.backward:
+            seq.update({f"shared_{s}": shared_fns[s] for s in shared_fns if s not in ("gate_up", "down")})
+            if folded:
+                seq["combine_row_scale"] = lambda: ops.combine_row_scale(scores, plan)
+                order = [s for s in ("dh", "drows") if s in bwd_stages]
+                seq.update({f"grouped_{s}": stage_fns[s] for s in order})
+                seq["permute_rows_bwd"] = lambda: ops.permute_rows_bwd(drows, plan)
+                seq["combine_scores_bwd"] = lambda: ops.combine_scores_bwd(buf["dot_partial"], plan)
+                seq.update({f"grouped_{s}": stage_fns[s] for s in bwd_stages if s not in order})
+            else:
+                seq["combine_bwd"] = lambda: ops.combine_bwd(gout, y, scores, plan)
+                seq.update({f"grouped_{s}": stage_fns[s] for s in bwd_stages})
+                seq["permute_rows_bwd"] = lambda: ops.permute_rows_bwd(drows, plan)
+            seq["router_select_bwd"] = lambda: ops.router_select_bwd(logits, ids, scores, None, wl.score_func,
+                                                                     wl.route_norm, wl.route_scale)
+            seq["router_gate_bwd"] = lambda: ops.router_gate_bwd(logits, x, gw)
+        seq_ms = time_sequence(seq, it)
+        stage_ms = {s: seq_ms[f"grouped_{s}"] for s in stage_fns}
+        shared_ms = {s: seq_ms[f"shared_{s}"] for s in shared_fns}
+        in_step = {k for k in seq if not k.startswith(("grouped_", "shared_"))}
+        other_ms = {k: seq_ms[k] for k in in_step}
+        # the public dispatcher API's movers, which the fused step does not launch
+        if "permute_rows_fwd" not in other_ms:
+            other_ms["permute_rows_fwd"] = time_events(lambda: ops.permute_rows_fwd(x, plan), it)
+        if wl.backward and "combine_bwd" not in other_ms:
+            other_ms["combine_bwd"] = time_events(lambda: ops.combine_bwd(gout, y, scores, plan), it)
         # the callers' side of the path, outside the timed step: the decoder layer's norm in
         # front of the block and the statistics of a quantile-balanced router
         outside_ms = {}

@@ -37,8 +37,9 @@
 // stage, refills those registers with the step after, and issues its MFMAs.  The
 // pipeline tail is peeled at compile time: every load of the steady state is
 // unconditional, so the compiler counts outstanding loads exactly instead of draining
-// the queue once per K step.  Operand addresses are a wave-uniform 64-bit base plus a
-// fixed 32-bit per-thread offset.
+// the queue once per K step.  Operands are fetched with buffer loads: a wave-uniform
+// resource (the tile's origin), a fixed 32-bit per-thread offset and a scalar K offset,
+// so no per-thread 64-bit address arithmetic or address registers sit in the loop.
 //
 // MFMA of the row-tiled kernels: v_mfma_f32_16x16x32_bf16.  Per lane 8 bf16 of each operand (row lane%16,
 // k = 8*(lane/16)..+7), 4 fp32 of the result (column lane%16, rows 4*(lane/16) + i).
@@ -65,6 +66,12 @@ constexpr int NT = 512;  // threads per workgroup
 // use is rounded to bf16 right after)
 __device__ __forceinline__ float fast_sigmoid(float x) {
   return __builtin_amdgcn_rcpf(1.0f + __expf(-x));
+}
+
+// Raw buffer resource over `base` (wave-uniform): byte offsets up to 4 GiB, no stride, no
+// swizzle; loads through it take a 32-bit per-thread offset and a scalar offset.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, -1, 0x00020000);
 }
 
 // int32 data that no kernel of this file writes (the plan's arrays), for uniform lookups
@@ -219,9 +226,10 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
       bcol[nj] = wn * (32 * NJ) + nj * 16;
   }
 
-  // Operand addresses are a wave-uniform 64-bit base (tile, K step, chunk index) plus a
-  // 32-bit per-thread byte offset, the form global loads take without any 64-bit vector
-  // arithmetic.  The B offsets never change; the A offsets follow the tile's rows.
+  // Operand addresses are a wave-uniform buffer resource (the tile's origin) plus a fixed 32-bit
+  // per-thread byte offset plus a scalar offset (K step, chunk round): the form buffer loads take
+  // without any per-thread 64-bit arithmetic or address registers.  The B offsets never change;
+  // the A offsets follow the tile's rows.
   constexpr bool B_REGULAR = !B_KS || (NT % (BNT / 8) == 0);  // chunk index -> fixed row stride
   constexpr int NBV = B_REGULAR ? 1 : NB;
   const int ldb = B_KS ? Ncols : (MODE == RM_GATEUP ? D : F);
@@ -237,10 +245,8 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
     }
   }
   // state of the tile whose operands are being fetched
-  const char* ubA0;  // A rows (k = 0)
-  const char* ubA1;  // DX: second half of the contraction (dup)
-  const char* ubB0;  // B tile origin in the first weight stack
-  int64_t b1_bytes;  // second weight stack - first (one flat address space)
+  __amdgpu_buffer_rsrc_t rsA0, rsA1;  // A rows (k = 0); DX: second half of the contraction (dup)
+  __amdgpu_buffer_rsrc_t rsB0, rsB1;  // B tile origin in the first / second weight stack
   uint32_t voffA[NA];
   // source rows of the A tile: the tile's own rows, or token rows through the gather index
   auto load_asrc = [&](const TileMeta& m, int (&asrc)[NA]) {
@@ -252,38 +258,41 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
   };
   auto setup = [&](const TileMeta& m, const int (&asrc)[NA]) {
     const int64_t arow = GATHER ? 0 : static_cast<int64_t>(m.row0) * lda;
-    ubA0 = reinterpret_cast<const char*>(p.a0 + arow);
-    ubA1 = (MODE == RM_DX) ? reinterpret_cast<const char*>(p.a1 + arow) : ubA0;
+    rsA0 = make_rsrc(p.a0 + arow);
+    rsA1 = (MODE == RM_DX) ? make_rsrc(p.a1 + arow) : rsA0;
 #pragma unroll
     for (int i = 0; i < NA; ++i)
       voffA[i] = (static_cast<uint32_t>(asrc[i]) * static_cast<uint32_t>(lda) + static_cast<uint32_t>(kc_chunk * 8)) * 2u;
     const uint16_t* B0 = p.b0 + m.e * wsz;
     const uint16_t* B1 = (MODE == RM_GATEUP || MODE == RM_DX) ? p.b1 + m.e * wsz : B0;
-    b1_bytes = (B1 - B0) * 2;
     // KC: the tile's first weight row is n0; KS: its first column is n0
-    ubB0 = reinterpret_cast<const char*>(B0 + (B_KS ? static_cast<int64_t>(m.n0) : static_cast<int64_t>(m.n0) * ldb));
+    const int64_t borg = B_KS ? static_cast<int64_t>(m.n0) : static_cast<int64_t>(m.n0) * ldb;
+    rsB0 = make_rsrc(B0 + borg);
+    rsB1 = make_rsrc(B1 + borg);
   };
   // chunk i of the A / B tile of the K step that starts at k0
   auto load_a = [&](int k0, int i) -> u32x4 {
-    const char* base = ubA0 + static_cast<int64_t>(k0) * 2;
-    if constexpr (MODE == RM_DX) base = (k0 >= F ? ubA1 + static_cast<int64_t>(k0 - F) * 2 : base);
-    return *reinterpret_cast<const u32x4*>(base + voffA[i]);
+    if constexpr (MODE == RM_DX) {
+      if (k0 >= F) return __builtin_amdgcn_raw_buffer_load_b128(rsA1, voffA[i], (k0 - F) * 2, 0);
+    }
+    return __builtin_amdgcn_raw_buffer_load_b128(rsA0, voffA[i], k0 * 2, 0);
   };
   auto load_b = [&](int k0, int i) -> u32x4 {
-    const char* base = ubB0;
     if constexpr (MODE == RM_GATEUP) {
       // rows 0..BNT/2 of the tile come from w1, the rest from w3, same f range
-      base += (i >= NB / 2 ? b1_bytes : 0) + (static_cast<int64_t>(64 * (i % (NB / 2))) * ldb + k0) * 2;
+      const int so = (64 * (i % (NB / 2)) * ldb + k0) * 2;
+      return __builtin_amdgcn_raw_buffer_load_b128(i >= NB / 2 ? rsB1 : rsB0, voffB[0], so, 0);
     } else if constexpr (MODE == RM_DOWN) {
-      base += (static_cast<int64_t>(64 * i) * ldb + k0) * 2;
+      return __builtin_amdgcn_raw_buffer_load_b128(rsB0, voffB[0], (64 * i * ldb + k0) * 2, 0);
     } else {
       int kk0 = k0;
+      bool second = false;
       if constexpr (MODE == RM_DX) {
-        if (k0 >= F) { kk0 = k0 - F; base += b1_bytes; }
+        if (k0 >= F) { kk0 = k0 - F; second = true; }
       }
-      base += static_cast<int64_t>(kk0 + (B_REGULAR ? i * (NT / (BNT / 8)) : 0)) * ldb * 2;
+      const int so = (kk0 + (B_REGULAR ? i * (NT / (BNT / 8)) : 0)) * ldb * 2;
+      return __builtin_amdgcn_raw_buffer_load_b128(second ? rsB1 : rsB0, voffB[B_REGULAR ? 0 : i], so, 0);
     }
-    return *reinterpret_cast<const u32x4*>(base + voffB[B_REGULAR ? 0 : i]);
   };
   auto kofs = [&](int ks) { return ks * BK; };
   // request every chunk of K step `step` of the fetch tile
