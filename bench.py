@@ -53,6 +53,10 @@ def parse():
     ap.add_argument("--stage-iters", type=int, default=10)
     ap.add_argument("--no-probe", action="store_true",
                     help="skip the sustained-MFMA probe (about 0.8 s of matrix-core work) and the vendor GEMM")
+    ap.add_argument("--power", action="store_true",
+                    help="also loop each grouped GEMM, the whole step, the vendor GEMM, the MFMA probe and a copy for "
+                         "--power-seconds each while sampling the card's power sensor (hwmon); adds a \"power\" object")
+    ap.add_argument("--power-seconds", type=float, default=2.5)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (known traffic, for scaling rocprof FETCH_SIZE / WRITE_SIZE)")
     return ap.parse_args()
@@ -99,10 +103,9 @@ def time_sequence(fns, iters, warmup=2):
     return {name: sum(a.elapsed_time(b) for a, b in pairs) / iters for name, pairs in events.items()}
 
 
-def sustained_mfma(dev):
-    """What the matrix cores hold on the two MFMA shapes the grouped GEMMs use, with
-    register-resident operands of random bits (bench_probe/libmi355probe.so): rate and core
-    clock, both under the card's own power management.  None when the probe is not built."""
+def mfma_probe(dev):
+    """(launch(shape, random_bits, iters), blocks, clocks) over bench_probe/libmi355probe.so, or
+    None when the probe is not built.  shape 1 = 16x16x32, 0 = 32x32x16."""
     import ctypes
 
     import torch
@@ -117,21 +120,91 @@ def sustained_mfma(dev):
     blocks = 4 * torch.cuda.get_device_properties(dev).multi_processor_count
     sink = torch.zeros(1, dtype=torch.float32, device=dev)
     clocks = torch.zeros(2 * blocks, dtype=torch.int64, device=dev)
+
+    def launch(shape, rnd, iters):
+        rc = lib.mi355_probe_mfma(sink.data_ptr(), clocks.data_ptr(), blocks, iters, rnd, shape,
+                                  torch.cuda.current_stream().cuda_stream)
+        assert rc == 0
+
+    return launch, blocks, clocks
+
+
+def sustained_mfma(dev):
+    """What the matrix cores hold on the two MFMA shapes the grouped GEMMs use, with
+    register-resident operands of random bits (bench_probe/libmi355probe.so): rate and core
+    clock, both under the card's own power management.  None when the probe is not built."""
+    probe = mfma_probe(dev)
+    if probe is None:
+        return None
+    run, blocks, clocks = probe
     out = {}
     # 16x16x32 is the shape of the row-tiled grouped GEMMs, 32x32x16 that of the weight gradients
     for shape, name, iters in ((1, "16x16x32", 50000), (0, "32x32x16", 100000)):
         out[name] = {}
         for label, rnd in (("random_bits", 1), ("constant_bits", 0)):
-            def launch():
-                rc = lib.mi355_probe_mfma(sink.data_ptr(), clocks.data_ptr(), blocks, iters, rnd, shape,
-                                          torch.cuda.current_stream().cuda_stream)
-                assert rc == 0
-            ms = time_events(launch, 2, warmup=1)
+            ms = time_events(lambda: run(shape, rnd, iters), 2, warmup=1)
             flops = blocks * 8.0 * iters * 262144 * (shape + 1)
             c = clocks.view(blocks, 2).double()
             out[name][label] = {"TFLOP/s": round(flops / (ms * 1e-3) / 1e12, 1),
                                 "core_clock_mhz": round(float((c[:, 0] / c[:, 1]).mean()) * 100.0, 0)}
     return out
+
+
+def power_table(cases, seconds):
+    """Average socket power (W) while each callable of ``cases`` runs in a loop for ``seconds``,
+    read from the amdgpu hwmon sensor every 20 ms (the first 0.8 s of each loop are dropped: the
+    sensor averages).  ``None`` in ``cases`` means idle.  Returns None when no sensor is readable."""
+    import glob
+    import threading
+
+    import torch
+
+    def read(path):
+        try:
+            return int(open(path).read().strip())
+        except (OSError, ValueError):
+            return None
+
+    sensor = cap = None
+    for h in sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*")):
+        for name in ("power1_average", "power1_input"):
+            if read(os.path.join(h, name)) is not None:
+                sensor, cap = os.path.join(h, name), read(os.path.join(h, "power1_cap"))
+                break
+        if sensor:
+            break
+    if sensor is None:
+        return None
+
+    def sample(stop, out):
+        while not stop.is_set():
+            v = read(sensor)
+            if v is not None:
+                out.append((time.time(), v / 1e6))
+            time.sleep(0.02)
+
+    table = {}
+    for name, fn in cases.items():
+        out, stop = [], threading.Event()
+        th = threading.Thread(target=sample, args=(stop, out))
+        th.start()
+        t0, n = time.time(), 0
+        if fn is None:
+            time.sleep(min(seconds, 1.5))
+        else:
+            while time.time() - t0 < seconds:
+                for _ in range(20):
+                    fn()
+                torch.cuda.synchronize()
+                n += 20
+        dt = time.time() - t0
+        stop.set()
+        th.join()
+        watts = [w for t, w in out if t - t0 > 0.8] or [w for _, w in out]
+        table[name] = {"watts": round(sum(watts) / max(len(watts), 1), 1)}
+        if n:
+            table[name]["ms_per_call_looped"] = round(dt / n * 1e3, 4)
+    return {"sensor": sensor, "cap_watts": None if cap is None else cap / 1e6, "cases": table}
 
 
 def cpu_baseline(wl, sample_tokens):
@@ -367,7 +440,7 @@ def per_kernel_times(args, wl, block, x, gout, dev):
             gbs = other_bytes[s] / (ms * 1e-3) / 1e9
             ent.update({"GB/s": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4)})
         kernels[s] = ent
-    return kernels, stage_ms, stage_flops, shared_ms, shared_flops, R_rows, folded
+    return kernels, stage_ms, stage_flops, shared_ms, shared_flops, R_rows, folded, stage_fns
 
 
 def main():
@@ -410,7 +483,7 @@ def main():
     tokens_per_s = T * args.steps / dt
 
     x2, g2 = x.reshape(-1, wl.dim), gout.reshape(-1, wl.dim)
-    kernels, stage_ms, stage_flops, shared_ms, shared_flops, R_rows, folded = per_kernel_times(
+    kernels, stage_ms, stage_flops, shared_ms, shared_flops, R_rows, folded, stage_fns = per_kernel_times(
         args, wl, block, x2, g2, dev)
     peak = PEAK_BF16_TFLOPS if wl.dtype == torch.bfloat16 else PEAK_FP32_TFLOPS
 
@@ -500,6 +573,36 @@ def main():
         "roofline": roofline,
         "kernels": kernels,
     }
+    if args.power:
+        cases = {"idle": None}
+        cases.update({f"grouped_{s}": fn for s, fn in stage_fns.items()})
+        cases["whole_step"] = step
+        if wl.dtype == torch.bfloat16:
+            a = torch.randn(max(R_rows, 1), wl.dim, device=dev).bfloat16()
+            b = torch.randn(2 * wl.hidden_dim, wl.dim, device=dev).bfloat16()
+            cases["vendor_dense_gemm"] = lambda: torch.mm(a, b.t())
+            pl = mfma_probe(dev)
+            if pl is not None:
+                # operands in registers: matrix cores alone, with random and with constant operand bits
+                cases["mfma_probe_16x16x32_random_bits"] = lambda: pl[0](1, 1, 2000)
+                cases["mfma_probe_16x16x32_constant_bits"] = lambda: pl[0](1, 0, 2000)
+        big = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        big2 = torch.empty_like(big)
+        cases["copy_1GiB"] = lambda: big2.copy_(big)
+        result["power"] = power_table(cases, args.power_seconds)
+        if result["power"] is not None:
+            for name, ent in result["power"]["cases"].items():
+                key = name[len("grouped_"):]
+                if key in stage_flops and "ms_per_call_looped" in ent:
+                    ent["TFLOP/s_looped"] = round(stage_flops[key] / (ent["ms_per_call_looped"] * 1e-3) / 1e12, 1)
+            if "vendor_dense_gemm" in result["power"]["cases"]:
+                ent = result["power"]["cases"]["vendor_dense_gemm"]
+                ent["TFLOP/s_looped"] = round(2.0 * a.shape[0] * b.shape[0] * wl.dim / (ent["ms_per_call_looped"] * 1e-3) / 1e12, 1)
+            for name, ent in result["power"]["cases"].items():
+                if name.startswith("mfma_probe"):
+                    ent["TFLOP/s_looped"] = round(pl[1] * 8.0 * 2000 * 262144 * 2 / (ent["ms_per_call_looped"] * 1e-3) / 1e12, 1)
+            ent = result["power"]["cases"]["copy_1GiB"]
+            ent["GB/s_looped"] = round(2.0 * (1 << 30) / (ent["ms_per_call_looped"] * 1e-3) / 1e9, 1)
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)
