@@ -29,7 +29,7 @@ def test_library_loads_and_exports_every_declared_symbol():
         assert name in _lib.SIGNATURES, f"{name} has no ctypes prototype"
     assert set(_lib.SIGNATURES) == set(names)
     assert lib.mi355_moe_abi_version() == _lib.ABI_VERSION == 2
-    assert lib.mi355_grouped_tile_m(1) in (128, 256)  # 256 unless MI355_ROW_LAYOUT=wide
+    assert lib.mi355_grouped_tile_m(1) == 256 and lib.mi355_grouped_tile_m(0) == 256
 
 
 def test_argument_validation_reports_errors_without_a_gpu():

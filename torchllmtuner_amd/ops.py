@@ -27,7 +27,8 @@ _O = torch.ops.mi355_moe
 _DT = {torch.float32: 0, torch.bfloat16: 1}
 SCORE_FUNCS = {"sigmoid": 0, "softmax": 1, "sqrtsoftplus": 2}
 SELECT_TOPK, SELECT_FIXED, SELECT_BALANCED = 0, 1, 2
-TILE_M = 256  # rows per entry of a plan's tile list (mi355_grouped_tile_m)
+# most rows an entry of a plan's tile list covers: the library's row-tile height
+TILE_M = int(_lib.load().mi355_grouped_tile_m(_DT[torch.bfloat16]))
 
 
 def _dt(t: torch.Tensor) -> int:
