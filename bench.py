@@ -324,6 +324,10 @@ def per_kernel_times(args, wl, block, x, gout, dev):
                        dot_partial=torch.empty(rows.shape[0], ops.combine_bwd_slots(x.dtype, D, F),
                                                dtype=torch.float32, device=dev))
 
+            if not wl.backward:
+                # as in a step without gradients: gate and up are not written
+                buf["gate"] = buf["up"] = None
+
             def run_stage(s):
                 if s in ("dh", "dw2"):
                     ops.grouped_swiglu_combine_stage(s, buf, plan)

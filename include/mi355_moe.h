@@ -341,7 +341,10 @@ int mi355_combine_bwd(const void* dout, const void* y, int dtype,
  * never out of bounds), and the call returns MI355_EINVAL without launching when
  * token_of_row is given with T < 1 or with T*D*2 >= 2^32 bytes (the gather addresses its
  * source with 32-bit byte offsets).  Ignored when token_of_row is NULL.
- * gate/up/h are saved for the backward (each (row_capacity,F)).
+ * gate/up/h are saved for the backward (each (row_capacity,F)).  A caller that will never
+ * run the backward may pass gate = up = NULL (both): for bf16 with D and F multiples of 64
+ * (>= 384) those two outputs are then not written at all; for any other dtype or shape
+ * that is MI355_EINVAL (the other paths use the buffers as intermediates).
  * The kernels walk the plan's tile list in tiles of mi355_grouped_tile_m(dtype) rows
  * (256), so the list must have been built with that value.
  */

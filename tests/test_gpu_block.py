@@ -209,6 +209,25 @@ def test_bf16_block_with_no_or_few_tokens(T):
         assert err < 2e-2, f"{k}: rel-L2 {err}"
 
 
+def test_forward_without_gradients_skips_gate_and_up_and_returns_the_same_bits():
+    """Under no_grad the fused forward does not write gate and up (nobody will read them); the
+    block's output must not change by a bit, and a differentiated forward right after still works."""
+    print("block forward only", flush=True)
+    T, D, E, K, F = 700, 512, 16, 4, 384
+    spec = R.RouterSpec(E, K, score_func="softmax", route_norm=True)
+    p = make_params(E, D, F, torch.bfloat16, seed=21)
+    block = build_block(p, spec, D, F, torch.bfloat16, DEV)
+    x = torch.randn(T, D, generator=torch.Generator().manual_seed(22)).bfloat16().to(DEV)
+    block.eval()
+    with torch.no_grad():
+        plain = block(x)
+    xin = x.clone().requires_grad_()
+    tracked = block(xin)
+    assert torch.equal(plain, tracked)
+    tracked.float().sum().backward()
+    assert torch.isfinite(xin.grad.float()).all() and float(xin.grad.float().abs().sum()) > 0
+
+
 def test_dispatcher_api_matches_reference_contract():
     """dispatch/combine through the public dispatcher classes, analytic expectation
     out = x * 2 * sum(scores) (tests/unit_tests/cpu/models/test_moe_token_dispatch.py:249-309)."""

@@ -74,6 +74,11 @@ def test_gather_entry_points_reject_unaddressable_token_matrices_without_launchi
     # fp32 rows cannot be gathered at all
     rc = lib.mi355_grouped_swiglu_fwd(p, p, 8, p, p, p, 0, p, p, p, p, p, tiles, p, p, p, p, El, D, F, R, None)
     assert rc == -1 and b"bf16 only" in lib.mi355_moe_last_error()
+    # gate and up are omitted together or not at all, and only where the bf16 MFMA path runs
+    rc = lib.mi355_grouped_swiglu_fwd(p, None, 8, p, p, p, 1, p, p, p, p, p, tiles, None, p, p, p, El, D, F, R, None)
+    assert rc == -1 and b"together" in lib.mi355_moe_last_error()
+    rc = lib.mi355_grouped_swiglu_fwd(p, None, 8, p, p, p, 0, p, p, p, p, p, tiles, None, None, p, p, El, D, F, R, None)
+    assert rc == -1 and b"can only be omitted" in lib.mi355_moe_last_error()
     # the allocation-free plan refuses what its built-in scratch cannot hold
     assert lib.mi355_permute_plan_static_max_bytes() == 8 << 20
     rc = lib.mi355_permute_plan_static(p, 1 << 20, 8, 128, 0, 128, 1, 256, p, p, p, p, p, p, 1 << 23, p, p, p,

@@ -79,12 +79,14 @@ def test_every_operator_is_registered_with_a_fake_kernel_and_propagates_shapes()
             "grouped_swiglu_bwd": (O.grouped_swiglu_bwd(rows, rows, None, w1, w3, w2, rf, rf, rf, *seg, True, True, False),
                                    [((N, D), BF), ((El, F, D), BF), ((El, F, D), BF), ((El, D, F), BF)]),
             "gather_experts_combine_fwd": (
-                O.gather_experts_combine_fwd(x, wts, w1, w3, w2, tok, sor, ros, *seg, K, N, True),
+                O.gather_experts_combine_fwd(x, wts, w1, w3, w2, tok, sor, ros, *seg, K, N, True, True),
                 [((T, D), BF), ((N, F), BF), ((N, F), BF)]),
             "gather_experts_combine_bwd": (
                 O.gather_experts_combine_bwd(x, x, wts, w1, w3, w2, rf, rf, tok, sor, ros, *seg, K, True, True),
                 [((T, D), BF), ((El, F, D), BF), ((El, F, D), BF), ((El, D, F), BF), ((T, K), F32)]),
         }
+        fwd_only = O.gather_experts_combine_fwd(x, wts, w1, w3, w2, tok, sor, ros, *seg, K, N, True, False)
+        assert [tuple(t.shape) for t in fwd_only] == [(T, D), (0, F), (0, F)]
         assert O.quantile_observe(_fake((E, 100), I64), logits, _fake((T,)), _fake((E,)), None) is None
         seen.add("quantile_observe")
         for name, (out, want) in cases.items():

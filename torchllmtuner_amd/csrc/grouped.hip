@@ -147,10 +147,16 @@ extern "C" int mi355_grouped_swiglu_fwd(const void* rows, const int32_t* token_o
   if (int rc = check_gather("grouped_swiglu_fwd", row_capacity > 0 ? token_of_row : nullptr, num_tokens, D, dtype)) return rc;
   if (row_capacity == 0 || tile_capacity == 0) return MI355_OK;
   MI355_REQUIRE(rows && w1 && w3 && w2 && seg_offsets && seg_counts && tile_expert && tile_row0 &&
-                    num_tiles && gate && up && h && y,
+                    num_tiles && h && y,
                 "grouped_swiglu_fwd: null pointer");
+  // gate and up may both be null (nobody will run the backward): the bf16 MFMA path then skips
+  // those two output streams; the other paths use them as their own intermediates
+  MI355_REQUIRE((gate == nullptr) == (up == nullptr), "grouped_swiglu_fwd: gate and up must be given or omitted together");
+  const bool fast = dtype == MI355_BF16 && bf16_fast_path_ok(D, F);
+  MI355_REQUIRE(gate != nullptr || fast,
+                "grouped_swiglu_fwd: gate and up can only be omitted for bf16 with D and F multiples of 64 (>= 384)");
   hipStream_t s = as_stream(stream);
-  if (dtype == MI355_BF16 && bf16_fast_path_ok(D, F))
+  if (fast)
     return bf16_grouped_fwd(rows, token_of_row, num_tokens, w1, w3, w2, seg_offsets, seg_counts, tile_expert,
                             tile_row0, num_tiles, tile_capacity, gate, up, h, y, D, F, 3, s);
   if (token_of_row)

@@ -123,7 +123,9 @@ __device__ __forceinline__ float row16_sum(float v) {
   return v;
 }
 
-template <int MODE, int NJ, bool GATHER, int WM>
+// SAVE_GU (GATEUP only): also write gate and up, which the backward reads; a forward-only caller
+// leaves them out -- a third of the kernel's output bytes and of its epilogue's LDS traffic.
+template <int MODE, int NJ, bool GATHER, int WM, bool SAVE_GU = true>
 __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
   constexpr int WN = 8 / WM;               // waves along the columns (WM along the rows)
   constexpr int TBM = 64 * WM;             // rows of the tile
@@ -416,8 +418,9 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
   uint16_t* st = smem + wave * (64 * 136);  // 8 waves x 17 KiB < 160 KiB; the barrier ending the K loop freed the tiles
   if constexpr (MODE == RM_GATEUP) {
     // per 32-row half: three 32 x 64 tiles gate | up | h at columns 0, 64, 128 of a
-    // [32][192+8] region (12.5 KiB per wave)
-    using S = WaveStage<192>;
+    // [32][192+8] region (12.5 KiB per wave); without gate and up, h alone in a [32][64+8] region
+    constexpr int NT3 = SAVE_GU ? 3 : 1;       // output tiles per row
+    using S = WaveStage<64 * NT3>;
     uint16_t* sg = smem + wave * (32 * S::PITCH);
     const int f0 = n0 + wn * 64;
 #pragma unroll
@@ -436,22 +439,24 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
             const float s = round_bf16(g[r] * fast_sigmoid(g[r]));
             h[r] = s * u[r];
           }
-          S::put16(sg, ml, j * 16, lane, g[0], g[1], g[2], g[3]);
-          S::put16(sg, ml, 64 + j * 16, lane, u[0], u[1], u[2], u[3]);
-          S::put16(sg, ml, 128 + j * 16, lane, h[0], h[1], h[2], h[3]);
+          if constexpr (SAVE_GU) {
+            S::put16(sg, ml, j * 16, lane, g[0], g[1], g[2], g[3]);
+            S::put16(sg, ml, 64 + j * 16, lane, u[0], u[1], u[2], u[3]);
+          }
+          S::put16(sg, ml, (SAVE_GU ? 128 : 0) + j * 16, lane, h[0], h[1], h[2], h[3]);
         }
       __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the wave's own LDS writes have landed
       __builtin_amdgcn_wave_barrier();
-      // 32 rows x 3 tiles x 8 chunks = 768 chunks, 12 per lane
+      // 32 rows x NT3 tiles x 8 chunks, 4 NT3 per lane
 #pragma unroll 4
-      for (int it = 0; it < 12; ++it) {
+      for (int it = 0; it < 4 * NT3; ++it) {
         const int idx = it * 64 + lane;
-        const int m = idx / 24, rem = idx % 24, t = rem >> 3, c = rem & 7;
+        const int m = idx / (8 * NT3), rem = idx % (8 * NT3), t = rem >> 3, c = rem & 7;
         const int f = f0 + c * 8;  // < F: tiles never overhang in the columns
         const int mr = wm + half * 32 + m;
         if (mr < valid) {
           const u32x4 v = *reinterpret_cast<const u32x4*>(sg + m * S::PITCH + t * 64 + c * 8);
-          uint16_t* dst = (t == 0 ? p.o0 : (t == 1 ? p.o1 : p.o2)) + static_cast<int64_t>(row0 + mr) * F + f;
+          uint16_t* dst = (!SAVE_GU ? p.o2 : (t == 0 ? p.o0 : (t == 1 ? p.o1 : p.o2))) + static_cast<int64_t>(row0 + mr) * F + f;
           *reinterpret_cast<u32x4*>(dst) = v;
         }
       }
@@ -920,17 +925,17 @@ constexpr int W_LDS_BYTES = 8 * 64 * 136 * 2;  // 139264: the 8 epilogue regions
 // width: output columns; gate/up tiles hold both halves of their column range.  Tiles are always
 // 256 wide (a 192-wide KS tile would not hold the swizzle: 24 chunks per row are not a multiple
 // of the 16 the key permutes); an overhanging last tile shifts back.
-template <int MODE, bool GATHER = false>
+template <int MODE, bool GATHER = false, bool SAVE_GU = true>
 static int launch_row(RowArgs& a, int64_t width, int64_t tile_capacity, hipStream_t s, const char* what) {
   constexpr int div = MODE == RM_GATEUP ? 2 : 1;
   a.n_tiles = (int)((width + 256 / div - 1) / (256 / div));
   static PerDeviceOnce configured;  // one per kernel instantiation
   if (configured.needed()) {
-    if (int rc = set_lds(row_tiled_kernel<MODE, 4, GATHER, 4>, W_LDS_BYTES)) return rc;
+    if (int rc = set_lds(row_tiled_kernel<MODE, 4, GATHER, 4, SAVE_GU>, W_LDS_BYTES)) return rc;
     configured.done();
   }
   const unsigned blocks = std::min(round8(tile_capacity * a.n_tiles), resident_blocks());
-  hipLaunchKernelGGL((row_tiled_kernel<MODE, 4, GATHER, 4>), dim3(blocks), dim3(NT), W_LDS_BYTES, s, a);
+  hipLaunchKernelGGL((row_tiled_kernel<MODE, 4, GATHER, 4, SAVE_GU>), dim3(blocks), dim3(NT), W_LDS_BYTES, s, a);
   return check_launch(what);
 }
 
@@ -946,11 +951,16 @@ int bf16_grouped_fwd(const void* rows, const int32_t* token_of_row, int64_t num_
     a.a0 = (const uint16_t*)rows; a.a_src = token_of_row; a.a_rows = (int)num_tokens;
     a.b0 = (const uint16_t*)w1; a.b1 = (const uint16_t*)w3;
     a.o0 = (uint16_t*)gate; a.o1 = (uint16_t*)up; a.o2 = (uint16_t*)h;
-    if (token_of_row) {
-      if (int rc = launch_row<RM_GATEUP, true>(a, F, tile_capacity, s, "grouped gate/up")) return rc;
-    } else {
-      if (int rc = launch_row<RM_GATEUP>(a, F, tile_capacity, s, "grouped gate/up")) return rc;
-    }
+    // gate == up == null: a forward-only caller; the kernel then writes h alone
+    const bool save = gate != nullptr;
+    int rc;
+    if (token_of_row)
+      rc = save ? launch_row<RM_GATEUP, true>(a, F, tile_capacity, s, "grouped gate/up")
+                : launch_row<RM_GATEUP, true, false>(a, F, tile_capacity, s, "grouped gate/up (h only)");
+    else
+      rc = save ? launch_row<RM_GATEUP>(a, F, tile_capacity, s, "grouped gate/up")
+                : launch_row<RM_GATEUP, false, false>(a, F, tile_capacity, s, "grouped gate/up (h only)");
+    if (rc) return rc;
   }
   if (stages & STAGE_DOWN) {
     RowArgs b = a;

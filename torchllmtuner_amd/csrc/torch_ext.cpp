@@ -440,12 +440,13 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> grouped_swiglu_bwd(
 }
 
 // out[t] = sum_k weights[t,k] * experts(x)[row(t,k)]: gathered expert product, then the combine.
-// Returns (out, gate, up); y and h are dropped (the fused backward recomputes h).
+// Returns (out, gate, up); y and h are dropped (the fused backward recomputes h).  save_gate_up = false
+// (nobody will differentiate): gate and up are not written at all and come back empty.
 std::tuple<Tensor, Tensor, Tensor> gather_experts_combine_fwd(
     const Tensor& x_, const Tensor& weights_, const Tensor& w1_, const Tensor& w3_, const Tensor& w2_,
     const Tensor& token_of_row, const Tensor& slot_of_row, const Tensor& row_of_slot, const Tensor& seg_offsets,
     const Tensor& seg_counts, const Tensor& tile_expert, const Tensor& tile_row0, const Tensor& num_tiles, int64_t K,
-    int64_t row_capacity, bool round_terms) {
+    int64_t row_capacity, bool round_terms, bool save_gate_up) {
   (void)slot_of_row;  // for the backward only (the row -> slot index behind the row scales)
   Launch L(x_);
   const Tensor x = x_.contiguous(), w1 = w1_.contiguous(), w3 = w3_.contiguous(), w2 = w2_.contiguous();
@@ -453,11 +454,13 @@ std::tuple<Tensor, Tensor, Tensor> gather_experts_combine_fwd(
   const Tensor w = cf(weights_);
   const int64_t T = x.size(0), D = x.size(1), El = w1.size(0), F = w1.size(1), R = row_capacity;
   const Plan p = plan_of(seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles);
-  Tensor gate = at::empty({R, F}, x.options()), up = at::empty({R, F}, x.options());
+  const int64_t Rs = save_gate_up ? R : 0;
+  Tensor gate = at::empty({Rs, F}, x.options()), up = at::empty({Rs, F}, x.options());
   Tensor h = at::empty({R, F}, x.options()), y = at::empty({R, D}, x.options());
   check(mi355_grouped_swiglu_fwd(ptr(x), iptr(token_of_row), T, ptr(w1), ptr(w3), ptr(w2), dtype_code(x),
                                  p.seg_offsets, p.seg_counts, p.tile_expert, p.tile_row0, p.num_tiles,
-                                 p.tile_capacity, ptr(gate), ptr(up), ptr(h), ptr(y), El, D, F, R, L.stream),
+                                 p.tile_capacity, save_gate_up ? ptr(gate) : nullptr, save_gate_up ? ptr(up) : nullptr, ptr(h),
+                                 ptr(y), El, D, F, R, L.stream),
         "grouped_swiglu_fwd");
   Tensor out = at::empty({T, D}, x.options());
   check(mi355_combine_fwd(ptr(y), dtype_code(y), fptr(w), iptr(row_of_slot), ptr(out), T, D, K, (int)round_terms,
@@ -569,7 +572,7 @@ TORCH_LIBRARY(mi355_moe, m) {
   m.def(
       "gather_experts_combine_fwd(Tensor x, Tensor weights, Tensor w1, Tensor w3, Tensor w2, Tensor token_of_row, "
       "Tensor slot_of_row, Tensor row_of_slot, Tensor seg_offsets, Tensor seg_counts, Tensor tile_expert, Tensor tile_row0, "
-      "Tensor num_tiles, int top_k, int row_capacity, bool round_terms) -> (Tensor, Tensor, Tensor)");
+      "Tensor num_tiles, int top_k, int row_capacity, bool round_terms, bool save_gate_up) -> (Tensor, Tensor, Tensor)");
   m.def(
       "gather_experts_combine_bwd(Tensor dout, Tensor x, Tensor weights, Tensor w1, Tensor w3, Tensor w2, "
       "Tensor gate, Tensor up, Tensor token_of_row, Tensor slot_of_row, Tensor row_of_slot, Tensor seg_offsets, "

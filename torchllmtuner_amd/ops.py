@@ -215,9 +215,10 @@ def _(dy, rows, token_of_row, w1, w3, w2, gate, up, h, seg_offsets, seg_counts, 
 
 @_fake("gather_experts_combine_fwd")
 def _(x, weights, w1, w3, w2, token_of_row, slot_of_row, row_of_slot, seg_offsets, seg_counts, tile_expert,
-      tile_row0, num_tiles, top_k, row_capacity, round_terms):
+      tile_row0, num_tiles, top_k, row_capacity, round_terms, save_gate_up):
     F = w1.shape[1]
-    return torch.empty_like(x), x.new_empty((row_capacity, F)), x.new_empty((row_capacity, F))
+    rows = row_capacity if save_gate_up else 0
+    return torch.empty_like(x), x.new_empty((rows, F)), x.new_empty((rows, F))
 
 
 @_fake("gather_experts_combine_bwd")
@@ -391,7 +392,9 @@ _autograd("grouped_swiglu_fwd", _gs_backward, _gs_setup)
 
 # -- gathered experts + combine: one backward for both halves
 def _gec_setup(ctx, inputs, output):
-    x, weights, w1, w3, w2, tok, sor, ros, so, sc, te, tr, nt, top_k, _cap, _round = inputs
+    x, weights, w1, w3, w2, tok, sor, ros, so, sc, te, tr, nt, top_k, _cap, _round, saved = inputs
+    if not saved:
+        raise RuntimeError("gather_experts_combine_fwd was run without its gate / up outputs and cannot be differentiated")
     _out, gate, up = output
     ctx.save_for_backward(x, weights, w1, w3, w2, gate, up, tok, sor, ros, so, sc, te, tr, nt)
     ctx.top_k = top_k
@@ -402,12 +405,12 @@ def _gec_backward(ctx, dout, _dgate, _dup):
     x, weights, w1, w3, w2, gate, up, tok, sor, ros, so, sc, te, tr, nt = ctx.saved_tensors
     need = ctx.needs_input_grad
     if dout is None:
-        return (None,) * 16
+        return (None,) * 17
     need_dw = need[2] or need[3] or need[4]
     dx, dw1, dw3, dw2, dweights = _O.gather_experts_combine_bwd(
         dout, x, weights, w1, w3, w2, gate, up, tok, sor, ros, so, sc, te, tr, nt, ctx.top_k, need[0], need_dw)
     return ((dx if need[0] else None), (dweights.to(weights.dtype) if need[1] else None),
-            (dw1 if need[2] else None), (dw3 if need[3] else None), (dw2 if need[4] else None)) + (None,) * 11
+            (dw1 if need[2] else None), (dw3 if need[3] else None), (dw2 if need[4] else None)) + (None,) * 12
 
 
 _autograd("gather_experts_combine_fwd", _gec_backward, _gec_setup)
@@ -715,14 +718,17 @@ def gather_experts_combine(x_TD, weights_TK, w1_EFD, w3_EFD, w2_EDF, plan: Permu
     in its epilogue, where the same pass yields the gradient of the routing weights (the row's
     unscaled dh times its h, summed over the hidden columns); dW2 contracts the gathered
     ``dout`` rows with ``weights * h``.  Nothing of size (R, D) is kept between forward and
-    backward, and of the (R, F) tensors only gate and up."""
+    backward, and of the (R, F) tensors only gate and up -- and when no input asks for a gradient
+    (inference) the forward does not write those two either."""
     _dev(x_TD, weights_TK, w1_EFD, w3_EFD, w2_EDF)
     _check_experts(x_TD, w1_EFD, w3_EFD, w2_EDF, plan)
     if not gather_supported(x_TD, w1_EFD.shape[1]):
         raise ValueError("gather_experts_combine needs bf16 with D and F multiples of 64 (>= 384)")
+    differentiable = torch.is_grad_enabled() and any(
+        t.requires_grad for t in (x_TD, weights_TK, w1_EFD, w3_EFD, w2_EDF))
     out, _gate, _up = _O.gather_experts_combine_fwd(
         x_TD, weights_TK, w1_EFD, w3_EFD, w2_EDF, plan.token_of_row, plan.slot_of_row, plan.row_of_slot,
-        *plan.segments(), plan.top_k, plan.row_capacity, bool(round_terms))
+        *plan.segments(), plan.top_k, plan.row_capacity, bool(round_terms), differentiable)
     return out
 
 
@@ -782,12 +788,13 @@ def grouped_swiglu_stage(stage: str, buf: dict, plan: PermutePlan):
     """Launch exactly one of the seven bf16 MFMA kernels on pre-allocated buffers.
 
     ``buf`` maps the C argument names (dy, rows, w1, w3, w2, gate, up, h, y, dgate,
-    dup, drows, dw1, dw3, dw2) to device tensors.
+    dup, drows, dw1, dw3, dw2) to device tensors; gate and up may be missing for the gate/up
+    stage of a forward-only caller.
     """
     rows = buf["rows"]
     dev = _dev(rows)
     D = rows.shape[1]
-    R = buf["gate"].shape[0]
+    R = buf["h"].shape[0]
     El, F, _ = buf["w1"].shape
     g = lambda k: _p(buf.get(k))
     with torch.cuda.device(dev):
