@@ -57,6 +57,7 @@ def parse():
                     help="also loop each grouped GEMM, the whole step, the vendor GEMM, the MFMA probe and a copy for "
                          "--power-seconds each while sampling the card's power sensor (hwmon); adds a \"power\" object")
     ap.add_argument("--power-seconds", type=float, default=2.5)
+    ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay of the same step")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (known traffic, for scaling rocprof FETCH_SIZE / WRITE_SIZE)")
     return ap.parse_args()
@@ -205,6 +206,46 @@ def power_table(cases, seconds):
         if n:
             table[name]["ms_per_call_looped"] = round(dt / n * 1e3, 4)
     return {"sensor": sensor, "cap_watts": None if cap is None else cap / 1e6, "cases": table}
+
+
+def hip_graph_step(block, x, gout, wl, steps, warmup):
+    """The same step captured once as a HIP graph and replayed ``steps`` times: what a caller
+    gets who removes the host's per-kernel work (about thirty launches per step).  Every kernel
+    of the block is asynchronous, allocates through PyTorch's allocator only and never reads a
+    size back to the host, so the whole forward + backward captures as it is.  Returns
+    ms per step, or a string saying why the capture failed."""
+    import torch
+
+    try:
+        params = [p for p in block.parameters() if p.requires_grad]
+        xin = x.detach().clone().requires_grad_(wl.backward)
+
+        def step():
+            if wl.backward:
+                return torch.autograd.grad(block(xin), [xin] + params, gout)
+            with torch.no_grad():
+                return block(xin)
+
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            keep = step()  # noqa: F841  (the graph's output buffers stay alive with it)
+        for _ in range(warmup):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps * 1e3
+    except Exception as e:  # the eager figure stands on its own
+        return f"{type(e).__name__}: {e}"
 
 
 def cpu_baseline(wl, sample_tokens):
@@ -486,6 +527,8 @@ def main():
     ms_per_step = dt / args.steps * 1e3
     tokens_per_s = T * args.steps / dt
 
+    graph_ms = None if args.no_graph else hip_graph_step(block, x, gout, wl, args.steps, args.warmup)
+
     x2, g2 = x.reshape(-1, wl.dim), gout.reshape(-1, wl.dim)
     kernels, stage_ms, stage_flops, shared_ms, shared_flops, R_rows, folded, stage_fns = per_kernel_times(
         args, wl, block, x2, g2, dev)
@@ -577,6 +620,11 @@ def main():
         "roofline": roofline,
         "kernels": kernels,
     }
+    if isinstance(graph_ms, float):
+        # the same K steps replayed from one captured HIP graph (value / ms_per_step above are the eager calls)
+        result["hip_graph"] = {"ms_per_step": round(graph_ms, 4), "tokens_per_s": round(T / (graph_ms * 1e-3), 1)}
+    elif graph_ms is not None:
+        result["hip_graph"] = {"error": graph_ms[:300]}
     if args.power:
         cases = {"idle": None}
         cases.update({f"grouped_{s}": fn for s, fn in stage_fns.items()})

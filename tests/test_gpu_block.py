@@ -228,6 +228,50 @@ def test_forward_without_gradients_skips_gate_and_up_and_returns_the_same_bits()
     assert torch.isfinite(xin.grad.float()).all() and float(xin.grad.float().abs().sum()) > 0
 
 
+@pytest.mark.parametrize("dtype,D,F,dispatcher", [(torch.float32, 256, 512, "local"), (torch.bfloat16, 512, 384, "local"),
+                                                   (torch.bfloat16, 384, 512, "padded")])
+def test_block_step_replays_from_a_hip_graph(dtype, D, F, dispatcher):
+    """Forward + backward of the block captured once as a HIP graph: no kernel of the path
+    synchronises the host, reads a size back or allocates outside PyTorch's allocator, so the
+    whole step captures as it is.  Every replay -- with eager steps and synchronisations between
+    them, and with new token values in the captured input buffer -- must reproduce the eager
+    step's output and gradients bit for bit (the kernels use no atomics)."""
+    print(f"block under a HIP graph {dtype} D={D} F={F} {dispatcher}", flush=True)
+    T, E, K = 600, 16, 4
+    spec = R.RouterSpec(E, K, score_func="softmax", route_norm=True)
+    p = make_params(E, D, F, dtype, seed=31)
+    kw = dict(pad_multiple=64) if dispatcher == "padded" else {}
+    block = build_block(p, spec, D, F, dtype, DEV, dispatcher=dispatcher, **kw)
+    block.train()
+    g = torch.Generator().manual_seed(32)
+    xin = torch.randn(T, D, generator=g).to(dtype).to(DEV).requires_grad_()
+    gout = torch.randn(T, D, generator=g).to(dtype).to(DEV)
+    params = [q for q in block.parameters() if q.requires_grad]
+
+    def step():
+        return torch.autograd.grad(block(xin), [xin] + params, gout)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = step()
+    for rep in range(3):
+        with torch.no_grad():
+            xin.copy_(torch.randn(T, D, generator=g).to(dtype))  # new tokens, new routing
+        eager = [t.clone() for t in step()]
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, want in zip(captured, eager):
+            assert torch.equal(got, want), f"replay {rep} differs from the eager step"
+
+
 def test_dispatcher_api_matches_reference_contract():
     """dispatch/combine through the public dispatcher classes, analytic expectation
     out = x * 2 * sum(scores) (tests/unit_tests/cpu/models/test_moe_token_dispatch.py:249-309)."""
