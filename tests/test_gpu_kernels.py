@@ -333,6 +333,8 @@ def test_grouped_experts_bf16_generic_shapes(ops, counts, D, Fd):
     ((128, 128), 64, 64), ((5, 6, 4, 7), 128, 64), ((200, 0, 129, 1, 300), 256, 192),
     ((0, 0, 0), 64, 128), ((513, 77), 512, 320), ((1000,), 256, 768),
     ((200, 0, 129), 384, 768), ((131, 260), 768, 384),
+    # one segment (a dense layer run through the grouped kernels): ragged and whole last tiles
+    ((1000,), 384, 512), ((512,), 512, 384), ((3,), 384, 384),
     # more experts than XCDs with a skewed, tie-laden histogram: the weight-gradient walk by
     # descending count must still visit every expert's every tile exactly once
     ((300, 0, 5, 700, 1, 64, 65, 0, 128, 129, 2, 5, 4, 250, 0, 90, 17, 33, 640), 384, 512),
