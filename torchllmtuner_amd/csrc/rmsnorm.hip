@@ -208,6 +208,128 @@ __global__ __launch_bounds__(256) void rms_bwd_fused_kernel(const T* __restrict_
   for (int d = threadIdx.x; d < D; d += 256) partial[static_cast<int64_t>(blockIdx.x) * D + d] = colsum[d];
 }
 
+// 16 bytes of T as N floats and back
+template <typename T, int N>
+__device__ __forceinline__ void unpack16(const u32x4& q, float (&v)[N]) {
+  if constexpr (std::is_same<T, float>::value) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = __uint_as_float(q[j]);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      v[2 * j] = __uint_as_float(q[j] << 16);
+      v[2 * j + 1] = __uint_as_float(q[j] & 0xffff0000u);
+    }
+  }
+}
+template <typename T, int N>
+__device__ __forceinline__ u32x4 pack16(const float (&v)[N]) {
+  u32x4 q;
+  if constexpr (std::is_same<T, float>::value) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) q[j] = __float_as_uint(v[j]);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) q[j] = pack_bf16x2(v[2 * j], v[2 * j + 1]);
+  }
+  return q;
+}
+
+// The same pass for rows of at most 4 x 64 sixteen-byte groups (2048 bf16 or 1024 fp32 columns): a
+// wave holds its row of dy and x in registers, so the row is read from memory once (the kernel
+// above reads it for the row's dot product and again, from cache, for dx), the weights stay in
+// registers across the rows, and the next row of the wave is requested before the current one is
+// reduced -- with one row in flight per wave the kernel waited out a memory round trip per row.
+template <typename T, int ITER>
+__global__ __launch_bounds__(256) void rms_bwd_rows_in_registers_kernel(
+    const T* __restrict__ dy, const T* __restrict__ x, const T* __restrict__ w, const float* __restrict__ rstd,
+    T* __restrict__ dx, float* __restrict__ partial, int rows, int D, int rows_per_block) {
+  constexpr int N = kVec<T>;
+  extern __shared__ float colsum[];  // [D]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float acc[ITER][N], g[ITER][N];
+  const u32x4 zero = {0, 0, 0, 0};
+#pragma unroll
+  for (int k = 0; k < ITER; ++k) {
+    const int i = (k * kWave + lane) * N;
+    u32x4 q = zero;
+    if (i < D) q = *reinterpret_cast<const u32x4*>(w + i);
+    unpack16<T, N>(q, g[k]);
+#pragma unroll
+    for (int j = 0; j < N; ++j) acc[k][j] = 0.0f;
+  }
+  const int r0 = blockIdx.x * rows_per_block;
+  const int r1 = min(r0 + rows_per_block, rows);
+  u32x4 cdy[ITER], cx[ITER];
+  auto fetch = [&](int row, u32x4 (&a)[ITER], u32x4 (&b)[ITER]) {
+    const int64_t o = static_cast<int64_t>(row) * D;
+#pragma unroll
+    for (int k = 0; k < ITER; ++k) {
+      const int i = (k * kWave + lane) * N;
+      a[k] = zero;
+      b[k] = zero;
+      if (i < D) {
+        a[k] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(dy + o + i));
+        b[k] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(x + o + i));
+      }
+    }
+  };
+  int row = r0 + wave;
+  if (row < r1) fetch(row, cdy, cx);
+  for (; row < r1; row += 4) {
+    u32x4 ndy[ITER], nx[ITER];
+    const bool more = row + 4 < r1;
+    if (more) fetch(row + 4, ndy, nx);
+    const float r = rstd[row];
+    float dot = 0.0f;
+#pragma unroll
+    for (int k = 0; k < ITER; ++k) {
+      float a[N], b[N];
+      unpack16<T, N>(cdy[k], a);
+      unpack16<T, N>(cx[k], b);
+#pragma unroll
+      for (int j = 0; j < N; ++j) dot += (a[j] * g[k][j]) * (b[j] * r);
+    }
+    const float c = wave_sum(dot) / static_cast<float>(D);
+    const int64_t o = static_cast<int64_t>(row) * D;
+#pragma unroll
+    for (int k = 0; k < ITER; ++k) {
+      const int i = (k * kWave + lane) * N;
+      float a[N], b[N], out[N];
+      unpack16<T, N>(cdy[k], a);
+      unpack16<T, N>(cx[k], b);
+#pragma unroll
+      for (int j = 0; j < N; ++j) {
+        const float xh = b[j] * r;
+        out[j] = r * (a[j] * g[k][j] - xh * c);
+        acc[k][j] += a[j] * xh;
+      }
+      if (dx && i < D) *reinterpret_cast<u32x4*>(dx + o + i) = pack16<T, N>(out);
+    }
+    if (more) {
+#pragma unroll
+      for (int k = 0; k < ITER; ++k) {
+        cdy[k] = ndy[k];
+        cx[k] = nx[k];
+      }
+    }
+  }
+  for (int turn = 0; turn < 4; ++turn) {
+    if (wave == turn) {
+#pragma unroll
+      for (int k = 0; k < ITER; ++k) {
+        const int i = (k * kWave + lane) * N;
+        if (i < D) {
+#pragma unroll
+          for (int j = 0; j < N; ++j) colsum[i + j] = turn == 0 ? acc[k][j] : colsum[i + j] + acc[k][j];
+        }
+      }
+    }
+    __syncthreads();
+  }
+  for (int d = threadIdx.x; d < D; d += 256) partial[static_cast<int64_t>(blockIdx.x) * D + d] = colsum[d];
+}
+
 // rows per workgroup of the column sums: 64, more once that would exceed 4096 workgroups
 __host__ __device__ inline int64_t dw_rows_per_chunk(int64_t rows) {
   const int64_t per = (rows + 4095) / 4096;
@@ -330,6 +452,12 @@ extern "C" int mi355_rms_norm_bwd(const void* dy, const void* x, const void* wei
       const int used = (int)((rows + rpb - 1) / rpb);
       auto launch = [&](auto iter) {
         constexpr int ITER = decltype(iter)::value;
+        if constexpr (ITER <= 4) {
+          hipLaunchKernelGGL((rms_bwd_rows_in_registers_kernel<T, ITER>), dim3(used), dim3(256), (size_t)D * 4, s,
+                             static_cast<const T*>(dy), static_cast<const T*>(x), static_cast<const T*>(weight), rstd,
+                             static_cast<T*>(dx), static_cast<float*>(workspace), (int)rows, (int)D, rpb);
+          return;
+        }
         hipLaunchKernelGGL((rms_bwd_fused_kernel<T, ITER>), dim3(used), dim3(256), (size_t)D * 4, s,
                            static_cast<const T*>(dy), static_cast<const T*>(x), static_cast<const T*>(weight), rstd,
                            static_cast<T*>(dx), static_cast<float*>(workspace), (int)rows, (int)D, rpb);
