@@ -272,6 +272,65 @@ def test_block_step_replays_from_a_hip_graph(dtype, D, F, dispatcher):
             assert torch.equal(got, want), f"replay {rep} differs from the eager step"
 
 
+def _random_case(rng):
+    dtype = rng.choice([torch.float32, torch.bfloat16])
+    T = rng.choice([1, 2, 7, 64, 130, 257, 600])
+    D = rng.choice([64, 96, 128, 384, 448, 512])
+    F = rng.choice([64, 128, 384, 576, 640])
+    E = rng.choice([2, 5, 8, 64])
+    K = rng.choice([k for k in (1, 2, 3, 6) if k <= E])
+    spec = R.RouterSpec(E, K, score_func=rng.choice(["softmax", "sigmoid", "sqrtsoftplus"]),
+                        route_norm=rng.choice([True, False]), route_scale=rng.choice([1.0, 2.5]))
+    kind = rng.choice(["local", "padded", "share", "local"])
+    kw, El = {}, E
+    if kind == "padded":
+        kw = dict(dispatcher="padded", pad_multiple=rng.choice([1, 8, 128]))
+    elif kind == "share":
+        lo = rng.randrange(0, E - 1)
+        hi = rng.randrange(lo + 1, E + 1)
+        kw, El = dict(dispatcher="share", local=(lo, hi)), hi - lo
+    batch = rng.choice([True, False]) and T % 2 == 0
+    return dtype, T, D, F, E, K, spec, kw, El, batch
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_randomised_small_shapes_match_the_oracle(seed):
+    """Sixteen seeded random configurations per seed -- dtype, token count (down to one token),
+    widths on and off the MFMA path, expert count, top-k, score function, norm, scale, dispatcher
+    (local, padded, one rank's share), flat or (B, S, D) input -- forward and every gradient
+    against the oracle.  A token whose choice is a few-ulp near tie may flip; then only the
+    routing bound is checked for that case."""
+    import random
+
+    rng = random.Random(seed)
+    for it in range(16):
+        dtype, T, D, F, E, K, spec, kw, El, batch = _random_case(rng)
+        print(f"block random case {seed}/{it}: {dtype} T={T} D={D} F={F} E={E} K={K} {spec.score_func} "
+              f"norm={spec.route_norm} scale={spec.route_scale} {kw} batch={batch}", flush=True)
+        p = make_params(E, D, F, dtype, seed=100 * seed + it, std=0.05, El=El)
+        g = torch.Generator().manual_seed(1000 * seed + it)
+        shape = (2, T // 2, D) if batch else (T, D)
+        x = torch.randn(*shape, generator=g).to(dtype)
+        gout = torch.randn(*shape, generator=g).to(dtype)
+        got, want, aux, block = _run_pair(p, spec, x, gout, dtype, D, F, **kw)
+        ok = stable_tokens(aux["logits"], spec)
+        with torch.no_grad():
+            _, ids = block.router.route(x.reshape(-1, D).to(DEV), block.expert_bias_E)
+        differ = ~(ids.cpu() == aux["ids_TK"]).all(-1)
+        assert not differ[ok].any(), "routing differs on tokens that are not near ties"
+        if differ.any():
+            continue
+        for k in want:
+            gm, wm = float(got[k].detach().float().abs().max()), float(want[k].detach().float().abs().max())
+            if k == "router_w_ED" and K == 1 and spec.route_norm and max(gm, wm) < 1e-4:
+                continue  # d/ds of s / (s + 1e-20) is zero: both sides hold rounding noise only
+            if wm == 0.0:
+                assert gm == 0.0, k
+                continue
+            err = rel_max(got[k], want[k]) if dtype == torch.float32 else rel_l2(got[k].float(), want[k].float())
+            assert err < (1e-5 if dtype == torch.float32 else 2e-2), f"{k}: {err}"
+
+
 def test_dispatcher_api_matches_reference_contract():
     """dispatch/combine through the public dispatcher classes, analytic expectation
     out = x * 2 * sum(scores) (tests/unit_tests/cpu/models/test_moe_token_dispatch.py:249-309)."""
