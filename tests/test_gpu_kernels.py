@@ -345,6 +345,24 @@ def test_grouped_experts_bf16_mfma(ops, counts, D, Fd):
 
 
 # ---------------------------------------------------------------- balance loss
+@pytest.mark.parametrize("seed", [0, 1])
+def test_grouped_experts_bf16_mfma_random_segments(ops, seed):
+    """Twenty seeded random segment lists per seed on the MFMA path: widths with odd and even
+    numbers of 64-wide K steps, one to seventeen experts, counts around every tile and block
+    boundary (0, 1, 15..17, 63..65, 255..257, 511..513, 1100)."""
+    import random
+
+    rng = random.Random(seed)
+    sizes = [0, 0, 1, 3, 15, 16, 17, 63, 64, 65, 200, 255, 256, 257, 300, 511, 512, 513, 700, 1100]
+    for it in range(20):
+        D, Fd = rng.choice([384, 448, 512, 640, 1024]), rng.choice([384, 448, 576, 768])
+        counts = tuple(rng.choice(sizes) for _ in range(rng.choice([1, 2, 3, 5, 9, 17])))
+        if sum(counts) > 4000:
+            counts = tuple(c // 3 for c in counts)
+        print(f"experts bf16 mfma random {seed}/{it}: D={D} F={Fd} counts={counts}", flush=True)
+        _experts_case(ops, torch.bfloat16, counts, D, Fd, std=0.05, seed=100 * seed + it)
+
+
 @pytest.mark.parametrize("T,E,K,padded", [(12, 4, 2, False), (1000, 128, 8, True), (4096, 256, 8, True),
                                           (0, 8, 2, False), (77, 320, 5, False)])
 def test_balance_loss_fwd_bwd(ops, T, E, K, padded):
