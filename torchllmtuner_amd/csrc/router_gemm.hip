@@ -265,28 +265,38 @@ __global__ __launch_bounds__(X_NT, 2) void gate_dx_kernel(const float* __restric
   for (int m = 0; m < 2; ++m)
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[m][i] = 0.0f;
-  for (int k0 = 0; k0 < E; k0 += BK) {
-    // A: 128 rows x 8 chunks of 8 experts = 1024 units, 2 per thread
+  // One LDS stage; the operands of K step k+1 are requested into registers before the MFMAs of
+  // step k (with nothing in flight during the MFMAs every step waited out a memory round trip).
+  // A: 128 rows x 8 chunks of 8 experts = 1024 units, 2 per thread; B: 64 experts x 16 chunks =
+  // 1024 units per piece, 2 per thread.
+  f32x4 ra[2][2];
+  u32x4 rb[2][2];
+  auto fetch = [&](int k0) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int u = tid + X_NT * i;
-      const int r = u >> 3, c = u & 7;
-      const float* src = dlogits + static_cast<int64_t>(min(t0 + r, T - 1)) * E + k0 + c * 8;
-      u32x4 hi, mid, lo;
-      split8(*reinterpret_cast<const f32x4*>(src), *reinterpret_cast<const f32x4*>(src + 4), hi, mid, lo);
-      *reinterpret_cast<u32x4*>(A_hi + kc_off(r, c)) = hi;
-      *reinterpret_cast<u32x4*>(A_mid + kc_off(r, c)) = mid;
+      const float* src = dlogits + static_cast<int64_t>(min(t0 + (u >> 3), T - 1)) * E + k0 + (u & 7) * 8;
+      ra[i][0] = *reinterpret_cast<const f32x4*>(src);
+      ra[i][1] = *reinterpret_cast<const f32x4*>(src + 4);
+      const uint16_t* bsrc = ws + static_cast<int64_t>(k0 + (u >> 4)) * D + n0 + (u & 15) * 8;
+      rb[i][0] = *reinterpret_cast<const u32x4*>(bsrc);
+      rb[i][1] = *reinterpret_cast<const u32x4*>(bsrc + ED);
     }
-    // B: 64 experts x 16 chunks = 1024 units per piece, 2 per thread
+  };
+  fetch(0);
+  for (int k0 = 0; k0 < E; k0 += BK) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int u = tid + X_NT * i;
-      const int k = u >> 4, c = u & 15;
-      const uint16_t* src = ws + static_cast<int64_t>(k0 + k) * D + n0 + c * 8;
-      *reinterpret_cast<u32x4*>(B_hi + ks_off<X_BN>(k, c)) = *reinterpret_cast<const u32x4*>(src);
-      *reinterpret_cast<u32x4*>(B_mid + ks_off<X_BN>(k, c)) = *reinterpret_cast<const u32x4*>(src + ED);
+      u32x4 hi, mid, lo;
+      split8(ra[i][0], ra[i][1], hi, mid, lo);
+      *reinterpret_cast<u32x4*>(A_hi + kc_off(u >> 3, u & 7)) = hi;
+      *reinterpret_cast<u32x4*>(A_mid + kc_off(u >> 3, u & 7)) = mid;
+      *reinterpret_cast<u32x4*>(B_hi + ks_off<X_BN>(u >> 4, u & 15)) = rb[i][0];
+      *reinterpret_cast<u32x4*>(B_mid + ks_off<X_BN>(u >> 4, u & 15)) = rb[i][1];
     }
     __syncthreads();
+    if (k0 + BK < E) fetch(k0 + BK);
 #pragma unroll
     for (int kk = 0; kk < BK / 16; ++kk) {
       const bf16x8 bh = frag_ks<X_BN>(B_hi, wn, kk, lane);
@@ -347,26 +357,39 @@ __global__ __launch_bounds__(W_NT, 2) void gate_dw_kernel(const float* __restric
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[n][i] = 0.0f;
   const u32x4 zero = {0, 0, 0, 0};
-  for (int tk = t_begin; tk < t_end; tk += BK) {
-    // 64 tokens x 16 chunks of 8 experts (A) / 8 columns (B) = 1024 units each, 2 per thread
+  // 64 tokens x 16 chunks of 8 experts (A) / 8 columns (B) = 1024 units each, 2 per thread; one LDS
+  // stage, the next K step's operands requested into registers before the MFMAs of the current one
+  f32x4 ra[2][2];
+  u32x4 rb[2];
+  auto fetch = [&](int tk) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int u = tid + W_NT * i;
       const int k = u >> 4, c = u & 15;
-      const int t = tk + k;
-      const bool live = t < t_end;
-      const int tc = min(t, T - 1);
+      const int tc = min(tk + k, T - 1);
       const float* src = dlogits + static_cast<int64_t>(tc) * E + min(m0 + c * 8, E - 8);
+      ra[i][0] = *reinterpret_cast<const f32x4*>(src);
+      ra[i][1] = *reinterpret_cast<const f32x4*>(src + 4);
+      rb[i] = *reinterpret_cast<const u32x4*>(x + static_cast<int64_t>(tc) * D + n0 + c * 8);
+    }
+  };
+  if (t_begin < t_end) fetch(t_begin);
+  for (int tk = t_begin; tk < t_end; tk += BK) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int u = tid + W_NT * i;
+      const int k = u >> 4, c = u & 15;
+      const bool live = tk + k < t_end;
       u32x4 hi, mid, lo;
-      split8(*reinterpret_cast<const f32x4*>(src), *reinterpret_cast<const f32x4*>(src + 4), hi, mid, lo);
+      split8(ra[i][0], ra[i][1], hi, mid, lo);
       const int o = ks_off<W_BM>(k, c);
       *reinterpret_cast<u32x4*>(A_p + o) = live ? hi : zero;
       *reinterpret_cast<u32x4*>(A_p + BK * W_BM + o) = live ? mid : zero;
       *reinterpret_cast<u32x4*>(A_p + 2 * BK * W_BM + o) = live ? lo : zero;
-      *reinterpret_cast<u32x4*>(B_s + ks_off<W_BN>(k, c)) =
-          *reinterpret_cast<const u32x4*>(x + static_cast<int64_t>(tc) * D + n0 + c * 8);
+      *reinterpret_cast<u32x4*>(B_s + ks_off<W_BN>(k, c)) = rb[i];
     }
     __syncthreads();
+    if (tk + BK < t_end) fetch(tk + BK);
 #pragma unroll
     for (int kk = 0; kk < BK / 16; ++kk) {
       bf16x8 bf[2];
