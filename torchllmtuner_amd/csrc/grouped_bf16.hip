@@ -901,7 +901,10 @@ int set_lds(K kernel, int bytes) {
 // one tile wide (a last tile that would overhang is shifted back, never clamped).
 int bf16_row_tile_m() { return 256; }
 
-bool bf16_fast_path_ok(int64_t D, int64_t F) { return D % 64 == 0 && F % 64 == 0 && D >= 384 && F >= 384; }
+// ... and one expert's weight matrix below 2 GiB: operand loads address a tile with 32-bit byte offsets.
+bool bf16_fast_path_ok(int64_t D, int64_t F) {
+  return D % 64 == 0 && F % 64 == 0 && D >= 384 && F >= 384 && D * F < (1ll << 30);
+}
 
 enum { STAGE_GATEUP = 1, STAGE_DOWN = 2, STAGE_DH = 4, STAGE_DX = 8, STAGE_DW2 = 16, STAGE_DW1 = 32, STAGE_DW3 = 64 };
 
