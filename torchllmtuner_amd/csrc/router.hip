@@ -17,14 +17,59 @@ __device__ __forceinline__ float softplus_f32(float x) {
   return x > 20.0f ? x : log1pf(expf(x));  // torch's threshold=20, beta=1
 }
 
-// (value, index) arg-max across the wave; ties go to the lower index.
+// Wave reductions of this file run on DPP row operations (VALU rate) plus four lane reads, not on
+// shuffles: a shuffle is an LDS permute, and a token's selection needs about a hundred of them --
+// with one wavefront per token the LDS pipe of a CU, not memory, was what the select kernels waited
+// for.  The four controls below exchange within a row of 16 lanes (pairs, quads, halves, the row),
+// so after them every lane holds its row's result; lanes 0, 16, 32, 48 then give the four rows.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+template <int CTRL>
+__device__ __forceinline__ int dpp_i32(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, false);
+}
+constexpr int kDppPairs = 0xB1, kDppQuads = 0x4E, kDppHalfMirror = 0x141, kDppRowMirror = 0x140;
+
+__device__ __forceinline__ float lane_f32(float v, int l) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), l));
+}
+
+// sum over the wave, left in every lane
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+  v += dpp_f32<kDppPairs>(v);
+  v += dpp_f32<kDppQuads>(v);
+  v += dpp_f32<kDppHalfMirror>(v);
+  v += dpp_f32<kDppRowMirror>(v);
+  return (lane_f32(v, 0) + lane_f32(v, 16)) + (lane_f32(v, 32) + lane_f32(v, 48));
+}
+__device__ __forceinline__ float wave_max_dpp(float v) {
+  v = fmaxf(v, dpp_f32<kDppPairs>(v));
+  v = fmaxf(v, dpp_f32<kDppQuads>(v));
+  v = fmaxf(v, dpp_f32<kDppHalfMirror>(v));
+  v = fmaxf(v, dpp_f32<kDppRowMirror>(v));
+  return fmaxf(fmaxf(lane_f32(v, 0), lane_f32(v, 16)), fmaxf(lane_f32(v, 32), lane_f32(v, 48)));
+}
+
+// the better of two (value, index) candidates: the larger value, ties to the lower index
+__device__ __forceinline__ void take_better(float& v, int& idx, float ov, int oi) {
+  if (ov > v || (ov == v && oi < idx)) { v = ov; idx = oi; }
+}
+
+// (value, index) arg-max across the wave, left in every lane; ties go to the lower index.
 __device__ __forceinline__ void wave_argmax(float& v, int& idx) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) {
-    const float ov = __shfl_xor(v, o, kWave);
-    const int oi = __shfl_xor(idx, o, kWave);
-    if (ov > v || (ov == v && oi < idx)) { v = ov; idx = oi; }
-  }
+  { const float ov = dpp_f32<kDppPairs>(v); const int oi = dpp_i32<kDppPairs>(idx); take_better(v, idx, ov, oi); }
+  { const float ov = dpp_f32<kDppQuads>(v); const int oi = dpp_i32<kDppQuads>(idx); take_better(v, idx, ov, oi); }
+  { const float ov = dpp_f32<kDppHalfMirror>(v); const int oi = dpp_i32<kDppHalfMirror>(idx); take_better(v, idx, ov, oi); }
+  { const float ov = dpp_f32<kDppRowMirror>(v); const int oi = dpp_i32<kDppRowMirror>(idx); take_better(v, idx, ov, oi); }
+  float a = lane_f32(v, 0), b = lane_f32(v, 32);
+  int ai = __builtin_amdgcn_readlane(idx, 0), bi = __builtin_amdgcn_readlane(idx, 32);
+  take_better(a, ai, lane_f32(v, 16), __builtin_amdgcn_readlane(idx, 16));
+  take_better(b, bi, lane_f32(v, 48), __builtin_amdgcn_readlane(idx, 48));
+  take_better(a, ai, b, bi);
+  v = a;
+  idx = ai;
 }
 
 template <int VPL>
@@ -47,14 +92,14 @@ __device__ __forceinline__ void compute_scores(const float* __restrict__ row, in
     float m = x[0];
 #pragma unroll
     for (int j = 1; j < VPL; ++j) m = fmaxf(m, x[j]);
-    m = wave_max(m);
+    m = wave_max_dpp(m);
     float sum = 0.0f;
 #pragma unroll
     for (int j = 0; j < VPL; ++j) {
       s[j] = (lane + j * kWave < E) ? expf(x[j] - m) : 0.0f;
       sum += s[j];
     }
-    sum = wave_sum(sum);
+    sum = wave_sum_dpp(sum);
 #pragma unroll
     for (int j = 0; j < VPL; ++j) s[j] = s[j] / sum;
   } else if (score_func == MI355_SCORE_SIGMOID) {
@@ -155,13 +200,13 @@ __global__ __launch_bounds__(256) void select_fwd_kernel(
         if (bi == 0x7fffffff || c[j] > bv) { bv = c[j]; bi = lane + j * kWave; }
       }
       wave_argmax(bv, bi);
-      const int owner = bi & 63, slot = bi >> 6;
+      const int owner = __builtin_amdgcn_readfirstlane(bi & 63), slot = bi >> 6;
       float sv = 0.0f;
       if (lane == owner) {
         taken |= 1u << slot;
         sv = pick<VPL>(s, slot);
       }
-      sv = __shfl(sv, owner, kWave);
+      sv = lane_f32(sv, owner);  // owner is wave-uniform: a lane read, not a shuffle
       if (lane == k) { my_w = sv; my_id = bi; }
     }
     if (cutoff_out) {
@@ -183,8 +228,8 @@ __global__ __launch_bounds__(256) void select_fwd_kernel(
     my_id = static_cast<int>(base % E);
     // gather the unbiased score of each slot's expert from its owner lane
     for (int k = 0; k < K; ++k) {
-      const int want = __shfl(my_id, k, kWave);
-      const float got = __shfl(pick<VPL>(s, want >> 6), want & 63, kWave);
+      const int want = __builtin_amdgcn_readlane(my_id, k);
+      const float got = lane_f32(pick<VPL>(s, want >> 6), __builtin_amdgcn_readfirstlane(want & 63));
       if (lane == k) my_w = got;
     }
   }
@@ -193,7 +238,7 @@ __global__ __launch_bounds__(256) void select_fwd_kernel(
     my_w = 1.0f / static_cast<float>(K);
   } else {
     if (route_norm) {
-      const float sum = wave_sum(lane < K ? my_w : 0.0f);
+      const float sum = wave_sum_dpp(lane < K ? my_w : 0.0f);
       my_w = my_w / (sum + 1e-20f);
     }
     my_w = my_w * route_scale;
@@ -206,7 +251,7 @@ __global__ __launch_bounds__(256) void select_fwd_kernel(
     // one-hot routing map of the token, one byte per expert
     unsigned chosen = 0;
     for (int k = 0; k < K; ++k) {
-      const int idk = __shfl(my_id, k, kWave);
+      const int idk = __builtin_amdgcn_readlane(my_id, k);
       if ((idk & 63) == lane) chosen |= 1u << (idk >> 6);
     }
 #pragma unroll
@@ -251,16 +296,16 @@ __global__ __launch_bounds__(256) void select_bwd_kernel(
     const float dw = lane < K ? dweights[static_cast<int64_t>(t) * K + lane] : 0.0f;
     float g;
     if (route_norm) {
-      const float denom = wave_sum(sk) + 1e-20f;
-      const float dot = wave_sum(dw * sk);
+      const float denom = wave_sum_dpp(sk) + 1e-20f;
+      const float dot = wave_sum_dpp(dw * sk);
       g = route_scale * (dw / denom - dot / (denom * denom));
     } else {
       g = route_scale * dw;
     }
     // scatter-add into the dense score gradient, serially so a repeated id adds up
     for (int k = 0; k < K; ++k) {
-      const int idk = __shfl(id, k, kWave);
-      const float gk = __shfl(g, k, kWave);
+      const int idk = __builtin_amdgcn_readlane(id, k);
+      const float gk = lane_f32(g, k);
       if (lane == 0) ds[idk] += gk;
     }
   }
@@ -276,7 +321,7 @@ __global__ __launch_bounds__(256) void select_bwd_kernel(
     float dot = 0.0f;
 #pragma unroll
     for (int j = 0; j < VPL; ++j) dot += (lane + j * kWave < E) ? s[j] * d[j] : 0.0f;
-    dot = wave_sum(dot);
+    dot = wave_sum_dpp(dot);
 #pragma unroll
     for (int j = 0; j < VPL; ++j) d[j] = s[j] * (d[j] - dot);
   } else if (score_func == MI355_SCORE_SIGMOID) {
