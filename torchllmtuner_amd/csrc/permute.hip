@@ -24,9 +24,19 @@ constexpr int kBatch = 16;  // histogram loads in flight per lane in the scan
 
 __global__ __launch_bounds__(256) void plan_rank_kernel(const int64_t* __restrict__ ids, int N,
                                                         int E, int32_t* __restrict__ rank_in_wave,
-                                                        int32_t* __restrict__ wave_hist) {
+                                                        int32_t* __restrict__ wave_hist,
+                                                        int32_t* __restrict__ slot_of_row,
+                                                        int32_t* __restrict__ token_of_row, int row_capacity) {
   extern __shared__ int32_t cnt[];  // [4][E]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // rows that end up without a slot (padding, unused capacity) read -1: every row starts as -1 here
+  // and the rows kernel overwrites the real ones (a launch of its own for this fill cost as much
+  // as the rows kernel)
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < row_capacity;
+       i += static_cast<int64_t>(gridDim.x) * 256) {
+    slot_of_row[i] = -1;
+    if (token_of_row) token_of_row[i] = -1;
+  }
   volatile int32_t* my = cnt + wave * E;
   for (int e = lane; e < E; e += kWave) my[e] = 0;
   __syncthreads();
@@ -452,10 +462,9 @@ static int plan_impl(const int64_t* ids, int64_t T, int64_t K, int64_t E, int64_
   const int nwaves = nblocks * kWavesPerBlock;
   if (nblocks > 0) {
     hipLaunchKernelGGL(plan_rank_kernel, dim3(nblocks), dim3(256), (size_t)kWavesPerBlock * E * 4, s,
-                       ids, (int)N, (int)E, rank_in_wave, wave_hist);
+                       ids, (int)N, (int)E, rank_in_wave, wave_hist, slot_of_row, token_of_row, (int)row_capacity);
     if (int rc = check_launch("plan_rank")) return rc;
-  }
-  if (row_capacity > 0) {
+  } else if (row_capacity > 0) {  // no slots at all: only the fill is left to do
     hipLaunchKernelGGL(fill_i32_kernel, dim3((unsigned)((row_capacity + 255) / 256)), dim3(256), 0, s,
                        slot_of_row, token_of_row, row_capacity, -1);
     if (int rc = check_launch("plan_fill")) return rc;
