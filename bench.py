@@ -57,6 +57,9 @@ def parse():
                     help="also loop each grouped GEMM, the whole step, the vendor GEMM, the MFMA probe and a copy for "
                          "--power-seconds each while sampling the card's power sensor (hwmon); adds a \"power\" object")
     ap.add_argument("--power-seconds", type=float, default=2.5)
+    ap.add_argument("--kloop", action="store_true",
+                    help="also run the stand-alone K-loop study of bench_probe/kloop.hip (needs 4.4 GB of device memory); "
+                         "with --power each case is also looped under the power sensor")
     ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay of the same step")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (known traffic, for scaling rocprof FETCH_SIZE / WRITE_SIZE)")
@@ -148,6 +151,59 @@ def sustained_mfma(dev):
             c = clocks.view(blocks, 2).double()
             out[name][label] = {"TFLOP/s": round(flops / (ms * 1e-3) / 1e12, 1),
                                 "core_clock_mhz": round(float((c[:, 0] / c[:, 1]).mean()) * 100.0, 0)}
+    return out
+
+
+KLOOP_VARIANTS = ("product_loop", "without_skip_branches", "direct_to_lds", "four_waves_128x128")
+
+
+def kloop_study(dev, watts=None):
+    """Stand-alone K loops of the grouped GEMMs' shape (bench_probe/kloop.hip: 256 x 256 x 64 tile
+    steps, normally distributed bf16 operands, no epilogue, every tile full) in four schedules,
+    each with all operands resident in L2 and with the B half of every step streamed from HBM
+    (32 KB per step and workgroup): TFLOP/s, and watts when ``watts`` (a function: callable ->
+    average watts while it loops) is given.  None when the probe library is not built."""
+    import ctypes
+
+    import torch
+
+    path = os.path.join(ROOT, "bench_probe", "libmi355probe.so")
+    if not os.path.exists(path):
+        return None
+    lib = ctypes.CDLL(path)
+    if not hasattr(lib, "mi355_probe_kloop"):
+        return None
+    vp = ctypes.c_void_p
+    lib.mi355_probe_kloop.argtypes = [ctypes.c_int, ctypes.c_int, vp, vp, vp, ctypes.c_int, ctypes.c_int, vp]
+    lib.mi355_probe_kloop.restype = ctypes.c_int
+    for f in (lib.mi355_probe_kloop_hot_elems, lib.mi355_probe_kloop_cold_elems):
+        f.argtypes, f.restype = [ctypes.c_int], ctypes.c_long
+    blocks = torch.cuda.get_device_properties(dev).multi_processor_count
+    gen = torch.Generator(device=dev).manual_seed(0)
+    hot = torch.randn(lib.mi355_probe_kloop_hot_elems(blocks), device=dev, generator=gen).bfloat16()
+    cold = torch.empty(lib.mi355_probe_kloop_cold_elems(blocks), dtype=torch.bfloat16, device=dev)
+    piece = 1 << 27
+    for i in range(0, cold.numel(), piece):  # in pieces: the fp32 draw of the whole buffer would be 8.6 GB
+        cold[i:i + piece] = torch.randn(min(piece, cold.numel() - i), device=dev, generator=gen).bfloat16()
+    sink = torch.zeros(1, dtype=torch.float32, device=dev)
+    ksteps = 2048
+    flops = blocks * ksteps * 2.0 * 256 * 256 * 64
+
+    def launch(v, stream_hbm, n=ksteps):
+        rc = lib.mi355_probe_kloop(v, stream_hbm, hot.data_ptr(), cold.data_ptr(), sink.data_ptr(), blocks, n,
+                                   torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, rc
+
+    out = {"ksteps": ksteps, "workgroups": blocks, "stream_bytes_per_step_and_workgroup": 32768}
+    for v, name in enumerate(KLOOP_VARIANTS):
+        ent = {}
+        for stream_hbm, key in ((0, "operands_in_l2"), (1, "b_operand_from_hbm")):
+            launch(v, stream_hbm, 64)
+            best = min(time_events(lambda: launch(v, stream_hbm), 1, warmup=0) for _ in range(3))
+            ent[key] = {"TFLOP/s": round(flops / (best * 1e-3) / 1e12, 1), "us_per_k_step": round(best * 1e3 / ksteps, 3)}
+            if watts is not None:
+                ent[key]["watts"] = watts(lambda: launch(v, stream_hbm, 512))
+        out[name] = ent
     return out
 
 
@@ -655,6 +711,13 @@ def main():
                     ent["TFLOP/s_looped"] = round(pl[1] * 8.0 * 2000 * 262144 * 2 / (ent["ms_per_call_looped"] * 1e-3) / 1e12, 1)
             ent = result["power"]["cases"]["copy_1GiB"]
             ent["GB/s_looped"] = round(2.0 * (1 << 30) / (ent["ms_per_call_looped"] * 1e-3) / 1e9, 1)
+    if args.kloop:
+        watts = None
+        if args.power:
+            def watts(fn):
+                t = power_table({"case": fn}, args.power_seconds)
+                return None if t is None else t["cases"]["case"]["watts"]
+        result["kloop_study"] = kloop_study(dev, watts)
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)
