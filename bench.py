@@ -154,15 +154,20 @@ def sustained_mfma(dev):
     return out
 
 
-KLOOP_VARIANTS = ("product_loop", "without_skip_branches", "direct_to_lds", "four_waves_128x128")
+KLOOP_VARIANTS = ("product_loop", "without_skip_branches", "direct_to_lds", "four_waves_128x128",
+                  "staging_without_fragment_reads", "fragment_reads_without_staging", "mfma_only")
+KLOOP_PLACEMENTS = ("windows_per_workgroup", "b_operand_from_hbm", "one_shared_window")
 
 
 def kloop_study(dev, watts=None):
     """Stand-alone K loops of the grouped GEMMs' shape (bench_probe/kloop.hip: 256 x 256 x 64 tile
-    steps, normally distributed bf16 operands, no epilogue, every tile full) in four schedules,
-    each with all operands resident in L2 and with the B half of every step streamed from HBM
-    (32 KB per step and workgroup): TFLOP/s, and watts when ``watts`` (a function: callable ->
-    average watts while it loops) is given.  None when the probe library is not built."""
+    steps, normally distributed bf16 operands, no epilogue, every tile full): four schedules and
+    three ablations of the second (no fragment reads / no staging / neither), each with a 2 MiB
+    operand window per workgroup (34 MB in all: the memory-side cache), with the B half of every
+    step streamed from HBM (32 KB per step and workgroup; schedules only) and with one window
+    shared by all workgroups (resident in every L2): TFLOP/s, and watts when ``watts`` (a
+    function: callable -> average watts while it loops) is given.  None when the probe library
+    is not built."""
     import ctypes
 
     import torch
@@ -189,20 +194,22 @@ def kloop_study(dev, watts=None):
     ksteps = 2048
     flops = blocks * ksteps * 2.0 * 256 * 256 * 64
 
-    def launch(v, stream_hbm, n=ksteps):
-        rc = lib.mi355_probe_kloop(v, stream_hbm, hot.data_ptr(), cold.data_ptr(), sink.data_ptr(), blocks, n,
+    def launch(v, placement, n=ksteps):
+        rc = lib.mi355_probe_kloop(v, placement, hot.data_ptr(), cold.data_ptr(), sink.data_ptr(), blocks, n,
                                    torch.cuda.current_stream().cuda_stream)
         assert rc == 0, rc
 
     out = {"ksteps": ksteps, "workgroups": blocks, "stream_bytes_per_step_and_workgroup": 32768}
     for v, name in enumerate(KLOOP_VARIANTS):
         ent = {}
-        for stream_hbm, key in ((0, "operands_in_l2"), (1, "b_operand_from_hbm")):
-            launch(v, stream_hbm, 64)
-            best = min(time_events(lambda: launch(v, stream_hbm), 1, warmup=0) for _ in range(3))
+        for placement, key in enumerate(KLOOP_PLACEMENTS):
+            if placement == 1 and v > 3:
+                continue
+            launch(v, placement, 64)
+            best = min(time_events(lambda: launch(v, placement), 1, warmup=0) for _ in range(3))
             ent[key] = {"TFLOP/s": round(flops / (best * 1e-3) / 1e12, 1), "us_per_k_step": round(best * 1e3 / ksteps, 3)}
             if watts is not None:
-                ent[key]["watts"] = watts(lambda: launch(v, stream_hbm, 512))
+                ent[key]["watts"] = watts(lambda: launch(v, placement, 512))
         out[name] = ent
     return out
 

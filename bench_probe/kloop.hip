@@ -1,9 +1,10 @@
 // Stand-alone K loops of the grouped GEMMs' shape, used by the benchmark only (not part of the
 // MoE C ABI): 256 x 256 x 64 tile steps over operands of the caller's choice, no tile list, no
-// epilogue, every tile full.  They answer two questions the product kernels cannot be asked
-// directly: what a change of the loop's schedule is worth with every operand resident in L2, and
-// what is left of that once half of each step's operands stream from HBM the way an expert's
-// weights do.  Variants:
+// epilogue, every tile full.  They answer three questions the product kernels cannot be asked
+// directly: what a change of the loop's schedule is worth with every operand resident on the
+// chip, what is left of that once half of each step's operands stream from HBM the way an
+// expert's weights do, and how the loop's energy divides between the MFMAs, the fragment reads
+// from LDS and the staging of the next step's operands into LDS.  Variants:
 //   0  the product's loop: per K32 block the A fragments, then two halves of four B fragments,
 //      a quarter of the next step's staging (global -> registers -> LDS) with each half, and the
 //      MFMAs of each 16-row block behind a wave-uniform branch (the skip of empty blocks);
@@ -11,7 +12,11 @@
 //   2  operands loaded straight into LDS (buffer loads with the LDS destination; the swizzle of
 //      the layout is applied on the global side), requested one K step ahead;
 //   3  four waves, 128 x 128 per wave (a third fewer fragment reads), fragments of the next K32
-//      block read before the MFMAs of the current one.
+//      block read before the MFMAs of the current one;
+//   4  variant 1 with the staging but without the fragment reads (the MFMAs reuse the fragments
+//      of the first step);
+//   5  variant 1 with the fragment reads but without the staging (LDS keeps its first contents);
+//   6  variant 1 with neither: the MFMAs alone.
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -58,7 +63,7 @@ __device__ __forceinline__ u32x4 buffer_words(const void* base) {
 // resident operands: workgroup b reads a window of (BM + BN) rows x 2048 k starting at element
 // b * hot_stride of `hot`; streamed operands (STREAM): the B half of a step instead comes from
 // `cold`, 32 KB per step and workgroup that no other step or workgroup touches
-template <int BRANCHES, int STREAM>
+template <int BRANCHES, int STREAM, int FRAGMENTS = 1, int STAGING = 1>
 __global__ __launch_bounds__(512) void kloop_product(const uint16_t* __restrict__ hot, const uint16_t* __restrict__ cold,
                                                      float* out, int ksteps, long hot_stride, int active) {
   constexpr int NT = 512;
@@ -75,6 +80,9 @@ __global__ __launch_bounds__(512) void kloop_product(const uint16_t* __restrict_
   const uint16_t* gp = hot + static_cast<long>(blockIdx.x) * hot_stride + row * 2048 + chunk * 8;
   for (int i = 0; i < 8; ++i) st[i] = *reinterpret_cast<const u32x4*>(gp + static_cast<long>(i) * (NT / 8) * 2048);
   const int act = __builtin_amdgcn_readfirstlane(active);
+  bf16x8 af0[4], bf0[8];  // the first step's fragments, all the MFMAs see without FRAGMENTS
+  for (int a = 0; a < 4; ++a) af0[a] = frag16(smem, wm + a * 16, 0, lane);
+  for (int b = 0; b < 8; ++b) bf0[b] = frag16(smem + BM * BK, wn + b * 16, 0, lane);
   for (int ks = 0; ks < ksteps; ++ks) {
     const uint16_t* As = smem + (ks & 1) * STAGE;
     const uint16_t* Bs = As + BM * BK;
@@ -86,15 +94,15 @@ __global__ __launch_bounds__(512) void kloop_product(const uint16_t* __restrict_
     for (int kk = 0; kk < 2; ++kk) {
       bf16x8 af[4];
 #pragma unroll
-      for (int a = 0; a < 4; ++a) af[a] = frag16(As, wm + a * 16, kk, lane);
+      for (int a = 0; a < 4; ++a) af[a] = FRAGMENTS ? frag16(As, wm + a * 16, kk, lane) : af0[a];
 #pragma unroll
       for (int hb = 0; hb < 2; ++hb) {
         bf16x8 bf[4];
 #pragma unroll
-        for (int b = 0; b < 4; ++b) bf[b] = frag16(Bs, wn + (hb * 4 + b) * 16, kk, lane);
+        for (int b = 0; b < 4; ++b) bf[b] = FRAGMENTS ? frag16(Bs, wn + (hb * 4 + b) * 16, kk, lane) : bf0[hb * 4 + b];
         const int q = kk * 2 + hb;
 #pragma unroll
-        for (int i = q * 2; i < q * 2 + 2; ++i) {
+        for (int i = q * 2; STAGING && i < q * 2 + 2; ++i) {
           *reinterpret_cast<u32x4*>(Nx + lds0 + i * (NT / 8) * BK) = st[i];
           st[i] = (STREAM && i >= 4) ? *reinterpret_cast<const u32x4*>(gb + (i - 4) * 4096)
                                      : *reinterpret_cast<const u32x4*>(gk + static_cast<long>(i) * (NT / 8) * 2048);
@@ -241,15 +249,20 @@ bool allow_lds(K kernel) {
 extern "C" long mi355_probe_kloop_hot_elems(int blocks) { return static_cast<long>(blocks) * (BM + BN) * 2048 / 16 + (BM + BN) * 2048l + 2 * STAGE; }
 extern "C" long mi355_probe_kloop_cold_elems(int blocks) { return static_cast<long>(blocks) * kStreamSteps * kStreamStep; }
 
-// One launch of `blocks` workgroups running `ksteps` K steps of variant 0..3 (see the head of this
-// file); stream_hbm != 0: the B half of every step streams from `cold`.  flops = blocks * ksteps *
-// 2 * 256 * 256 * 64.  Returns 0, or a negative value for a bad argument / failed launch.
-extern "C" int mi355_probe_kloop(int variant, int stream_hbm, const void* hot, const void* cold, float* sink,
+// One launch of `blocks` workgroups running `ksteps` K steps of variant 0..6 (see the head of this
+// file).  placement 0: every workgroup re-reads its own 2 MiB window of `hot`, the windows 128 KiB
+// apart (34 MB for 256 workgroups: more than the L2 of an XCD, within the memory-side cache);
+// 1: the same, but the B half of every step streams from `cold` (variants 0..3 only); 2: all
+// workgroups re-read one 2 MiB window (resident in every L2).  flops = blocks * ksteps * 2 * 256 *
+// 256 * 64.  Returns 0, or a negative value for a bad argument / failed launch.
+extern "C" int mi355_probe_kloop(int variant, int placement, const void* hot, const void* cold, float* sink,
                                  int blocks, int ksteps, void* stream) {
-  if (!hot || !sink || blocks < 1 || ksteps < 1 || variant < 0 || variant > 3 || (stream_hbm && !cold)) return -1;
+  if (!hot || !sink || blocks < 1 || ksteps < 1 || variant < 0 || variant > 6 || placement < 0 || placement > 2) return -1;
+  const int stream_hbm = placement == 1;
+  if (stream_hbm && (!cold || variant > 3)) return -1;
   const uint16_t* h = static_cast<const uint16_t*>(hot);
   const uint16_t* c = static_cast<const uint16_t*>(cold);
-  const long stride = (BM + BN) * 2048l / 16;
+  const long stride = placement == 2 ? 0 : (BM + BN) * 2048l / 16;
   const size_t lds = 2 * STAGE * 2;
   hipStream_t s = static_cast<hipStream_t>(stream);
 #define MI355_KLOOP(kernel, threads, ...)                                                  \
@@ -261,6 +274,9 @@ extern "C" int mi355_probe_kloop(int variant, int stream_hbm, const void* hot, c
   if (variant == 1) { if (stream_hbm) MI355_KLOOP((kloop_product<0, 1>), 512, 4); else MI355_KLOOP((kloop_product<0, 0>), 512, 4); }
   if (variant == 2) { if (stream_hbm) MI355_KLOOP(kloop_direct<1>, 512); else MI355_KLOOP(kloop_direct<0>, 512); }
   if (variant == 3) { if (stream_hbm) MI355_KLOOP(kloop_four_waves<1>, 256); else MI355_KLOOP(kloop_four_waves<0>, 256); }
+  if (variant == 4) MI355_KLOOP((kloop_product<0, 0, 0, 1>), 512, 4);
+  if (variant == 5) MI355_KLOOP((kloop_product<0, 0, 1, 0>), 512, 4);
+  if (variant == 6) MI355_KLOOP((kloop_product<0, 0, 0, 0>), 512, 4);
 #undef MI355_KLOOP
   return hipGetLastError() == hipSuccess ? 0 : -2;
 }
