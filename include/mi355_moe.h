@@ -239,7 +239,7 @@ int mi355_permute_plan(const int64_t* ids_TK, int64_t T, int64_t K, int64_t E,
  * mi355_permute_plan without a workspace argument, for callers that cannot allocate device
  * memory (code under HIP graph capture, tight serving loops, harnesses that forbid it).  No
  * counterpart in the reference.  Same arguments, outputs and results as mi355_permute_plan;
- * the scratch (slot ranks, per-wave histograms) lives in an array inside the library,
+ * the scratch (slot ranks, per-workgroup histograms) lives in an array inside the library,
  * mi355_permute_plan_static_max_bytes() = 8 MiB per GPU, held until the process ends.
  * Returns MI355_EINVAL without launching when mi355_permute_plan_workspace_bytes(T,K,E)
  * exceeds that (e.g. N = T*K = 2^20 slots with E <= 128 fits; N = 131072, E = 256 fits).

@@ -67,12 +67,19 @@ SELECT_CASES = [
     dict(T=300, E=64, K=6, score_func="sigmoid", bias=True),
     dict(T=300, E=24, K=3, score_func="sqrtsoftplus", route_norm=True, route_scale=0.5),
     dict(T=257, E=320, K=5, score_func="softmax", num_expert_groups=5, num_limited_groups=2),
+    # groups of 2, 16, 24 (no aligned lane run), 128 (two registers per lane) experts
+    dict(T=300, E=16, K=3, score_func="softmax", num_expert_groups=8, num_limited_groups=2),
+    dict(T=300, E=128, K=6, score_func="sigmoid", route_norm=True, num_expert_groups=8, num_limited_groups=3, bias=True),
+    dict(T=300, E=96, K=4, score_func="sigmoid", num_expert_groups=4, num_limited_groups=2, bias=True),
+    dict(T=300, E=256, K=8, score_func="softmax", route_norm=True, num_expert_groups=2, num_limited_groups=1),
+    dict(T=300, E=512, K=8, score_func="sigmoid", num_expert_groups=4, num_limited_groups=2, bias=True),
     dict(T=10, E=4, K=2, score_func="sigmoid", fixed_router=True, route_scale=7.0),
     dict(T=10, E=4, K=2, score_func="sigmoid", debug_force_load_balance=True, route_norm=True, route_scale=2.0),
 ]
 
 
-@pytest.mark.parametrize("case", SELECT_CASES, ids=lambda c: f"E{c['E']}K{c['K']}{c['score_func']}")
+@pytest.mark.parametrize("case", SELECT_CASES,
+                         ids=lambda c: f"E{c['E']}K{c['K']}{c['score_func']}" + (f"G{c['num_expert_groups']}" if "num_expert_groups" in c else ""))
 def test_router_select_fwd_bwd(ops, case):
     print(f"router_select {case}", flush=True)
     c = dict(case)

@@ -4,13 +4,16 @@
 //   1. plan_rank    each wave walks 256 consecutive slots in 64-slot chunks; within
 //                   a chunk a slot's rank among equal experts is counted with 64
 //                   lane reads, and the running per-wave expert counts live in LDS
-//                   (one writer per expert and chunk).  Emits the rank of every
-//                   slot inside its wave and the wave's histogram.
-//   2. plan_scan    one workgroup: per-expert exclusive scan of the wave histograms
-//                   (ascending wave = ascending slot, which is what makes the sort
-//                   stable), the padded segment offsets, and the MFMA tile list.
-//   3. plan_rows    row = segment offset + waves-before + rank-in-wave, written both
-//                   ways (row_of_slot, slot_of_row).
+//                   (one writer per expert and chunk).  The four waves of a workgroup
+//                   then add the counts of the waves before them: emits the rank of
+//                   every slot inside its workgroup's 1024 slots and the workgroup's
+//                   histogram.
+//   2. plan_scan    one workgroup: per-expert exclusive scan of the workgroup
+//                   histograms (ascending workgroup = ascending slot, which is what
+//                   makes the sort stable), the padded segment offsets, and the MFMA
+//                   tile list.
+//   3. plan_rows    row = segment offset + workgroups-before + rank-in-workgroup,
+//                   written both ways (row_of_slot, slot_of_row).
 // The row movers are pure bandwidth kernels: one wave per token, 16-byte lanes.
 #include "common.h"
 
@@ -23,8 +26,8 @@ constexpr int kSlotsPerBlock = kSlotsPerWave * kWavesPerBlock;
 constexpr int kBatch = 16;  // histogram loads in flight per lane in the scan
 
 __global__ __launch_bounds__(256) void plan_rank_kernel(const int64_t* __restrict__ ids, int N,
-                                                        int E, int32_t* __restrict__ rank_in_wave,
-                                                        int32_t* __restrict__ wave_hist,
+                                                        int E, int32_t* __restrict__ rank_in_block,
+                                                        int32_t* __restrict__ block_hist,
                                                         int32_t* __restrict__ slot_of_row,
                                                         int32_t* __restrict__ token_of_row, int row_capacity) {
   extern __shared__ int32_t cnt[];  // [4][E]
@@ -41,10 +44,12 @@ __global__ __launch_bounds__(256) void plan_rank_kernel(const int64_t* __restric
   for (int e = lane; e < E; e += kWave) my[e] = 0;
   __syncthreads();
 
-  const int gw = blockIdx.x * kWavesPerBlock + wave;
-  const int begin = gw * kSlotsPerWave;
-  for (int c = 0; c < kSlotsPerWave; c += kWave) {
-    const int slot = begin + c + lane;
+  const int begin = (blockIdx.x * kWavesPerBlock + wave) * kSlotsPerWave;
+  constexpr int kChunks = kSlotsPerWave / kWave;
+  int e_of[kChunks], rank_of[kChunks];
+#pragma unroll
+  for (int c = 0; c < kChunks; ++c) {
+    const int slot = begin + c * kWave + lane;
     const bool valid = slot < N;
     int e = valid ? static_cast<int>(ids[slot]) : -1;
     if (e < 0 || e >= E) e = -1;  // an id outside [0, E) is not counted and gets no row
@@ -58,23 +63,39 @@ __global__ __launch_bounds__(256) void plan_rank_kernel(const int64_t* __restric
       below += (j < lane) ? same : 0;
       above += (j > lane) ? same : 0;
     }
+    e_of[c] = e;
+    rank_of[c] = 0;
     if (e >= 0) {
       const int base = my[e];
-      rank_in_wave[slot] = base + below;
+      rank_of[c] = base + below;
       __builtin_amdgcn_wave_barrier();
       if (above == 0) my[e] = base + below + 1;  // one writer per expert: its highest lane
     }
     __builtin_amdgcn_wave_barrier();
   }
   __syncthreads();
-  for (int e = lane; e < E; e += kWave) wave_hist[static_cast<int64_t>(gw) * E + e] = my[e];
+  // the slots of the waves before this one in the workgroup come first
+#pragma unroll
+  for (int c = 0; c < kChunks; ++c) {
+    const int e = e_of[c];
+    if (e < 0) continue;
+    int before = 0;
+    for (int w = 0; w < wave; ++w) before += cnt[w * E + e];
+    rank_in_block[begin + c * kWave + lane] = rank_of[c] + before;
+  }
+  for (int e = threadIdx.x; e < E; e += 256) {
+    int sum = 0;
+#pragma unroll
+    for (int w = 0; w < kWavesPerBlock; ++w) sum += cnt[w * E + e];
+    block_hist[static_cast<int64_t>(blockIdx.x) * E + e] = sum;
+  }
 }
 
-// One workgroup of 1024 lanes.  The per-expert scan over the wave histograms is
-// split into `parts` contiguous ranges of waves so its loads pipeline: pass 1 sums
+// One workgroup of 1024 lanes.  The per-expert scan over the workgroup histograms of
+// plan_rank is split into `parts` contiguous ranges so its loads pipeline: pass 1 sums
 // each range, a short serial scan joins them, pass 2 writes the exclusive prefixes.
 __global__ __launch_bounds__(1024) void plan_scan_kernel(
-    const int32_t* __restrict__ wave_hist, int32_t* __restrict__ wave_prefix, int num_waves, int E,
+    const int32_t* __restrict__ hist, int32_t* __restrict__ prefix, int num_hist, int E,
     int lo, int hi, int align, int tile_m, int32_t* __restrict__ counts_E,
     int32_t* __restrict__ seg_offsets, int32_t* __restrict__ seg_counts,
     int32_t* __restrict__ tile_expert, int32_t* __restrict__ tile_row0,
@@ -88,22 +109,21 @@ __global__ __launch_bounds__(1024) void plan_scan_kernel(
   int32_t* pad_sh = tile_off_sh + El + 1;      // El
   int32_t* nt_sh = pad_sh + El;                // El
   const int tid = threadIdx.x;
-  const int per = (num_waves + parts - 1) / parts;
+  const int per = (num_hist + parts - 1) / parts;
 
   for (int idx = tid; idx < E * parts; idx += blockDim.x) {
     const int e = idx % E, part = idx / E;
-    const int w0 = part * per, w1 = min(num_waves, w0 + per);
+    const int w0 = part * per, w1 = min(num_hist, w0 + per);
     // sixteen loads in flight at a time: one at a time, each would wait out a full memory
     // round trip, and this workgroup has nothing else to hide it behind
-    int sum = 0, w = w0;
-    for (; w + kBatch <= w1; w += kBatch) {
+    int sum = 0;
+    for (int w = w0; w < w1; w += kBatch) {
       int v[kBatch];
 #pragma unroll
-      for (int i = 0; i < kBatch; ++i) v[i] = wave_hist[static_cast<int64_t>(w + i) * E + e];
+      for (int i = 0; i < kBatch; ++i) v[i] = w + i < w1 ? hist[static_cast<int64_t>(w + i) * E + e] : 0;
 #pragma unroll
       for (int i = 0; i < kBatch; ++i) sum += v[i];
     }
-    for (; w < w1; ++w) sum += wave_hist[static_cast<int64_t>(w) * E + e];
     part_sum[part * E + e] = sum;
   }
   __syncthreads();
@@ -121,52 +141,59 @@ __global__ __launch_bounds__(1024) void plan_scan_kernel(
   __syncthreads();
   for (int idx = tid; idx < E * parts; idx += blockDim.x) {
     const int e = idx % E, part = idx / E;
-    const int w0 = part * per, w1 = min(num_waves, w0 + per);
-    int run = part_sum[part * E + e], w = w0;
-    for (; w + kBatch <= w1; w += kBatch) {
+    const int w0 = part * per, w1 = min(num_hist, w0 + per);
+    int run = part_sum[part * E + e];
+    for (int w = w0; w < w1; w += kBatch) {
       int v[kBatch];
 #pragma unroll
-      for (int i = 0; i < kBatch; ++i) v[i] = wave_hist[static_cast<int64_t>(w + i) * E + e];
+      for (int i = 0; i < kBatch; ++i) v[i] = w + i < w1 ? hist[static_cast<int64_t>(w + i) * E + e] : 0;
 #pragma unroll
       for (int i = 0; i < kBatch; ++i) {
-        wave_prefix[static_cast<int64_t>(w + i) * E + e] = run;
+        if (w + i < w1) prefix[static_cast<int64_t>(w + i) * E + e] = run;
         run += v[i];
       }
     }
-    for (; w < w1; ++w) {
-      const int64_t i = static_cast<int64_t>(w) * E + e;
-      wave_prefix[i] = run;
-      run += wave_hist[i];
-    }
   }
-  // padded rows and tiles per local expert, then every lane sums what lies before its
-  // expert: El broadcast LDS reads per lane, no serial chain (a one-lane scan with its two
-  // integer divisions per expert took longer than everything else in this kernel)
+  // padded rows and tiles per local expert; then, for every expert (and one past the last), what
+  // lies before it.  Each of these El + 1 sums runs over all El experts: the lanes of the
+  // workgroup share them, several lanes per sum over a slice of the experts each, joined by
+  // integer adds in LDS (with one lane per sum -- 129 busy lanes of 1024, 128 rounds of LDS
+  // reads each -- this step was half of the kernel's time).
+  int32_t* rank_sh = nt_sh + El;  // El + 1
   for (int j = tid; j < El; j += blockDim.x) {
     const int c = cnt_sh[lo + j];
     pad_sh[j] = c + ((align - (c % align)) % align);
     nt_sh[j] = (c + tile_m - 1) / tile_m;
   }
+  for (int j = tid; j <= El; j += blockDim.x) seg_off_sh[j] = tile_off_sh[j] = rank_sh[j] = 0;
   __syncthreads();
   // ... and its place among the local experts by descending row count (ties to the lower
   // index): the order in which the weight-gradient kernels start their tiles, longest
   // contraction first
-  for (int j = tid; j <= El; j += blockDim.x) {
+  const int sums = El + 1;
+  const int lanes_per_sum = max(1, static_cast<int>(blockDim.x) / sums);
+  const int slice = (El + lanes_per_sum - 1) / lanes_per_sum;
+  for (int idx = tid; idx < sums * lanes_per_sum; idx += blockDim.x) {
+    const int j = idx % sums, o0 = (idx / sums) * slice, o1 = min(El, o0 + slice);
     const int c = j < El ? cnt_sh[lo + j] : 0;
     int off = 0, toff = 0, rank = 0;
-    for (int o = 0; o < El; ++o) {
+#pragma unroll 4
+    for (int o = o0; o < o1; ++o) {
       const bool before = o < j;
       off += before ? pad_sh[o] : 0;
       toff += before ? nt_sh[o] : 0;
       const int co = cnt_sh[lo + o];
       rank += (co > c || (co == c && before)) ? 1 : 0;
     }
-    seg_off_sh[j] = off;
-    tile_off_sh[j] = toff;
-    if (j < El) seg_counts[El + rank] = j;
-    else *num_tiles = toff < tile_capacity ? toff : tile_capacity;
+    atomicAdd(&seg_off_sh[j], off);
+    atomicAdd(&tile_off_sh[j], toff);
+    atomicAdd(&rank_sh[j], rank);
   }
   __syncthreads();
+  for (int j = tid; j <= El; j += blockDim.x) {
+    if (j < El) seg_counts[El + rank_sh[j]] = j;
+    else *num_tiles = tile_off_sh[j] < tile_capacity ? tile_off_sh[j] : tile_capacity;
+  }
   for (int j = tid; j <= El; j += blockDim.x) seg_offsets[j] = seg_off_sh[j];
   for (int j = tid; j < El; j += blockDim.x) {
     const int c = cnt_sh[lo + j];
@@ -202,7 +229,8 @@ __global__ __launch_bounds__(256) void segments_from_counts_kernel(
   __syncthreads();
   for (int j = tid; j <= El; j += blockDim.x) {
     int64_t before = 0;
-    for (int o = 0; o < j; ++o) before += raw_sh[o];
+#pragma unroll 16
+    for (int o = 0; o < El; ++o) before += o < j ? raw_sh[o] : 0;
     const int off = static_cast<int>(min(before, static_cast<int64_t>(row_capacity)));
     seg_off_sh[j] = off;
     if (j < El) cnt_sh[j] = min(raw_sh[j], row_capacity - off);
@@ -213,6 +241,7 @@ __global__ __launch_bounds__(256) void segments_from_counts_kernel(
   for (int j = tid; j <= El; j += blockDim.x) {
     const int c = j < El ? cnt_sh[j] : 0;
     int toff = 0, rank = 0;
+#pragma unroll 16
     for (int o = 0; o < El; ++o) {
       const int co = cnt_sh[o];
       const bool before = o < j;
@@ -250,8 +279,8 @@ __global__ void fill_i32_kernel(int32_t* p, int32_t* q, int64_t n, int32_t v) {
 }
 
 __global__ __launch_bounds__(256) void plan_rows_kernel(
-    const int64_t* __restrict__ ids, const int32_t* __restrict__ rank_in_wave,
-    const int32_t* __restrict__ wave_prefix, const int32_t* __restrict__ seg_offsets, int N, int E,
+    const int64_t* __restrict__ ids, const int32_t* __restrict__ rank_in_block,
+    const int32_t* __restrict__ block_prefix, const int32_t* __restrict__ seg_offsets, int N, int E,
     int lo, int hi, int K, int32_t* __restrict__ row_of_slot, int32_t* __restrict__ slot_of_row,
     int32_t* __restrict__ token_of_row, int row_capacity) {
   const int slot = blockIdx.x * blockDim.x + threadIdx.x;
@@ -259,8 +288,8 @@ __global__ __launch_bounds__(256) void plan_rows_kernel(
   const int e = static_cast<int>(ids[slot]);  // outside [0, E): outside [lo, hi) too, no row
   int row = -1;
   if (e >= lo && e < hi) {
-    const int gw = slot / kSlotsPerWave;
-    row = seg_offsets[e - lo] + wave_prefix[static_cast<int64_t>(gw) * E + e] + rank_in_wave[slot];
+    const int blk = slot / kSlotsPerBlock;
+    row = seg_offsets[e - lo] + block_prefix[static_cast<int64_t>(blk) * E + e] + rank_in_block[slot];
     if (row >= 0 && row < row_capacity) {
       slot_of_row[row] = slot;
       if (token_of_row) token_of_row[row] = slot / K;
@@ -429,13 +458,12 @@ __global__ __launch_bounds__(256) void permute_rows_bwd_kernel(
 
 using namespace mi355;
 
-static int64_t plan_num_waves(int64_t N) { return (N + kSlotsPerWave - 1) / kSlotsPerWave; }
 static int64_t plan_num_blocks(int64_t N) { return (N + kSlotsPerBlock - 1) / kSlotsPerBlock; }
 
 extern "C" int64_t mi355_permute_plan_workspace_bytes(int64_t T, int64_t K, int64_t E) {
   const int64_t N = T * K;
-  // rank_in_wave[N] + wave_hist[blocks*4][E] + wave_prefix[blocks*4][E]
-  return (N + 2 * plan_num_blocks(N) * kWavesPerBlock * E + 64) * (int64_t)sizeof(int32_t);
+  // rank_in_block[N] + block_hist[blocks][E] + block_prefix[blocks][E]
+  return (N + 2 * plan_num_blocks(N) * E + 64) * (int64_t)sizeof(int32_t);
 }
 
 static int plan_impl(const int64_t* ids, int64_t T, int64_t K, int64_t E, int64_t lo, int64_t hi, int64_t align,
@@ -446,7 +474,7 @@ static int plan_impl(const int64_t* ids, int64_t T, int64_t K, int64_t E, int64_
   const int64_t N = T * K;
   MI355_REQUIRE(T >= 0 && K >= 1 && E >= 1 && N < (1ll << 30), "permute_plan: bad shape T=%lld K=%lld E=%lld",
                 (long long)T, (long long)K, (long long)E);
-  // (the scan workgroup keeps (parts + 1) * E + 4 * El + 2 words in LDS: 48 KiB at E = 2048)
+  // (the scan workgroup keeps (parts + 1) * E + 5 * El + 3 words in LDS: 56 KiB at E = 2048)
   MI355_REQUIRE(E <= 2048, "permute_plan: E=%lld exceeds 2048", (long long)E);
   MI355_REQUIRE(0 <= lo && lo < hi && hi <= E, "permute_plan: bad local range [%lld,%lld)", (long long)lo, (long long)hi);
   MI355_REQUIRE(align >= 1 && tile_m >= 1, "permute_plan: align and tile_m must be positive");
@@ -456,13 +484,12 @@ static int plan_impl(const int64_t* ids, int64_t T, int64_t K, int64_t E, int64_
                 "permute_plan: null pointer");
   MI355_REQUIRE(N == 0 || (ids && row_of_slot), "permute_plan: null pointer");
   MI355_REQUIRE(row_capacity == 0 || slot_of_row, "permute_plan: null slot_of_row");
-  int32_t* rank_in_wave = static_cast<int32_t*>(workspace);
-  int32_t* wave_hist = rank_in_wave + N;
+  int32_t* rank_in_block = static_cast<int32_t*>(workspace);
+  int32_t* block_hist = rank_in_block + N;
   const int nblocks = (int)plan_num_blocks(N);
-  const int nwaves = nblocks * kWavesPerBlock;
   if (nblocks > 0) {
     hipLaunchKernelGGL(plan_rank_kernel, dim3(nblocks), dim3(256), (size_t)kWavesPerBlock * E * 4, s,
-                       ids, (int)N, (int)E, rank_in_wave, wave_hist, slot_of_row, token_of_row, (int)row_capacity);
+                       ids, (int)N, (int)E, rank_in_block, block_hist, slot_of_row, token_of_row, (int)row_capacity);
     if (int rc = check_launch("plan_rank")) return rc;
   } else if (row_capacity > 0) {  // no slots at all: only the fill is left to do
     hipLaunchKernelGGL(fill_i32_kernel, dim3((unsigned)((row_capacity + 255) / 256)), dim3(256), 0, s,
@@ -470,18 +497,18 @@ static int plan_impl(const int64_t* ids, int64_t T, int64_t K, int64_t E, int64_
     if (int rc = check_launch("plan_fill")) return rc;
   }
   const int El = (int)(hi - lo);
-  int32_t* wave_prefix = wave_hist + (int64_t)nwaves * E;
+  int32_t* block_prefix = block_hist + (int64_t)nblocks * E;
   int parts = (int)(1024 / E);
   if (parts < 1) parts = 1;
   if (parts > 16) parts = 16;
   hipLaunchKernelGGL(plan_scan_kernel, dim3(1), dim3(1024),
-                     (size_t)((parts + 1) * E + 4 * El + 2) * 4, s, wave_hist, wave_prefix, nwaves,
+                     (size_t)((parts + 1) * E + 5 * El + 3) * 4, s, block_hist, block_prefix, nblocks,
                      (int)E, (int)lo, (int)hi, (int)align, (int)tile_m, counts_E, seg_offsets,
                      seg_counts, tile_expert, tile_row0, num_tiles, (int)tile_capacity, parts);
   if (int rc = check_launch("plan_scan")) return rc;
   if (N > 0) {
     hipLaunchKernelGGL(plan_rows_kernel, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, s, ids,
-                       rank_in_wave, wave_prefix, seg_offsets, (int)N, (int)E, (int)lo, (int)hi, (int)K,
+                       rank_in_block, block_prefix, seg_offsets, (int)N, (int)E, (int)lo, (int)hi, (int)K,
                        row_of_slot, slot_of_row, token_of_row, (int)row_capacity);
     if (int rc = check_launch("plan_rows")) return rc;
   }
@@ -502,7 +529,7 @@ extern "C" int mi355_permute_plan(const int64_t* ids, int64_t T, int64_t K, int6
 
 // ---- the same plan without a caller-provided workspace -------------------------------------
 // For callers that cannot allocate (under HIP graph capture, in a tight serving loop): the
-// ranks and per-wave histograms live in a file-scope device array, 8 MiB per GPU, held until
+// ranks and per-workgroup histograms live in a file-scope device array, 8 MiB per GPU, held until
 // the process ends.  The array's name is a host-side stand-in, not a device address: its
 // address on each device is asked for once, with that device current, and only that pointer
 // is ever handed to kernels.  Every call on a GPU shares that GPU's array: calls that overlap

@@ -72,6 +72,39 @@ __device__ __forceinline__ void wave_argmax(float& v, int& idx) {
   idx = ai;
 }
 
+// the two largest of {a1 >= a2} and {b1 >= b2}, equal values counted as often as they occur
+__device__ __forceinline__ void merge_top2(float& a1, float& a2, float b1, float b2) {
+  const float lo = fminf(a1, b1);
+  a1 = fmaxf(a1, b1);
+  a2 = fmaxf(lo, fmaxf(a2, b2));
+}
+template <int CTRL>
+__device__ __forceinline__ void top2_dpp(float& m1, float& m2) {
+  const float o1 = dpp_f32<CTRL>(m1), o2 = dpp_f32<CTRL>(m2);
+  merge_top2(m1, m2, o1, o2);
+}
+// The two largest values held by the `width` lanes (a power of two, 2..64; wave-uniform) of every
+// aligned run of lanes, left in all of them.  Each step exchanges between two halves that already
+// agree among themselves, so the mirrors of the DPP controls are as good as a butterfly.
+__device__ __forceinline__ void run_top2(float& m1, float& m2, int width) {
+  top2_dpp<kDppPairs>(m1, m2);
+  if (width >= 4) top2_dpp<kDppQuads>(m1, m2);
+  if (width >= 8) top2_dpp<kDppHalfMirror>(m1, m2);
+  if (width >= 16) top2_dpp<kDppRowMirror>(m1, m2);
+  if (width >= 32) {
+    // lane ^ 16 within each half of the wave (swizzle bit mode: and 0x1f, or 0, xor 0x10)
+    const float o1 = __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(m1), 0x401f));
+    const float o2 = __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(m2), 0x401f));
+    merge_top2(m1, m2, o1, o2);
+  }
+  if (width >= 64) {
+    float a1 = lane_f32(m1, 0), a2 = lane_f32(m2, 0);
+    merge_top2(a1, a2, lane_f32(m1, 32), lane_f32(m2, 32));
+    m1 = a1;
+    m2 = a2;
+  }
+}
+
 template <int VPL>
 __device__ __forceinline__ float pick(const float (&a)[VPL], int j) {
   float r = a[0];
@@ -155,35 +188,65 @@ __global__ __launch_bounds__(256) void select_fwd_kernel(
       // num_limited groups (ties to the lower group), mask the rest to -inf.
       const int P = E / num_groups;
       float gscore = -INFINITY;  // lane g (< num_groups) keeps group g's score
-      for (int g = 0; g < num_groups; ++g) {
-        float top2 = 0.0f;
-        unsigned used = 0;
-        for (int r = 0; r < 2; ++r) {
-          float bv = -INFINITY;
-          int bi = 0x7fffffff;
+      if (P < kWave && kWave % P == 0) {
+        // a group is an aligned run of P lanes of one register: the registers' runs are reduced side
+        // by side (independent chains), then lane g fetches the sum of its group's run
+        const int runs = kWave / P;  // groups per register
+        float sum[VPL];
 #pragma unroll
-          for (int j = 0; j < VPL; ++j) {
-            const int e = lane + j * kWave;
-            const bool in = e < E && e / P == g && !((used >> j) & 1u);
-            if (in && (c[j] > bv || bi == 0x7fffffff)) { bv = c[j]; bi = e; }
-          }
-          wave_argmax(bv, bi);
-          top2 += bv;
-          if ((bi & 63) == lane) used |= 1u << (bi >> 6);
+        for (int j = 0; j < VPL; ++j) {
+          float m1 = c[j], m2 = -INFINITY;
+          run_top2(m1, m2, P);
+          sum[j] = m1 + m2;
         }
-        if (lane == g) gscore = top2;
+        const int from = (lane % runs) * P;
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) {
+          const float got = __int_as_float(__builtin_amdgcn_ds_bpermute(from << 2, __float_as_int(sum[j])));
+          if (lane / runs == j) gscore = got;
+        }
+      } else if (P % kWave == 0) {
+        // a group is P / 64 whole registers: each lane folds its own values, then one wave-wide step
+        const int regs = P / kWave;
+        float m1 = -INFINITY, m2 = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) {
+          merge_top2(m1, m2, c[j], -INFINITY);
+          if ((j + 1) % regs == 0) {
+            run_top2(m1, m2, kWave);
+            if (lane == j / regs) gscore = m1 + m2;
+            m1 = m2 = -INFINITY;
+          }
+        }
+      } else {
+        for (int g = 0; g < num_groups; ++g) {
+          float top2 = 0.0f;
+          unsigned used = 0;
+          for (int r = 0; r < 2; ++r) {
+            float bv = -INFINITY;
+            int bi = 0x7fffffff;
+#pragma unroll
+            for (int j = 0; j < VPL; ++j) {
+              const int e = lane + j * kWave;
+              const bool in = e < E && e / P == g && !((used >> j) & 1u);
+              if (in && (c[j] > bv || bi == 0x7fffffff)) { bv = c[j]; bi = e; }
+            }
+            wave_argmax(bv, bi);
+            top2 += bv;
+            if ((bi & 63) == lane) used |= 1u << (bi >> 6);
+          }
+          if (lane == g) gscore = top2;
+        }
       }
-      unsigned long long keep = 0;  // bit g set = group kept
-      float gs = gscore;
-      for (int r = 0; r < num_limited; ++r) {
-        float bv = gs;
-        int bi = lane < num_groups ? lane : 0x7fffffff;
-        if (lane >= num_groups) bv = -INFINITY;
-        // lanes already chosen drop out
-        if ((keep >> lane) & 1ull) { bv = -INFINITY; bi = 0x7fffffff; }
-        wave_argmax(bv, bi);
-        keep |= 1ull << bi;
+      // a group is kept when fewer than num_limited groups beat it (a higher score, or the same
+      // score and a lower index): the groups a repeated arg-max would pick, without the repeats
+      const float mine = lane < num_groups ? gscore : -INFINITY;
+      int beaten_by = 0;
+      for (int g = 0; g < num_groups; ++g) {
+        const float sg = lane_f32(gscore, g);
+        beaten_by += (sg > mine || (sg == mine && g < lane)) ? 1 : 0;
       }
+      const unsigned long long keep = __ballot(lane < num_groups && beaten_by < num_limited);
 #pragma unroll
       for (int j = 0; j < VPL; ++j) {
         const int e = lane + j * kWave;
