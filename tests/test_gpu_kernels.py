@@ -65,6 +65,10 @@ SELECT_CASES = [
     dict(T=1024, E=256, K=8, score_func="sigmoid", route_norm=True, route_scale=2.5,
          num_expert_groups=8, num_limited_groups=4, bias=True),
     dict(T=300, E=64, K=6, score_func="sigmoid", bias=True),
+    # the 16-lanes-per-token kernel at its other widths and its K limits
+    dict(T=333, E=256, K=16, score_func="sqrtsoftplus", route_norm=True, bias=True),
+    dict(T=77, E=128, K=1, score_func="softmax"),
+    dict(T=100, E=256, K=17, score_func="softmax", route_norm=True),
     dict(T=300, E=24, K=3, score_func="sqrtsoftplus", route_norm=True, route_scale=0.5),
     dict(T=257, E=320, K=5, score_func="softmax", num_expert_groups=5, num_limited_groups=2),
     # groups of 2, 16, 24 (no aligned lane run), 128 (two registers per lane) experts
@@ -73,6 +77,9 @@ SELECT_CASES = [
     dict(T=300, E=96, K=4, score_func="sigmoid", num_expert_groups=4, num_limited_groups=2, bias=True),
     dict(T=300, E=256, K=8, score_func="softmax", route_norm=True, num_expert_groups=2, num_limited_groups=1),
     dict(T=300, E=512, K=8, score_func="sigmoid", num_expert_groups=4, num_limited_groups=2, bias=True),
+    # one lane per group and one group in all, in the 16-lanes-per-token kernel
+    dict(T=300, E=64, K=4, score_func="sigmoid", route_norm=True, num_expert_groups=16, num_limited_groups=4, bias=True),
+    dict(T=300, E=128, K=5, score_func="softmax", num_expert_groups=1, num_limited_groups=1),
     dict(T=10, E=4, K=2, score_func="sigmoid", fixed_router=True, route_scale=7.0),
     dict(T=10, E=4, K=2, score_func="sigmoid", debug_force_load_balance=True, route_norm=True, route_scale=2.0),
 ]
@@ -145,6 +152,19 @@ def test_router_select_exact_ties_go_to_lower_index(ops):
         w, ids, _ = ops.router_select_fwd(logits.to(DEV), None, 4, fn, False, 1.0)
         assert ids[0].tolist() == [0, 1, 2, 3]
         assert ids[1].tolist() == [3, 9, 0, 1]
+    # the same rule at the widths served by the 16-lanes-per-token kernel; the routing map and the
+    # cutoff (the best score left) follow the same choice
+    for E in (64, 128, 256):
+        logits = torch.zeros(19, E)
+        logits[1, 3] = logits[1, E - 7] = 1.0
+        logits[2, E - 1] = 2.0
+        for fn in ("softmax", "sigmoid", "sqrtsoftplus"):
+            w, ids, _, rmap = ops.router_select_fwd(logits.to(DEV), None, 4, fn, True, 1.0, 0, 0, 0, False, True)
+            assert ids[0].tolist() == [0, 1, 2, 3] and ids[18].tolist() == [0, 1, 2, 3]
+            assert ids[1].tolist() == [3, E - 7, 0, 1]
+            assert ids[2].tolist() == [E - 1, 0, 1, 2]
+            assert torch.equal(rmap.cpu(), torch.zeros(19, E, dtype=torch.bool).scatter_(-1, ids.cpu(), True))
+            assert torch.allclose(w.sum(-1).cpu(), torch.ones(19), atol=1e-6)
     # grouped known answer: tests/unit_tests/cpu/models/test_models_common.py:157-165
     s = torch.tensor([[0.80, 0.70, 0.00, 0.00, 0.90, 0.20, 0.00, 0.00]])
     lg = torch.log(s.clamp_min(1e-6) / (1 - s).clamp_min(1e-6))  # sigmoid^-1

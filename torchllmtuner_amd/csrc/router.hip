@@ -5,6 +5,8 @@
 // and every arg-max are wave-level shuffle reductions, and the K winners are
 // written by lanes 0..K-1.  No LDS, no atomics; HBM traffic is the (T,E) logits
 // once plus the (T,K) outputs.
+#include <type_traits>
+
 #include "common.h"
 #include "gemm_generic.h"
 
@@ -12,6 +14,7 @@ namespace mi355 {
 namespace {
 
 constexpr int kMaxVPL = 8;  // experts per lane -> E <= 512
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ float softplus_f32(float x) {
   return x > 20.0f ? x : log1pf(expf(x));  // torch's threshold=20, beta=1
@@ -323,6 +326,208 @@ __global__ __launch_bounds__(256) void select_fwd_kernel(
   }
 }
 
+// ---- the same selection with one token per row of 16 lanes -------------------------------------
+// For E = 64, 128 or 256, K <= 16 and 1, 2, 4, 8 or 16 expert groups (or none): four tokens per
+// wavefront, lane l of a row keeps experts l*VPR .. l*VPR + VPR - 1, so a group is a run of
+// 16 / num_groups whole lanes.  Every reduction is four
+// DPP steps inside the row and serves four tokens at once, where the wave-per-token kernel above
+// spends the same steps plus eight lane reads on one: the selection is bound by instruction
+// issue, not by memory, and this form issues about a third of the instructions per token.  The
+// choice (larger value, ties to the lower expert index) does not depend on the order of the
+// comparisons, so both kernels pick the same experts.
+__device__ __forceinline__ float row_max(float v) {
+  v = fmaxf(v, dpp_f32<kDppPairs>(v));
+  v = fmaxf(v, dpp_f32<kDppQuads>(v));
+  v = fmaxf(v, dpp_f32<kDppHalfMirror>(v));
+  return fmaxf(v, dpp_f32<kDppRowMirror>(v));
+}
+__device__ __forceinline__ float row_sum(float v) {
+  v += dpp_f32<kDppPairs>(v);
+  v += dpp_f32<kDppQuads>(v);
+  v += dpp_f32<kDppHalfMirror>(v);
+  return v + dpp_f32<kDppRowMirror>(v);
+}
+template <int CTRL>
+__device__ __forceinline__ void row_better(float& v, int& idx, float& carried) {
+  const float ov = dpp_f32<CTRL>(v), oc = dpp_f32<CTRL>(carried);
+  const int oi = dpp_i32<CTRL>(idx);
+  if (ov > v || (ov == v && oi < idx)) { v = ov; idx = oi; carried = oc; }
+}
+// (value, index) arg-max over a row, with a value carried along from the winner; left in all 16 lanes
+__device__ __forceinline__ void row_argmax(float& v, int& idx, float& carried) {
+  row_better<kDppPairs>(v, idx, carried);
+  row_better<kDppQuads>(v, idx, carried);
+  row_better<kDppHalfMirror>(v, idx, carried);
+  row_better<kDppRowMirror>(v, idx, carried);
+}
+
+template <int VPR>
+__global__ __launch_bounds__(256) void select_rows_kernel(
+    const float* __restrict__ logits, const float* __restrict__ expert_bias, float* __restrict__ weights,
+    int64_t* __restrict__ ids, float* __restrict__ scores_out, uint8_t* __restrict__ map_out,
+    float* __restrict__ cutoff_out, int T, int K, int score_func, int route_norm, float route_scale,
+    int num_groups, int num_limited) {
+  constexpr int E = 16 * VPR;
+  const int l = threadIdx.x & 15;
+  const int t_raw = blockIdx.x * 16 + (threadIdx.x >> 4);
+  const bool live = t_raw < T;
+  const int t = live ? t_raw : T - 1;  // a row past the end redoes the last token and stores nothing
+  const int e0 = l * VPR;
+
+  float x[VPR], s[VPR];
+  const f32x4* src = reinterpret_cast<const f32x4*>(logits + static_cast<int64_t>(t) * E + e0);
+#pragma unroll
+  for (int q = 0; q < VPR / 4; ++q) {
+    const f32x4 v = src[q];
+    x[q * 4] = v[0]; x[q * 4 + 1] = v[1]; x[q * 4 + 2] = v[2]; x[q * 4 + 3] = v[3];
+  }
+  if (score_func == MI355_SCORE_SOFTMAX) {
+    float m = x[0];
+#pragma unroll
+    for (int j = 1; j < VPR; ++j) m = fmaxf(m, x[j]);
+    m = row_max(m);
+    float sum = 0.0f;
+#pragma unroll
+    for (int j = 0; j < VPR; ++j) {
+      s[j] = expf(x[j] - m);
+      sum += s[j];
+    }
+    sum = row_sum(sum);
+#pragma unroll
+    for (int j = 0; j < VPR; ++j) s[j] = s[j] / sum;
+  } else if (score_func == MI355_SCORE_SIGMOID) {
+#pragma unroll
+    for (int j = 0; j < VPR; ++j) s[j] = 1.0f / (1.0f + expf(-x[j]));
+  } else {
+#pragma unroll
+    for (int j = 0; j < VPR; ++j) s[j] = sqrtf(softplus_f32(x[j]));
+  }
+  if (scores_out && live) {
+    f32x4* dst = reinterpret_cast<f32x4*>(scores_out + static_cast<int64_t>(t) * E + e0);
+#pragma unroll
+    for (int q = 0; q < VPR / 4; ++q) {
+      const f32x4 v = {s[q * 4], s[q * 4 + 1], s[q * 4 + 2], s[q * 4 + 3]};
+      dst[q] = v;
+    }
+  }
+
+  // choice values: the logit itself when nothing but a monotone score function stands between
+  // it and the choice (exact: two exp() implementations can order two nearly equal scores
+  // differently, never two logits), else score (+ bias)
+  float c[VPR];
+  if (expert_bias) {
+    const f32x4* bsrc = reinterpret_cast<const f32x4*>(expert_bias + e0);
+#pragma unroll
+    for (int q = 0; q < VPR / 4; ++q) {
+      const f32x4 b = bsrc[q];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) c[q * 4 + i] = s[q * 4 + i] + b[i];
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < VPR; ++j) c[j] = num_groups > 0 ? s[j] : x[j];
+  }
+  if (num_groups > 0) {
+    // group score = sum of the group's two best choice values: each lane folds its own, the lanes
+    // of a group join them; every lane then counts the groups that beat its own (a higher score,
+    // or the same score and a lower index), seeing each other group's score by a row rotation,
+    // and a group beaten by num_limited others or more is masked
+    const int m = 16 / num_groups;  // lanes per group
+    float m1 = -INFINITY, m2 = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < VPR; ++j) merge_top2(m1, m2, c[j], -INFINITY);
+    if (m >= 2) top2_dpp<kDppPairs>(m1, m2);
+    if (m >= 4) top2_dpp<kDppQuads>(m1, m2);
+    if (m >= 8) top2_dpp<kDppHalfMirror>(m1, m2);
+    if (m >= 16) top2_dpp<kDppRowMirror>(m1, m2);
+    const float gs = m1 + m2;
+    const int gid = l / m;
+    int beaten_by = 0;
+    auto other = [&](auto n_t) {
+      constexpr int n = decltype(n_t)::value;
+      if (n % m != 0) return;  // wave-uniform
+      const float og = dpp_f32<0x120 + n>(gs);  // row rotation by n lanes
+      const int oi = dpp_i32<0x120 + n>(gid);
+      beaten_by += (og > gs || (og == gs && oi < gid)) ? 1 : 0;
+    };
+    other(std::integral_constant<int, 1>{}); other(std::integral_constant<int, 2>{});
+    other(std::integral_constant<int, 3>{}); other(std::integral_constant<int, 4>{});
+    other(std::integral_constant<int, 5>{}); other(std::integral_constant<int, 6>{});
+    other(std::integral_constant<int, 7>{}); other(std::integral_constant<int, 8>{});
+    other(std::integral_constant<int, 9>{}); other(std::integral_constant<int, 10>{});
+    other(std::integral_constant<int, 11>{}); other(std::integral_constant<int, 12>{});
+    other(std::integral_constant<int, 13>{}); other(std::integral_constant<int, 14>{});
+    other(std::integral_constant<int, 15>{});
+    if (beaten_by >= num_limited) {
+#pragma unroll
+      for (int j = 0; j < VPR; ++j) c[j] = -INFINITY;
+    }
+  }
+
+  unsigned taken = 0;
+  float my_w = 0.0f;
+  int my_id = 0;
+  auto best_left = [&](float& bv, int& bi, float& bs) {
+    bv = -INFINITY;
+    bi = 0x7fffffff;
+    bs = 0.0f;
+#pragma unroll
+    for (int j = 0; j < VPR; ++j) {
+      if ((taken >> j) & 1u) continue;
+      if (bi == 0x7fffffff || c[j] > bv) { bv = c[j]; bi = e0 + j; bs = s[j]; }
+    }
+    row_argmax(bv, bi, bs);
+  };
+  for (int k = 0; k < K; ++k) {
+    float bv, bs;
+    int bi;
+    best_left(bv, bi, bs);
+    if (bi / VPR == l) taken |= 1u << (bi % VPR);
+    if (l == k) { my_w = bs; my_id = bi; }
+  }
+  if (cutoff_out) {
+    // the best choice value left after the K winners: the (K+1)-th of a sorted top-(K+1)
+    float bv, bs;
+    int bi;
+    best_left(bv, bi, bs);
+    if (l == 0 && live) cutoff_out[t] = bv;
+  }
+  if (route_norm) {
+    const float sum = row_sum(l < K ? my_w : 0.0f);
+    my_w = my_w / (sum + 1e-20f);
+  }
+  my_w = my_w * route_scale;
+  if (l < K && live) {
+    weights[static_cast<int64_t>(t) * K + l] = my_w;
+    ids[static_cast<int64_t>(t) * K + l] = my_id;
+  }
+  if (map_out && live) {
+    // one-hot routing map of the token, one byte per expert: this lane's VPR experts, four bytes a store
+    uint32_t* dst = reinterpret_cast<uint32_t*>(map_out + static_cast<int64_t>(t) * E + e0);
+#pragma unroll
+    for (int q = 0; q < VPR / 4; ++q) {
+      const unsigned b = taken >> (q * 4);
+      dst[q] = (b & 1u) | ((b & 2u) << 7) | ((b & 4u) << 14) | ((b & 8u) << 21);
+    }
+  }
+}
+
+// whether select_rows_kernel serves this call
+inline bool select_rows_ok(const float* logits, const float* bias, const float* scores, const uint8_t* map,
+                           int64_t E, int64_t K, int num_groups, int mode) {
+  return mode == MI355_SELECT_TOPK && (num_groups == 0 || (num_groups <= 16 && 16 % num_groups == 0)) && K <= 16 &&
+         (E == 64 || E == 128 || E == 256) &&
+         reinterpret_cast<uintptr_t>(logits) % 16 == 0 && reinterpret_cast<uintptr_t>(bias) % 16 == 0 &&
+         reinterpret_cast<uintptr_t>(scores) % 16 == 0 && reinterpret_cast<uintptr_t>(map) % 4 == 0;
+}
+template <typename... Args>
+void launch_select_rows(int64_t E, int64_t T, hipStream_t s, Args... args) {
+  const dim3 grid((unsigned)((T + 15) / 16));
+  if (E == 64) hipLaunchKernelGGL(select_rows_kernel<4>, grid, dim3(256), 0, s, args...);
+  else if (E == 128) hipLaunchKernelGGL(select_rows_kernel<8>, grid, dim3(256), 0, s, args...);
+  else hipLaunchKernelGGL(select_rows_kernel<16>, grid, dim3(256), 0, s, args...);
+}
+
 template <int VPL>
 __global__ __launch_bounds__(256) void select_bwd_kernel(
     const float* __restrict__ logits, const int64_t* __restrict__ ids,
@@ -528,6 +733,12 @@ extern "C" int mi355_router_select_fwd(const float* logits, const float* expert_
   }
   if (T == 0) return MI355_OK;
   MI355_REQUIRE(logits && weights && ids, "router_select_fwd: null pointer");
+  if (select_rows_ok(logits, expert_bias, scores_TE, routing_map_TE, E, K, num_groups, select_mode)) {
+    launch_select_rows(E, T, as_stream(stream), logits, expert_bias, weights, ids, scores_TE, routing_map_TE,
+                       static_cast<float*>(nullptr), (int)T, (int)K, score_func, route_norm, route_scale, num_groups,
+                       num_limited);
+    return check_launch("router_select_fwd");
+  }
   const dim3 grid((unsigned)((T + 3) / 4));
   DISPATCH_VPL(E, hipLaunchKernelGGL(select_fwd_kernel<VPL>, grid, dim3(256), 0, as_stream(stream),
                                      logits, expert_bias, weights, ids, scores_TE, routing_map_TE,
@@ -548,6 +759,12 @@ extern "C" int mi355_router_select_cutoff_fwd(const float* logits, const float* 
                 (long long)K, (long long)E);
   if (T == 0) return MI355_OK;
   MI355_REQUIRE(logits && weights && ids && cutoff_T, "router_select_cutoff_fwd: null pointer");
+  if (select_rows_ok(logits, expert_bias, scores_TE, nullptr, E, K, 0, MI355_SELECT_TOPK) &&
+      reinterpret_cast<uintptr_t>(cutoff_T) % 4 == 0) {
+    launch_select_rows(E, T, as_stream(stream), logits, expert_bias, weights, ids, scores_TE,
+                       static_cast<uint8_t*>(nullptr), cutoff_T, (int)T, (int)K, score_func, route_norm, route_scale, 0, 0);
+    return check_launch("router_select_cutoff_fwd");
+  }
   const dim3 grid((unsigned)((T + 3) / 4));
   DISPATCH_VPL(E, hipLaunchKernelGGL(select_fwd_kernel<VPL>, grid, dim3(256), 0, as_stream(stream),
                                      logits, expert_bias, weights, ids, scores_TE,
