@@ -1,10 +1,10 @@
 // Router: fp32 gate projection and the fused score / top-k / gather / norm pass.
 //
-// Selection kernel: one 64-lane wavefront owns one token.  Lane l keeps experts
-// l, l+64, l+128, ... in registers (coalesced logit loads), the softmax max / sum
-// and every arg-max are wave-level shuffle reductions, and the K winners are
-// written by lanes 0..K-1.  No LDS, no atomics; HBM traffic is the (T,E) logits
-// once plus the (T,K) outputs.
+// Selection kernels: a token is owned by one row of 16 lanes (E = 64, 128 or 256: four tokens
+// per wavefront, lane l keeps experts l*E/16 ...) or by one 64-lane wavefront (any E up to 512:
+// lane l keeps experts l, l+64, l+128, ...).  The scores stay in registers, the softmax max /
+// sum and every arg-max are DPP reductions, and the K winners are written by lanes 0..K-1.  No
+// LDS, no atomics; HBM traffic is the (T,E) logits once plus the (T,K) outputs.
 #include <type_traits>
 
 #include "common.h"
