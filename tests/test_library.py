@@ -177,3 +177,13 @@ def test_header_is_plain_c_and_links_against_the_library(tmp_path):
         check=True, capture_output=True)
     out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
     assert out == [str(len(names)), str(_lib.ABI_VERSION)]
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU: any other --gpus value exits with a message and no JSON line."""
+    import subprocess
+    import sys
+
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0
+    assert "one GPU" in (r.stdout + r.stderr) and "{" not in r.stdout
