@@ -388,6 +388,23 @@ def cpu_baseline(wl, sample_tokens):
     return out
 
 
+def swiglu_stage_bytes(rows, experts, D, F, s, saves_gate_up=True, dh_writes_scaled_h=True):
+    """Algorithmic HBM bytes of each grouped SwiGLU stage: every operand and every result once
+    (``rows`` routed rows or tokens, ``experts`` weight sets of (F, D), element size ``s``;
+    ``dh_writes_scaled_h``: the combine's backward is folded into dH, which then also writes
+    score * h for dW2)."""
+    x, a, w = rows * D * s, rows * F * s, experts * D * F * s
+    return {
+        "gate_up": x + 2 * w + (3 if saves_gate_up else 1) * a,  # rows, w1, w3 -> (gate, up,) h
+        "down": a + w + x,                                         # h, w2 -> y
+        "dh": x + w + 2 * a + (3 if dh_writes_scaled_h else 2) * a,  # dy, w2, gate, up -> dgate, dup(, score * h)
+        "drows": 2 * a + 2 * w + x,                                # dgate, dup, w1, w3 -> drows
+        "dw2": x + a + w,                                          # dy, h -> dW2
+        "dw1": x + a + w,                                          # rows, dgate -> dW1
+        "dw3": x + a + w,                                          # rows, dup -> dW3
+    }
+
+
 def per_kernel_times(args, wl, block, x, gout, dev):
     """HIP-event averages of the kernels of one step, each launched alone on the buffers of a
     real step.  Returns (kernels, stage_ms, stage_flops, routed_rows)."""
@@ -415,6 +432,8 @@ def per_kernel_times(args, wl, block, x, gout, dev):
                        "dw2": proj, "dw1": proj, "dw3": proj}
         if not wl.backward:
             stage_flops = {k: stage_flops[k] for k in ("gate_up", "down")}
+        n_local = (wl.local_experts[1] - wl.local_experts[0]) if wl.local_experts else E
+        stage_bytes = swiglu_stage_bytes(R_rows, n_local, D, F, s_bytes, saves_gate_up=wl.backward)
         stage_ms = {}
         folded = ops.gather_supported(x, F) and ops.combine_bwd_slots(x.dtype, D, F) > 0
         if folded:
@@ -454,7 +473,7 @@ def per_kernel_times(args, wl, block, x, gout, dev):
                                             wl.route_scale, wl.num_expert_groups or 0, wl.num_limited_groups or 0,
                                             want_map=True)
         lo, hi = wl.local_experts or (0, E)
-        shared_fns, shared_flops = {}, {}
+        shared_fns, shared_flops, shared_bytes = {}, {}, {}
         if wl.shared_hidden_dim and ops.gather_supported(x, wl.shared_hidden_dim):
             # the shared expert: a dense SwiGLU over all tokens on the same kernels (one segment)
             sh = block.shared_experts
@@ -468,6 +487,7 @@ def per_kernel_times(args, wl, block, x, gout, dev):
             sproj = 2.0 * T * D * Fs
             shared_flops = {"gate_up": 2 * sproj, "down": sproj, "dh": sproj, "drows": 2 * sproj, "dw2": sproj,
                             "dw1": sproj, "dw3": sproj}
+            shared_bytes = swiglu_stage_bytes(T, 1, D, Fs, s_bytes, dh_writes_scaled_h=False)
             if not wl.backward:
                 shared_flops = {k: shared_flops[k] for k in ("gate_up", "down")}
             shared_fns = {s: (lambda s=s: ops.grouped_swiglu_stage(s, sbuf, sp)) for s in shared_flops}
@@ -533,12 +553,22 @@ def per_kernel_times(args, wl, block, x, gout, dev):
         "rms_norm_bwd": 3 * T * D * s_bytes,
     }
     kernels = {}
+
+    def gemm_entry(ms, flops, nbytes):
+        # both sides of the roofline: the product's flops against the MFMA peak and its algorithmic
+        # bytes against the HBM peak; the one that bounds it is decided by flops per byte
+        tf = flops / (ms * 1e-3) / 1e12 if ms > 0 else 0.0
+        ent = {"ms": round(ms, 4), "TFLOP/s": round(tf, 1), "frac_mfma": round(tf / peak, 4)}
+        if nbytes and ms > 0:
+            gbs = nbytes / (ms * 1e-3) / 1e9
+            ent.update({"GB/s": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4),
+                        "flop_per_byte": round(flops / nbytes, 1)})
+        return ent
+
     for s, ms in stage_ms.items():
-        tf = stage_flops[s] / (ms * 1e-3) / 1e12 if ms > 0 else 0.0
-        kernels[f"grouped_{s}"] = {"ms": round(ms, 4), "TFLOP/s": round(tf, 1), "frac_mfma": round(tf / peak, 4)}
+        kernels[f"grouped_{s}"] = gemm_entry(ms, stage_flops[s], stage_bytes.get(s) if folded else None)
     for s, ms in shared_ms.items():
-        tf = shared_flops[s] / (ms * 1e-3) / 1e12
-        kernels[f"shared_{s}"] = {"ms": round(ms, 4), "TFLOP/s": round(tf, 1), "frac_mfma": round(tf / peak, 4)}
+        kernels[f"shared_{s}"] = gemm_entry(ms, shared_flops[s], shared_bytes.get(s))
     for s, ms in other_ms.items():
         ent = {"ms": round(ms, 4)}
         if s not in in_step:
@@ -548,7 +578,8 @@ def per_kernel_times(args, wl, block, x, gout, dev):
             gbs = other_bytes[s] / (ms * 1e-3) / 1e9
             ent.update({"GB/s": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4)})
         kernels[s] = ent
-    return kernels, stage_ms, stage_flops, shared_ms, shared_flops, R_rows, folded, stage_fns
+    return (kernels, stage_ms, stage_flops, shared_ms, shared_flops, R_rows, folded, stage_fns,
+            stage_bytes if folded else {}, shared_bytes)
 
 
 def main():
@@ -593,7 +624,8 @@ def main():
     graph_ms = None if args.no_graph else hip_graph_step(block, x, gout, wl, args.steps, args.warmup)
 
     x2, g2 = x.reshape(-1, wl.dim), gout.reshape(-1, wl.dim)
-    kernels, stage_ms, stage_flops, shared_ms, shared_flops, R_rows, folded, stage_fns = per_kernel_times(
+    (kernels, stage_ms, stage_flops, shared_ms, shared_flops, R_rows, folded, stage_fns, stage_bytes,
+     shared_bytes) = per_kernel_times(
         args, wl, block, x2, g2, dev)
     peak = PEAK_BF16_TFLOPS if wl.dtype == torch.bfloat16 else PEAK_FP32_TFLOPS
 
@@ -603,12 +635,12 @@ def main():
     groups = {}
     for s in stage_ms:
         key = "dw1+dw3" if s in ("dw1", "dw3") else s
-        g = groups.setdefault(f"grouped_{key}", {"ms": 0.0, "flops": 0.0, "launches": 0})
-        g["ms"] += stage_ms[s]; g["flops"] += stage_flops[s]; g["launches"] += 1
+        g = groups.setdefault(f"grouped_{key}", {"ms": 0.0, "flops": 0.0, "launches": 0, "bytes": 0.0})
+        g["ms"] += stage_ms[s]; g["flops"] += stage_flops[s]; g["launches"] += 1; g["bytes"] += stage_bytes.get(s, 0.0)
     for s in shared_ms:
         key = "dw1+dw3" if s in ("dw1", "dw3") else s
-        g = groups.setdefault(f"shared_{key}", {"ms": 0.0, "flops": 0.0, "launches": 0})
-        g["ms"] += shared_ms[s]; g["flops"] += shared_flops[s]; g["launches"] += 1
+        g = groups.setdefault(f"shared_{key}", {"ms": 0.0, "flops": 0.0, "launches": 0, "bytes": 0.0})
+        g["ms"] += shared_ms[s]; g["flops"] += shared_flops[s]; g["launches"] += 1; g["bytes"] += shared_bytes.get(s, 0.0)
     dominant = max(groups, key=lambda k: groups[k]["ms"])
     dg = groups[dominant]
     ach = dg["flops"] / (dg["ms"] * 1e-3) / 1e12
@@ -620,15 +652,27 @@ def main():
         parts = dominant[len("grouped_"):].split("+")
         if all(p in tb for p in parts):
             traffic = sum(tb[p] for p in parts) / len(parts)
+    # Which roof bounds the kernel: its flops per algorithmic byte against the ridge of the two
+    # published peaks (2500 TFLOP/s / 8 TB/s = 312 flop/B in bf16).  Left of the ridge the HBM roof
+    # is the lower one and the fraction is taken against it; both fractions are kept in the object.
+    ridge = peak * 1e12 / (PEAK_HBM_GBS * 1e9)
+    intensity = dg["flops"] / dg["bytes"] if dg["bytes"] else None
+    ach_gbs = dg["bytes"] / (dg["ms"] * 1e-3) / 1e9 if dg["bytes"] else None
+    hbm_bound = intensity is not None and intensity < ridge
     roofline = {
         "kernel": dominant,
         "launches_per_step": dg["launches"],
         "share_of_step": round(dg["ms"] / ms_per_step, 4),
-        "bound": "mfma",
-        "achieved": round(ach, 2),
-        "peak": peak,
-        "unit": "TFLOP/s",
-        "frac": round(ach / peak, 4),
+        "bound": "hbm" if hbm_bound else "mfma",
+        "achieved": round(ach_gbs, 1) if hbm_bound else round(ach, 2),
+        "peak": PEAK_HBM_GBS if hbm_bound else peak,
+        "unit": "GB/s" if hbm_bound else "TFLOP/s",
+        "frac": round(ach_gbs / PEAK_HBM_GBS, 4) if hbm_bound else round(ach / peak, 4),
+        "frac_mfma": round(ach / peak, 4),
+        "frac_hbm": None if ach_gbs is None else round(ach_gbs / PEAK_HBM_GBS, 4),
+        "flop_per_byte": None if intensity is None else round(intensity, 1),
+        "ridge_flop_per_byte": round(ridge, 1),
+        "algorithmic_bytes_per_launch": None if not dg["bytes"] else round(dg["bytes"] / dg["launches"]),
         "traffic": traffic,
         "avg_launch_ms": round(dg["ms"] / dg["launches"], 4),
         "all_grouped_gemms": {"TFLOP/s": round(gemm_flops / (gemm_ms * 1e-3) / 1e12, 1),
