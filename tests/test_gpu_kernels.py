@@ -567,7 +567,7 @@ def test_rows_not_covered_by_the_counts_come_back_as_zeros(ops):
 
 
 def test_plan_edge_cases_largest_expert_count_and_ids_out_of_range(ops):
-    """E = 2048, the largest expert count the plan accepts (its scan keeps 48 KiB in LDS there),
+    """E = 2048, the largest expert count the plan accepts (its scan keeps 56 KiB in LDS there),
     is still the stable argsort; one more expert is refused; a slot whose id lies outside [0, E)
     is not counted and gets no row."""
     g = torch.Generator().manual_seed(2)
