@@ -172,6 +172,36 @@ def test_router_select_exact_ties_go_to_lower_index(ops):
     assert ids.tolist() == [[0, 1]]
 
 
+@pytest.mark.parametrize("E,K,groups", [(64, 6, 0), (128, 8, 0), (256, 8, 0), (256, 8, 8), (128, 4, 4)])
+def test_both_select_kernels_make_the_same_choice(ops, E, K, groups):
+    """The 16-lanes-per-token kernel (16-byte aligned logits, E = 64 / 128 / 256) and the
+    wavefront-per-token kernel (any alignment) choose the same experts on every token: their
+    comparisons differ in order only, and (larger value, lower index) is a total order.  With
+    sigmoid scores nothing is summed before the choice, so weights and scores agree bit for bit
+    as well; with softmax the choice is made on the logits and the scores differ by rounding."""
+    print(f"select kernels agree E={E} K={K} groups={groups}", flush=True)
+    T = 1000
+    g = torch.Generator().manual_seed(E + K)
+    aligned = torch.randn(T, E, generator=g).to(DEV)
+    flat = torch.empty(T * E + 4, device=DEV)
+    flat[1:1 + T * E] = aligned.view(-1)
+    shifted = flat[1:1 + T * E].view(T, E)  # the same values 4 bytes into an allocation
+    assert aligned.data_ptr() % 16 == 0 and shifted.data_ptr() % 16 == 4
+    bias = (torch.rand(E, generator=g) * 0.2 - 0.1).to(DEV)
+    limited = max(1, groups // 2)
+    for fn, b in (("sigmoid", bias), ("sigmoid", None), ("softmax", None), ("sqrtsoftplus", bias)):
+        if fn == "softmax" and groups:
+            continue  # the scores, summed in a different order, enter the group choice there
+        ref = ops.router_select_fwd(shifted, b, K, fn, True, 2.0, groups, limited, 0, True, True)
+        out = ops.router_select_fwd(aligned, b, K, fn, True, 2.0, groups, limited, 0, True, True)
+        assert torch.equal(out[1], ref[1]), f"{fn}: the two kernels chose different experts"
+        assert torch.equal(out[3], ref[3])
+        if fn != "softmax":
+            assert torch.equal(out[0], ref[0]) and torch.equal(out[2], ref[2])
+        else:
+            assert rel_max(out[0], ref[0]) < 1e-6 and rel_max(out[2], ref[2]) < 1e-6
+
+
 # ---------------------------------------------------------------- permutation plan
 @pytest.mark.parametrize("T,K,E,align,local", [
     (3, 2, 3, 1, None), (6, 2, 4, 4, None), (700, 8, 128, 1, None), (700, 8, 128, 128, None),
