@@ -59,7 +59,7 @@ __global__ __launch_bounds__(256) void combine_fwd_kernel(
   // ascending-row visiting order (index_add's order): position of each valid slot
   int pos = 0;
   for (int j = 0; j < K; ++j) {
-    const int rj = __shfl(row, j, kWave);
+    const int rj = __builtin_amdgcn_readlane(row, j);  // j is wave-uniform: a lane read, not an LDS permute
     pos += (rj >= 0 && (rj < row || (rj == row && j < lane))) ? 1 : 0;
   }
   const int nvalid = __popcll(__ballot(row >= 0));
@@ -83,9 +83,9 @@ __global__ __launch_bounds__(256) void combine_fwd_kernel(
     auto request = [&](int base, int p0, uint4 (&v)[B][G], float (&ww)[B]) {
 #pragma unroll
       for (int j = 0; j < B; ++j) {
-        const int p = min(p0 + j, nvalid - 1);  // past the end: not loaded, not used
-        const int r = __builtin_amdgcn_readfirstlane(__shfl(o_row, p, kWave));
-        ww[j] = __shfl(o_w, p, kWave);
+        const int p = max(min(p0 + j, nvalid - 1), 0);  // past the end: not loaded, not used
+        const int r = __builtin_amdgcn_readlane(o_row, p);  // p is wave-uniform
+        ww[j] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(o_w), p));
         const uint4* src = reinterpret_cast<const uint4*>(y + static_cast<int64_t>(max(r, 0)) * D);
 #pragma unroll
         for (int g = 0; g < G; ++g) {
