@@ -34,12 +34,32 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_FP32_TFLOPS = 157.3   # MI355X dense fp32 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 
-# HBM bytes per launch, measured with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (scaled by a
-# 256 MiB copy: x2.0 and x1.0); the tables these come from are profiles/*_hbm_traffic.txt.
-MEASURED_HBM_BYTES = {
-    "c3": {"gate_up": 1511.8e6, "down": 844.8e6, "dh": 1255.4e6, "drows": 1434.6e6,
-           "dw2": 828.0e6, "dw1": 895.9e6, "dw3": 895.9e6},
-}
+PROFILE_TRAFFIC = {"c3": "moe_layer_qwen3_t8192_hbm_traffic.txt",
+                   "c4": "moe_layer_qwen3_t16384_skewed_padded_hbm_traffic.txt",
+                   "c5": "moe_layer_deepseek_v3_local_share_t4096_hbm_traffic.txt"}
+
+
+def measured_traffic(workload):
+    """HBM bytes per launch of the grouped stages as rocprofv3 counted them (FETCH_SIZE and
+    WRITE_SIZE, scaled by a copy of known size), read from the summary under profiles/: its
+    lines ``traffic <stage> <bytes>`` and ``measured at commit <sha>``.  Nothing is assumed when
+    the file or a stage is missing: the figure belongs to the commit the file names, not to
+    the run that prints it."""
+    name = PROFILE_TRAFFIC.get(workload)
+    path = os.path.join(ROOT, "profiles", name) if name else None
+    if not path or not os.path.exists(path):
+        return {}, None
+    table, commit = {}, None
+    for line in open(path):
+        f = line.split()
+        if len(f) == 3 and f[0] == "traffic":
+            try:
+                table[f[1]] = float(f[2])
+            except ValueError:
+                pass
+        elif line.startswith("measured at commit") and len(f) >= 4:
+            commit = f[3]
+    return table, commit
 
 
 def parse():
@@ -57,10 +77,12 @@ def parse():
                     help="also loop each grouped GEMM, the whole step, the vendor GEMM, the MFMA probe and a copy for "
                          "--power-seconds each while sampling the card's power sensor (hwmon); adds a \"power\" object")
     ap.add_argument("--power-seconds", type=float, default=2.5)
-    ap.add_argument("--kloop", action="store_true",
-                    help="also run the stand-alone K-loop study of bench_probe/kloop.hip (needs 4.4 GB of device memory); "
-                         "with --power each case is also looped under the power sensor")
     ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay of the same step")
+    ap.add_argument("--single-workload", dest="all_workloads", action="store_false",
+                    help="measure --workload only (default: the other four configurations follow it, a short run "
+                         "each, and are summarised under \"workloads\")")
+    ap.add_argument("--other-steps", type=int, default=20)
+    ap.add_argument("--other-warmup", type=int, default=10)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (known traffic, for scaling rocprof FETCH_SIZE / WRITE_SIZE)")
     return ap.parse_args()
@@ -151,66 +173,6 @@ def sustained_mfma(dev):
             c = clocks.view(blocks, 2).double()
             out[name][label] = {"TFLOP/s": round(flops / (ms * 1e-3) / 1e12, 1),
                                 "core_clock_mhz": round(float((c[:, 0] / c[:, 1]).mean()) * 100.0, 0)}
-    return out
-
-
-KLOOP_VARIANTS = ("product_loop", "without_skip_branches", "direct_to_lds", "four_waves_128x128",
-                  "staging_without_fragment_reads", "fragment_reads_without_staging", "mfma_only")
-KLOOP_PLACEMENTS = ("windows_per_workgroup", "b_operand_from_hbm", "one_shared_window")
-
-
-def kloop_study(dev, watts=None):
-    """Stand-alone K loops of the grouped GEMMs' shape (bench_probe/kloop.hip: 256 x 256 x 64 tile
-    steps, normally distributed bf16 operands, no epilogue, every tile full): four schedules and
-    three ablations of the second (no fragment reads / no staging / neither), each with a 2 MiB
-    operand window per workgroup (34 MB in all: the memory-side cache), with the B half of every
-    step streamed from HBM (32 KB per step and workgroup; schedules only) and with one window
-    shared by all workgroups (resident in every L2): TFLOP/s, and watts when ``watts`` (a
-    function: callable -> average watts while it loops) is given.  None when the probe library
-    is not built."""
-    import ctypes
-
-    import torch
-
-    path = os.path.join(ROOT, "bench_probe", "libmi355probe.so")
-    if not os.path.exists(path):
-        return None
-    lib = ctypes.CDLL(path)
-    if not hasattr(lib, "mi355_probe_kloop"):
-        return None
-    vp = ctypes.c_void_p
-    lib.mi355_probe_kloop.argtypes = [ctypes.c_int, ctypes.c_int, vp, vp, vp, ctypes.c_int, ctypes.c_int, vp]
-    lib.mi355_probe_kloop.restype = ctypes.c_int
-    for f in (lib.mi355_probe_kloop_hot_elems, lib.mi355_probe_kloop_cold_elems):
-        f.argtypes, f.restype = [ctypes.c_int], ctypes.c_long
-    blocks = torch.cuda.get_device_properties(dev).multi_processor_count
-    gen = torch.Generator(device=dev).manual_seed(0)
-    hot = torch.randn(lib.mi355_probe_kloop_hot_elems(blocks), device=dev, generator=gen).bfloat16()
-    cold = torch.empty(lib.mi355_probe_kloop_cold_elems(blocks), dtype=torch.bfloat16, device=dev)
-    piece = 1 << 27
-    for i in range(0, cold.numel(), piece):  # in pieces: the fp32 draw of the whole buffer would be 8.6 GB
-        cold[i:i + piece] = torch.randn(min(piece, cold.numel() - i), device=dev, generator=gen).bfloat16()
-    sink = torch.zeros(1, dtype=torch.float32, device=dev)
-    ksteps = 2048
-    flops = blocks * ksteps * 2.0 * 256 * 256 * 64
-
-    def launch(v, placement, n=ksteps):
-        rc = lib.mi355_probe_kloop(v, placement, hot.data_ptr(), cold.data_ptr(), sink.data_ptr(), blocks, n,
-                                   torch.cuda.current_stream().cuda_stream)
-        assert rc == 0, rc
-
-    out = {"ksteps": ksteps, "workgroups": blocks, "stream_bytes_per_step_and_workgroup": 32768}
-    for v, name in enumerate(KLOOP_VARIANTS):
-        ent = {}
-        for placement, key in enumerate(KLOOP_PLACEMENTS):
-            if placement == 1 and v > 3:
-                continue
-            launch(v, placement, 64)
-            best = min(time_events(lambda: launch(v, placement), 1, warmup=0) for _ in range(3))
-            ent[key] = {"TFLOP/s": round(flops / (best * 1e-3) / 1e12, 1), "us_per_k_step": round(best * 1e3 / ksteps, 3)}
-            if watts is not None:
-                ent[key]["watts"] = watts(lambda: launch(v, placement, 512))
-        out[name] = ent
     return out
 
 
@@ -312,9 +274,13 @@ def hip_graph_step(block, x, gout, wl, steps, warmup):
 
 
 def cpu_baseline(wl, sample_tokens):
-    """The oracle's pass (forward, + backward where the workload has one) on host cores:
-    a warm-up, then the median of three runs, over ``sample_tokens`` tokens of the workload's
-    layer (the full C1 block when it is that small); bf16 workloads are timed in fp32 as well."""
+    """The oracle's pass (forward, + backward where the workload has one) on host cores at the
+    workload's FULL token count: a short warm-up, then one timed run, reported as tokens/s.
+    A second, small sample (``sample_tokens`` tokens) is timed beside it as ``fixed_cost_s``: the
+    oracle's time hardly depends on the token count at the large shapes (its per-expert loop, like
+    the reference's, indexes the stacked weights, so autograd materialises a full (E, F, D)
+    gradient per expert and projection), which is why a rate taken over a sample would be an
+    artefact of the sample's size."""
     import torch
 
     from oracle import moe_ref as R
@@ -324,7 +290,7 @@ def cpu_baseline(wl, sample_tokens):
     cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
     torch.set_num_threads(cores)
 
-    def measure(wl, tokens, dtype):
+    def runner(wl, dtype):
         w = W.make_weights(wl)
         cast = lambda t: t.to(dtype)
         p = R.MoEParams(router_w_ED=w["router"].clone(), w1_EFD=cast(w["w1"]), w3_EFD=cast(w["w3"]),
@@ -359,31 +325,40 @@ def cpu_baseline(wl, sample_tokens):
                     out.backward(g)
             return time.perf_counter() - t0
 
-        run(min(128, tokens))  # warm-up: thread pool, allocator
-        times = [run(tokens) for _ in range(3)]
-        return tokens / statistics.median(times), times
+        return run
 
-    tokens = min(sample_tokens, wl.tokens)
-    rate, times = measure(wl, tokens, wl.dtype)
     name = {torch.float32: "fp32", torch.bfloat16: "bf16"}[wl.dtype]
+    run = runner(wl, wl.dtype)
+    small = min(sample_tokens, wl.tokens)
+    run(min(128, wl.tokens))  # warm-up: thread pool, allocator
+    if wl.tokens <= 1024:
+        times = [run(wl.tokens) for _ in range(3)]
+        full_s, how = statistics.median(times), f"median of 3 runs ({', '.join(f'{t:.3f}' for t in times)} s)"
+    else:
+        full_s = run(wl.tokens)
+        how = f"one run ({full_s:.2f} s)"
     out = {
-        "value": round(rate, 2),
+        "value": round(wl.tokens / full_s, 2),
         "unit": "tokens/s",
         "cores": cores,
         "kind": "port",
-        "sample": f"oracle {'fwd+bwd' if wl.backward else 'fwd'}, {tokens} tokens of the {wl.key} layer "
-                  f"(D={wl.dim},E={wl.num_experts},K={wl.top_k},F={wl.hidden_dim}), {name}, 128-token warm-up then "
-                  f"the median of 3 runs ({', '.join(f'{t:.2f}' for t in times)} s)",
+        "seconds": round(full_s, 3),
+        "sample": f"oracle {'fwd+bwd' if wl.backward else 'fwd'} of the whole {wl.key} layer at its full size, "
+                  f"T={wl.tokens} (D={wl.dim},E={wl.num_experts},K={wl.top_k},F={wl.hidden_dim}), {name}, after a "
+                  f"128-token warm-up: {how}",
     }
-    if wl.dtype == torch.bfloat16:
-        rate32, times32 = measure(wl, tokens, torch.float32)
-        out["fp32"] = {"value": round(rate32, 2), "unit": "tokens/s",
-                       "sample": f"the same sample with fp32 weights and activations "
-                                 f"({', '.join(f'{t:.2f}' for t in times32)} s)"}
+    if small < wl.tokens:
+        fixed = run(small)
+        out["fixed_cost_s"] = round(fixed, 3)
+        out["fixed_cost_note"] = (f"the same pass over {small} tokens takes {fixed:.2f} s: most of the oracle's time "
+                                  f"at this shape does not scale with the token count, so only the full-size run "
+                                  f"above is a rate")
     if wl.key != "c1":
         c1 = W.WORKLOADS["c1"]
-        rate1, times1 = measure(c1, c1.tokens, c1.dtype)
-        out["c1_full_size"] = {"value": round(rate1, 1), "unit": "tokens/s",
+        run1 = runner(c1, c1.dtype)
+        run1(c1.tokens)
+        times1 = [run1(c1.tokens) for _ in range(3)]
+        out["c1_full_size"] = {"value": round(c1.tokens / statistics.median(times1), 1), "unit": "tokens/s",
                                "sample": f"oracle fwd+bwd of the whole C1 block (T={c1.tokens}, fp32), median of 3"}
     return out
 
@@ -582,16 +557,14 @@ def per_kernel_times(args, wl, block, x, gout, dev):
             stage_bytes if folded else {}, shared_bytes)
 
 
-def main():
-    args = parse()
-    if args.gpus != 1:
-        print("bench.py measures one GPU; this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
-        sys.exit(2)
+def measure_workload(args, wl, steps, warmup, *, detail):
+    """Build the block of ``wl``, time ``steps`` whole steps after ``warmup`` and each kernel of a
+    step.  ``detail``: also the HIP-graph replay, the MFMA probe and the vendor GEMM (the
+    headline workload); without it only what the summary of the other workloads needs."""
     import torch
 
     from torchllmtuner_amd import workloads as W
 
-    wl = W.WORKLOADS[args.workload]
     dev = "cuda:0"
     x_cpu, gout_cpu = W.make_inputs(wl)
     block = W.build_block(wl, dev, x_for_skew=x_cpu)
@@ -610,18 +583,18 @@ def main():
             with torch.no_grad():
                 block(x)
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         step()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
-    ms_per_step = dt / args.steps * 1e3
-    tokens_per_s = T * args.steps / dt
+    ms_per_step = dt / steps * 1e3
+    tokens_per_s = T * steps / dt
 
-    graph_ms = None if args.no_graph else hip_graph_step(block, x, gout, wl, args.steps, args.warmup)
+    graph_ms = None if (args.no_graph or not detail) else hip_graph_step(block, x, gout, wl, steps, warmup)
 
     x2, g2 = x.reshape(-1, wl.dim), gout.reshape(-1, wl.dim)
     (kernels, stage_ms, stage_flops, shared_ms, shared_flops, R_rows, folded, stage_fns, stage_bytes,
@@ -646,41 +619,43 @@ def main():
     ach = dg["flops"] / (dg["ms"] * 1e-3) / 1e12
     gemm_flops = sum(stage_flops.values()) + sum(shared_flops.values())
     gemm_ms = sum(stage_ms.values()) + sum(shared_ms.values())
-    traffic = None
-    if args.workload in MEASURED_HBM_BYTES and dominant.startswith("grouped_"):
-        tb = MEASURED_HBM_BYTES[args.workload]
+    traffic = traffic_commit = None
+    tb, traffic_commit = measured_traffic(wl.key)
+    if dominant.startswith("grouped_"):
         parts = dominant[len("grouped_"):].split("+")
-        if all(p in tb for p in parts):
+        if parts and all(p in tb for p in parts):
             traffic = sum(tb[p] for p in parts) / len(parts)
-    # Which roof bounds the kernel: its flops per algorithmic byte against the ridge of the two
-    # published peaks (2500 TFLOP/s / 8 TB/s = 312 flop/B in bf16).  Left of the ridge the HBM roof
-    # is the lower one and the fraction is taken against it; both fractions are kept in the object.
+    # The grouped and shared-expert products are matrix-core work: the fraction is their flops
+    # (2*R*D*F per projection over real rows, padding excluded) per second against the dense
+    # bf16 MFMA peak.  Their algorithmic bytes against the HBM peak, the flops per byte and the
+    # ridge of the two published peaks (2500 TFLOP/s / 8 TB/s = 312 flop/B in bf16) are kept
+    # beside it: at these shapes the products sit close to the ridge.
     ridge = peak * 1e12 / (PEAK_HBM_GBS * 1e9)
     intensity = dg["flops"] / dg["bytes"] if dg["bytes"] else None
     ach_gbs = dg["bytes"] / (dg["ms"] * 1e-3) / 1e9 if dg["bytes"] else None
-    hbm_bound = intensity is not None and intensity < ridge
     roofline = {
         "kernel": dominant,
         "launches_per_step": dg["launches"],
         "share_of_step": round(dg["ms"] / ms_per_step, 4),
-        "bound": "hbm" if hbm_bound else "mfma",
-        "achieved": round(ach_gbs, 1) if hbm_bound else round(ach, 2),
-        "peak": PEAK_HBM_GBS if hbm_bound else peak,
-        "unit": "GB/s" if hbm_bound else "TFLOP/s",
-        "frac": round(ach_gbs / PEAK_HBM_GBS, 4) if hbm_bound else round(ach / peak, 4),
+        "bound": "mfma",
+        "achieved": round(ach, 2),
+        "peak": peak,
+        "unit": "TFLOP/s",
+        "frac": round(ach / peak, 4),
         "frac_mfma": round(ach / peak, 4),
         "frac_hbm": None if ach_gbs is None else round(ach_gbs / PEAK_HBM_GBS, 4),
         "flop_per_byte": None if intensity is None else round(intensity, 1),
         "ridge_flop_per_byte": round(ridge, 1),
         "algorithmic_bytes_per_launch": None if not dg["bytes"] else round(dg["bytes"] / dg["launches"]),
         "traffic": traffic,
+        "traffic_measured_at_commit": traffic_commit if traffic is not None else None,
         "avg_launch_ms": round(dg["ms"] / dg["launches"], 4),
         "all_grouped_gemms": {"TFLOP/s": round(gemm_flops / (gemm_ms * 1e-3) / 1e12, 1),
                               "frac": round(gemm_flops / (gemm_ms * 1e-3) / 1e12 / peak, 4),
                               "ms": round(gemm_ms, 4)},
     }
 
-    probe = None if (args.no_probe or wl.dtype != torch.bfloat16) else sustained_mfma(dev)
+    probe = None if (args.no_probe or not detail or wl.dtype != torch.bfloat16) else sustained_mfma(dev)
     if probe is not None:
         # the same instruction with operands in registers: the rate the card holds under
         # its own power management, next to the data-sheet peak above
@@ -708,15 +683,15 @@ def main():
         config["load_histogram_sorted"] = {"max": int(load[0]), "median": int(load[wl.num_experts // 2]),
                                            "min": int(load[-1]),
                                            "top20_share": round(float(load[: wl.num_experts // 5].sum()) / ids.numel(), 4)}
-    metric = ("MoE layer fwd+bwd tokens/s (Qwen3-30B-A3B shape, 1 GPU)" if args.workload == "c3"
+    metric = ("MoE layer fwd+bwd tokens/s (Qwen3-30B-A3B shape, 1 GPU)" if wl.key == "c3"
               else f"MoE layer {'fwd+bwd' if wl.backward else 'fwd'} tokens/s ({wl.key}, 1 GPU)")
     result = {
         "metric": metric,
         "value": round(tokens_per_s, 1),
         "unit": "tokens/s",
         "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
+        "steps": steps,
+        "warmup": warmup,
         "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True,
         "scaling": "weak",
@@ -732,7 +707,7 @@ def main():
         result["hip_graph"] = {"ms_per_step": round(graph_ms, 4), "tokens_per_s": round(T / (graph_ms * 1e-3), 1)}
     elif graph_ms is not None:
         result["hip_graph"] = {"error": graph_ms[:300]}
-    if args.power:
+    if args.power and detail:
         cases = {"idle": None}
         cases.update({f"grouped_{s}": fn for s, fn in stage_fns.items()})
         cases["whole_step"] = step
@@ -762,15 +737,44 @@ def main():
                     ent["TFLOP/s_looped"] = round(pl[1] * 8.0 * 2000 * 262144 * 2 / (ent["ms_per_call_looped"] * 1e-3) / 1e12, 1)
             ent = result["power"]["cases"]["copy_1GiB"]
             ent["GB/s_looped"] = round(2.0 * (1 << 30) / (ent["ms_per_call_looped"] * 1e-3) / 1e9, 1)
-    if args.kloop:
-        watts = None
-        if args.power:
-            def watts(fn):
-                t = power_table({"case": fn}, args.power_seconds)
-                return None if t is None else t["cases"]["case"]["watts"]
-        result["kloop_study"] = kloop_study(dev, watts)
+    return result
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU; this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
+        sys.exit(2)
+    import gc
+
+    import torch
+
+    from torchllmtuner_amd import workloads as W
+
+    wl = W.WORKLOADS[args.workload]
+    result = measure_workload(args, wl, args.steps, args.warmup, detail=True)
+    if args.all_workloads:
+        # the other four configurations, a short run each (no CPU leg, no probe, no graph): whole-step
+        # rate and the grouped products together against the MFMA peak; the top-level keys stay
+        # those of the workload chosen above
+        summary = {}
+        for key in ("c1", "c2", "c3", "c4", "c5"):
+            if key == wl.key:
+                r = result
+            else:
+                gc.collect()
+                torch.cuda.empty_cache()
+                r = measure_workload(args, W.WORKLOADS[key], args.other_steps, args.other_warmup, detail=False)
+            summary[key] = {"workload": r["config"]["workload"], "steps": r["steps"], "ms_per_step": r["ms_per_step"],
+                            "tokens_per_s": r["value"],
+                            "all_grouped_gemms_frac": r["roofline"]["all_grouped_gemms"]["frac"],
+                            "all_grouped_gemms_TFLOP/s": r["roofline"]["all_grouped_gemms"]["TFLOP/s"],
+                            "dtype": r["dtype"]}
+        result["workloads"] = summary
+        gc.collect()
+        torch.cuda.empty_cache()
     if args.calibrate_copy:
-        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0")
         dst = torch.empty_like(src)
         dst.copy_(src)
         torch.cuda.synchronize()

@@ -245,7 +245,9 @@ int mi355_permute_plan(const int64_t* ids_TK, int64_t T, int64_t K, int64_t E,
  * exceeds that (e.g. N = T*K = 2^20 slots with E <= 128 fits; N = 131072, E = 256 fits).
  * Calls no hipMalloc / hipFree and no allocating library routine.  All calls on one GPU share
  * that GPU's array: calls that overlap on one GPU (two streams or threads) race -- serialise
- * them, or use mi355_permute_plan with separate workspaces.
+ * them, or use mi355_permute_plan with separate workspaces.  The first call on a device looks
+ * the array's address up and must not run under stream capture (it returns MI355_EINVAL
+ * there): call once, uncaptured, beforehand -- T = 0 will do.
  */
 int64_t mi355_permute_plan_static_max_bytes(void);
 int mi355_permute_plan_static(const int64_t* ids_TK, int64_t T, int64_t K, int64_t E,

@@ -443,29 +443,17 @@ def test_full_size_properties_qwen3_t8192():
             ref[i] += float(scores[t, k]) * bf(w2[e].float() @ h)
     assert rel_l2(out[sample].float(), ref) < 2e-2
 
-    # --- sampled experts: weight gradients from plain matmuls over the same intermediates
+    # --- sampled experts: weight gradients recomputed from x, ids, scores and gout alone
+    _expert_weight_gradient_check(x, gout, ids, scores, w1, w3, w2, dw1, dw3, dw2, (0, 57, 127))
+    # --- routing-score gradient: the device's against <y, dout> recomputed from the inputs, then
+    # dW_router from fp32 autograd over the router path with the device's score gradient upstream
     with torch.no_grad():
         rows = ops.permute_rows_fwd(x, plan)
-        y, gate, up, h = ops.grouped_swiglu_fwd(rows, w1, w3, w2, plan)
-        dy, dsc = ops.combine_bwd(gout, y, scores, plan)
-    off = plan.seg_offsets.cpu().tolist()
-    for e in (0, 57, 127):
-        sl = slice(off[e], off[e + 1])
-        gf, uf, dyf = gate[sl].float(), up[sl].float(), dy[sl].float()
-        want_dw2 = dyf.T @ h[sl].float()
-        dh = bf(dyf @ w2[e].float())
-        sig = torch.sigmoid(gf)
-        dup = bf(dh * bf(gf * sig))
-        dgate = bf(bf(dh * uf) * (sig * (1 + gf * (1 - sig))))
-        assert rel_l2(dw2[e].float(), want_dw2) < 2e-2
-        assert rel_l2(dw1[e].float(), dgate.T @ rows[sl].float()) < 2e-2
-        assert rel_l2(dw3[e].float(), dup.T @ rows[sl].float()) < 2e-2
-    # router score gradient of the sampled tokens: <y[row], dout[t]>
-    for t in sample[:8]:
-        for k in range(K):
-            r = int(plan.row_of_slot[t * K + k])
-            want = float((y[r].float() * gout[t].float()).sum())
-            assert abs(float(dsc[t, k]) - want) <= 2e-2 * max(1.0, abs(want))
+        y, _, _, _ = ops.grouped_swiglu_fwd(rows, w1, w3, w2, plan)
+        _, dsc = ops.combine_bwd(gout, y, scores, plan)
+    want = _score_gradient_reference(x, gout, ids, w1, w3, w2, sample[:8])
+    assert bool(((dsc[sample[:8]] - want).abs() <= 2e-2 * want.abs().clamp_min(1.0)).all())
+    _router_weight_gradient_check(block, x, ids, dsc, dwr, spec, (0, 3, 17, 40, 57, 88, 101, 127))
 
 
 def _sampled_token_reference(x, ids, weights, w1, w3, w2, sample, lo=0, hi=None):
@@ -486,33 +474,73 @@ def _sampled_token_reference(x, ids, weights, w1, w3, w2, sample, lo=0, hi=None)
     return ref
 
 
-def _expert_weight_gradient_check(ops, x, gout, scores, plan, w1, w3, w2, dw1, dw3, dw2, experts, lo=0):
-    """Weight gradients of the sampled local experts from plain fp32 matmuls over the same
-    intermediates (materialised rows, the forward's gate / up / h, the combine's backward), with
-    the bf16 rounding points of the SwiGLU backward.  An expert without rows must get zeros."""
+def _expert_weight_gradient_check(x, gout, ids, scores, w1, w3, w2, dw1, dw3, dw2, experts, lo=0):
+    """Weight gradients of the sampled local experts recomputed from the block's INPUTS alone --
+    tokens, output gradient, the device's ids and routing scores, the weights -- with plain fp32
+    torch ops on the device and the bf16 rounding points of the reference's op sequence; no
+    intermediate of the kernels under test (rows, gate, up, h, dy) is read.  The rows of expert e
+    are its slots in ascending order (the stable expert-major order), row r stands for token
+    slot // K, and dy[r] = score[slot] * gout[token] (the combine's backward).  An expert without
+    rows must get zeros."""
     bf = lambda v: v.bfloat16().float()
-    with torch.no_grad():
-        rows = ops.permute_rows_fwd(x, plan)
-        y, gate, up, h = ops.grouped_swiglu_fwd(rows, w1, w3, w2, plan)
-        dy, dsc = ops.combine_bwd(gout, y, scores, plan)
-    off = plan.seg_offsets.cpu().tolist()
-    cnt = plan.seg_counts.cpu().tolist()
+    K = ids.shape[1]
+    flat_ids, flat_scores = ids.reshape(-1), scores.reshape(-1).float()
     for e in experts:
-        sl = slice(off[e], off[e] + cnt[e])
-        if cnt[e] == 0:
+        slots = (flat_ids == e + lo).nonzero().squeeze(-1)
+        if slots.numel() == 0:
             for dw in (dw1, dw3, dw2):
                 assert not dw[e].any(), f"expert {e + lo} has no rows but a gradient"
             continue
-        gf, uf, dyf = gate[sl].float(), up[sl].float(), dy[sl].float()
-        dh = bf(dyf @ w2[e].float())
+        tok = slots // K
+        rows = x[tok].float()
+        gf, uf = bf(rows @ w1[e].float().T), bf(rows @ w3[e].float().T)
         sig = torch.sigmoid(gf)
-        dup = bf(dh * bf(gf * sig))
+        silu = bf(gf * sig)
+        h = bf(silu * uf)
+        dyf = bf(flat_scores[slots][:, None] * gout[tok].float())
+        dh = bf(dyf @ w2[e].float())
+        dup = bf(dh * silu)
         dgate = bf(bf(dh * uf) * (sig * (1 + gf * (1 - sig))))
-        for name, got, want in (("dw2", dw2[e], dyf.T @ h[sl].float()), ("dw1", dw1[e], dgate.T @ rows[sl].float()),
-                                ("dw3", dw3[e], dup.T @ rows[sl].float())):
+        for name, got, want in (("dw2", dw2[e], dyf.T @ h), ("dw1", dw1[e], dgate.T @ rows), ("dw3", dw3[e], dup.T @ rows)):
             err = rel_l2(got.float(), want)
-            assert err < 2e-2, f"{name}[{e + lo}] ({cnt[e]} rows): rel-L2 {err}"
-    return y, dsc
+            assert err < 2e-2, f"{name}[{e + lo}] ({slots.numel()} rows): rel-L2 {err}"
+
+
+def _score_gradient_reference(x, gout, ids, w1, w3, w2, tokens, lo=0, hi=None):
+    """d out / d score[t, k] = <y(t, k), gout[t]> for the given tokens, y recomputed from the token
+    and the weights in fp32 with the expert MLP's bf16 rounding points (zero for experts outside
+    [lo, hi): their rows are not computed here)."""
+    bf = lambda v: v.bfloat16().float()
+    hi = w1.shape[0] + lo if hi is None else hi
+    want = torch.zeros(len(tokens), ids.shape[1], device=x.device)
+    for i, t in enumerate(tokens):
+        xt = x[t].float()
+        for k in range(ids.shape[1]):
+            e = int(ids[t, k])
+            if not lo <= e < hi:
+                continue
+            gate, up = bf(w1[e - lo].float() @ xt), bf(w3[e - lo].float() @ xt)
+            h = bf(bf(torch.nn.functional.silu(gate)) * up)
+            want[i, k] = (bf(w2[e - lo].float() @ h) * gout[t].float()).sum()
+    return want
+
+
+def _router_weight_gradient_check(block, x, ids, dscore, dwr, spec, experts):
+    """dW_router from fp32 autograd over the router path alone -- gate (+ logit bias), score
+    function, gather at the device's ids, norm, scale -- with the device's routing-score gradient
+    as the upstream gradient; the rows of the sampled experts and the whole matrix."""
+    wr = block.router.gate.weight.detach().float().clone().requires_grad_()
+    lb = None if block.router.gate.bias is None else block.router.gate.bias.detach().float()
+    logits = x.float() @ wr.T + (0 if lb is None else lb)
+    s = torch.softmax(logits, -1) if spec.score_func == "softmax" else torch.sigmoid(logits)
+    w = s.gather(-1, ids)
+    if spec.route_norm:
+        w = w / (w.sum(-1, keepdim=True) + 1e-20)
+    (w * spec.route_scale * dscore.float()).sum().backward()
+    for e in experts:
+        err = rel_l2(dwr[e].float(), wr.grad[e])
+        assert err < 2e-2, f"dW_router[{e}]: rel-L2 {err}"
+    assert rel_l2(dwr.float(), wr.grad) < 2e-2
 
 
 def _token_gradient_reference(block, x, gout, ids, sample, spec, lo=0, hi=None):
@@ -616,13 +644,14 @@ def test_full_size_properties_skewed_padded_t16384():
     assert rel_l2(out[sample].float(), ref_out) < 2e-2
     assert rel_l2(dx[sample].float(), ref_dx) < 2e-2
     hottest, coldest = int(counts.argmax()), int(counts[: E - 1].argmin())
-    y, dsc = _expert_weight_gradient_check(ops, x, gout, scores, plan, w1, w3, w2, dw1, dw3, dw2,
-                                           (hottest, 40, coldest, E - 1))
-    for t in sample[:6]:  # routing-score gradient: <y[row], dout[t]>
-        for k in range(K):
-            r = int(plan.row_of_slot[t * K + k])
-            want = float((y[r].float() * gout[t].float()).sum())
-            assert abs(float(dsc[t, k]) - want) <= 2e-2 * max(1.0, abs(want))
+    _expert_weight_gradient_check(x, gout, ids, scores, w1, w3, w2, dw1, dw3, dw2, (hottest, 40, coldest, E - 1))
+    with torch.no_grad():
+        rows = ops.permute_rows_fwd(x, plan)
+        y, _, _, _ = ops.grouped_swiglu_fwd(rows, w1, w3, w2, plan)
+        _, dsc = ops.combine_bwd(gout, y, scores, plan)
+    want = _score_gradient_reference(x, gout, ids, w1, w3, w2, sample[:6])
+    assert bool(((dsc[sample[:6]] - want).abs() <= 2e-2 * want.abs().clamp_min(1.0)).all())
+    _router_weight_gradient_check(block, x, ids, dsc, dwr, spec, (hottest, 1, 9, 40, 77, 100, coldest, 120))
 
 
 def test_full_size_properties_deepseek_local_share():
@@ -671,8 +700,16 @@ def test_full_size_properties_deepseek_local_share():
     assert rel_l2(out[sample].float(), ref_out) < 2e-2
     assert rel_l2(dx[sample].float(), ref_dx) < 2e-2
     lc = plan.seg_counts.cpu()
-    _expert_weight_gradient_check(ops, x, gout, scores, plan, w1, w3, w2, ie.w1_EFD.grad, ie.w3_EFD.grad,
+    _expert_weight_gradient_check(x, gout, ids, scores, w1, w3, w2, ie.w1_EFD.grad, ie.w3_EFD.grad,
                                   ie.w2_EDF.grad, (int(lc.argmax()), 7, int(lc.argmin())))
+    with torch.no_grad():
+        rows = ops.permute_rows_fwd(x, plan)
+        y, _, _, _ = ops.grouped_swiglu_fwd(rows, w1, w3, w2, plan)
+        _, dsc = ops.combine_bwd(gout, y, scores, plan)
+    want = _score_gradient_reference(x, gout, ids, w1, w3, w2, sample[:6], lo=0, hi=32)
+    assert bool(((dsc[sample[:6]] - want).abs() <= 2e-2 * want.abs().clamp_min(1.0)).all())
+    _router_weight_gradient_check(block, x, ids, dsc, block.router.gate.weight.grad, spec,
+                                  (0, 5, 31, 32, 100, 177, 200, 255))
     # the shared expert: a dense SwiGLU over all tokens, gradients from plain fp32 matmuls
     sh = block.shared_experts
     bf = lambda v: v.bfloat16().float()

@@ -50,6 +50,24 @@ def test_select_cutoff_is_the_k_plus_first_biased_score(ops, T, E, K):
     assert rel_max(w, picked / (picked.sum(-1, keepdim=True) + 1e-20) * 2.5) < 1e-6
 
 
+@pytest.mark.parametrize("T,E,K", [(300, 8, 2), (1000, 128, 8), (257, 256, 8), (64, 96, 60)])
+@pytest.mark.parametrize("score_func", ["sigmoid", "softmax"])
+def test_select_cutoff_without_a_bias_is_the_k_plus_first_score(ops, T, E, K, score_func):
+    """No expert bias: the cutoff is still a SCORE (the (K+1)-th largest), never a logit, in both
+    select kernels (E = 128 / 256 take the 16-lanes-per-token kernel, the others one wave per token)."""
+    print(f"select cutoff without bias T={T} E={E} K={K} {score_func}", flush=True)
+    logits, _, _ = _case(T, E, K, seed=3 * T + E)
+    w, ids, scores, cutoff = ops.router_select_cutoff_fwd(logits.to(DEV), None, K, score_func, True, 1.0)
+    scores, cutoff, ids = scores.cpu(), cutoff.cpu(), ids.cpu()
+    ref = torch.sigmoid(logits) if score_func == "sigmoid" else torch.softmax(logits, dim=-1)
+    assert rel_max(scores, ref) < 1e-5
+    order = torch.argsort(scores, dim=-1, descending=True, stable=True)
+    assert torch.equal(cutoff, scores.gather(-1, order[:, K:K + 1]).squeeze(-1))
+    assert torch.equal(ids, order[:, :K])
+    ref_ids, ref_cut = R.select_top_k_plus_one(scores, torch.zeros(E), K)
+    assert torch.equal(ids, ref_ids) and torch.equal(cutoff, ref_cut.squeeze(-1))
+
+
 @pytest.mark.parametrize("T,E,K,B", [(4, 4, 2, 10), (300, 8, 2, 10), (1000, 128, 8, 1000), (64, 256, 8, 37),
                                      (513, 60, 4, 5000)])
 @pytest.mark.parametrize("padded", [False, True])

@@ -73,7 +73,7 @@ def test_gather_entry_points_reject_unaddressable_token_matrices_without_launchi
         assert rc == -1 and needle in lib.mi355_moe_last_error()
     # fp32 rows cannot be gathered at all
     rc = lib.mi355_grouped_swiglu_fwd(p, p, 8, p, p, p, 0, p, p, p, p, p, tiles, p, p, p, p, El, D, F, R, None)
-    assert rc == -1 and b"bf16 only" in lib.mi355_moe_last_error()
+    assert rc == -3 and b"bf16 only" in lib.mi355_moe_last_error()  # MI355_EUNSUP, as the header says
     # gate and up are omitted together or not at all, and only where the bf16 MFMA path runs
     rc = lib.mi355_grouped_swiglu_fwd(p, None, 8, p, p, p, 1, p, p, p, p, p, tiles, None, p, p, p, El, D, F, R, None)
     assert rc == -1 and b"together" in lib.mi355_moe_last_error()

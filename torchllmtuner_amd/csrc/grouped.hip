@@ -118,7 +118,7 @@ int check_common(const char* who, int dtype, int64_t El, int64_t D, int64_t F, i
 // index to [0, num_tokens): the token matrix must hold at least one row and stay below 4 GiB.
 int check_gather(const char* who, const int32_t* token_of_row, int64_t num_tokens, int64_t D, int dtype) {
   if (!token_of_row) return MI355_OK;
-  MI355_REQUIRE(dtype == MI355_BF16, "%s: the token gather exists for bf16 only", who);
+  if (dtype != MI355_BF16) return fail(MI355_EUNSUP, "%s: the token gather exists for bf16 only", who);
   MI355_REQUIRE(num_tokens >= 1, "%s: token_of_row given but num_tokens = %lld", who, (long long)num_tokens);
   MI355_REQUIRE(num_tokens < (1ll << 31) && num_tokens * D * 2 < (1ll << 32),
                 "%s: gathered token matrix of %lld x %lld bf16 exceeds the 4 GiB the fused gather addresses; "

@@ -560,6 +560,13 @@ extern "C" int mi355_permute_plan_static(const int64_t* ids, int64_t T, int64_t 
     return fail(MI355_ELAUNCH, "permute_plan_static: no current device");
   void* ptr = plan_scratch_ptr[dev].load(std::memory_order_acquire);
   if (!ptr) {
+    // The first call on a device resolves the array's address, which may load the code object:
+    // not something to do while a stream records a graph.  A caller who captures calls this
+    // entry point once, uncaptured, beforehand (any size; T = 0 will do).
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(as_stream(stream), &capturing) == hipSuccess && capturing != hipStreamCaptureStatusNone)
+      return fail(MI355_EINVAL, "permute_plan_static: the first call on a device must not be under stream capture "
+                                "(call it once before capturing)");
     const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(plan_scratch));
     if (e != hipSuccess || !ptr)
       return fail(MI355_ELAUNCH, "permute_plan_static: hipGetSymbolAddress: %s", hipGetErrorString(e));

@@ -174,7 +174,8 @@ __global__ __launch_bounds__(256) void select_fwd_kernel(
     // scores, and every score function here is non-decreasing in the logit: the experts are
     // then chosen by LOGIT, which is exact -- two implementations of exp() that differ in the
     // last ulp can order two nearly equal scores differently, but never two logits.
-    const bool by_logit = !expert_bias && num_groups == 0;
+    // (not when the caller asks for the cutoff: that is a choice VALUE, the (K+1)-th score)
+    const bool by_logit = !expert_bias && num_groups == 0 && !cutoff_out;
     float c[VPL];
 #pragma unroll
     for (int j = 0; j < VPL; ++j) {
@@ -425,7 +426,7 @@ __global__ __launch_bounds__(256) void select_rows_kernel(
     }
   } else {
 #pragma unroll
-    for (int j = 0; j < VPR; ++j) c[j] = num_groups > 0 ? s[j] : x[j];
+    for (int j = 0; j < VPR; ++j) c[j] = (num_groups > 0 || cutoff_out) ? s[j] : x[j];  // the cutoff is a score
   }
   if (num_groups > 0) {
     // group score = sum of the group's two best choice values: each lane folds its own, the lanes

@@ -141,39 +141,76 @@ class RoutedExperts(nn.Module):
 
     def forward(self, x_TD, topk_scores_TK, topk_expert_ids_TK, num_local_tokens_per_expert_E):
         """Dispatch tokens to experts, run them, and combine the results."""
-        del num_local_tokens_per_expert_E  # the plan counts on the device
         dispatcher = self.token_dispatcher
-        dispatcher._check_routing(x_TD, topk_scores_TK, topk_expert_ids_TK)
         experts = self.inner_experts
-        round_terms = not dispatcher.accumulate_in_fp32
         observe = (
             self.dispatch_observation.measure(x_TD.device)
             if self.dispatch_observation is not None
             else nullcontext()
         )
+        if not _is_own_dispatcher(dispatcher):
+            # Any other dispatcher is driven through the protocol alone, exactly as
+            # llmtuner/models/common/moe/experts.py:321-343 does: dispatch -> experts -> combine.
+            # That covers objects that implement only dispatch / combine and subclasses of this
+            # package's dispatchers that override dispatch, combine, plan or _permute_tokens.
+            with observe:
+                rows, counts_e, metadata = dispatcher.dispatch(
+                    x_TD, topk_scores_TK, topk_expert_ids_TK, num_local_tokens_per_expert_E
+                )
+            return dispatcher.combine(experts(rows, counts_e), metadata, x_TD)
+        # This package's own dispatchers: the counts handed in are the plan's own (MoE.forward
+        # takes them from the same plan), so the layout is read from the plan directly.
+        dispatcher._check_routing(x_TD, topk_scores_TK, topk_expert_ids_TK)
+        round_terms = not dispatcher.accumulate_in_fp32
         fused = (
             _is_plain_grouped_experts(experts)  # hooks on, or a subclass of, the inner module must run
             and ops.gather_supported(x_TD, experts.hidden_dim)
             and x_TD.is_contiguous()
             and ops.combine_bwd_slots(x_TD.dtype, x_TD.shape[-1], experts.hidden_dim) > 0
         )
-        if fused:
-            # the dispatch is the plan alone: the row gather rides inside the expert kernels'
-            # operand loads, and the combine's backward inside their backward
+        try:
+            if fused:
+                # the dispatch is the plan alone: the row gather rides inside the expert kernels'
+                # operand loads, and the combine's backward inside their backward
+                with observe:
+                    plan = dispatcher.plan(topk_expert_ids_TK)
+                w1, w3, w2 = experts._weights_as(x_TD.dtype)
+                out = Fn.gather_experts_combine(x_TD, topk_scores_TK, w1, w3, w2, plan, round_terms)
+                return out.to(x_TD.dtype)
             with observe:
                 plan = dispatcher.plan(topk_expert_ids_TK)
-            w1, w3, w2 = experts._weights_as(x_TD.dtype)
-            out = Fn.gather_experts_combine(x_TD, topk_scores_TK, w1, w3, w2, plan, round_terms)
+                rows = Fn.permute_rows(x_TD, plan)
+            # rows per local expert as laid out (padding included), the counts the reference hands
+            # to its inner module; rows past the last segment are not covered and come back as zeros
+            covered = plan.seg_offsets[1:] - plan.seg_offsets[:-1]
+            y = experts(rows, covered)
+            out = Fn.combine(y, topk_scores_TK, plan, round_terms)
             return out.to(x_TD.dtype)
-        with observe:
-            plan = dispatcher.plan(topk_expert_ids_TK)
-            rows = Fn.permute_rows(x_TD, plan)
-        # rows per local expert as laid out (padding included), the counts the reference hands
-        # to its inner module; rows past the last segment are not covered and come back as zeros
-        covered = plan.seg_offsets[1:] - plan.seg_offsets[:-1]
-        y = experts(rows, covered)
-        out = Fn.combine(y, topk_scores_TK, plan, round_terms)
-        return out.to(x_TD.dtype)
+        finally:
+            # the plan lives on in the autograd graph as long as a backward needs it; the
+            # dispatcher's own reference would keep its N-sized index arrays until the next step
+            dispatcher.forget_plan()
+
+
+def _is_own_dispatcher(dispatcher) -> bool:
+    """True when ``dispatcher`` is one of this package's dispatchers with ``dispatch``, ``combine``,
+    ``plan`` and ``_permute_tokens`` as this package defines them (a subclass that overrides none
+    of them included): only then may RoutedExperts.forward replace the three protocol calls by
+    the planned / fused kernels, which compute the same thing."""
+    from . import token_dispatch as td
+
+    cls = type(dispatcher)
+    if not isinstance(dispatcher, td.LocalTokenDispatcher):
+        return False
+    own_dispatch = {c.__dict__["dispatch"] for c in (td.LocalTokenDispatcher, td.PaddedTokenDispatcher,
+                                                     td.LocalShareTokenDispatcher)}
+    if getattr(cls, "dispatch", None) not in own_dispatch:
+        return False
+    base = td.LocalTokenDispatcher
+    if cls.combine is not base.combine or cls.plan is not base.plan or cls._permute_tokens is not base._permute_tokens:
+        return False
+    # methods patched onto the instance count as overrides too
+    return not any(name in vars(dispatcher) for name in ("dispatch", "combine", "plan", "_permute_tokens"))
 
 
 def _is_plain_grouped_experts(module: nn.Module) -> bool:

@@ -19,7 +19,7 @@ import torch
 import torch.nn as nn
 
 from .auxiliary_loss import in_checkpoint_recompute
-from .experts import RoutedExperts
+from .experts import RoutedExperts, _is_own_dispatcher
 from .routing import QuantileBalancedTopKRouter, TokenChoiceTopKRouter
 
 __all__ = ["MoE", "in_checkpoint_recompute"]
@@ -135,15 +135,20 @@ class MoE(nn.Module):
                     f"got {tuple(padding_mask.shape)} for {tokens.shape[0]} tokens."
                 )
 
-        topk_scores_TK, topk_expert_ids_TK, _routing_map_TE = self.router(
+        topk_scores_TK, topk_expert_ids_TK, routing_map_TE = self.router(
             tokens, self.expert_bias_E, padding_mask_T=padding_mask
         )
         # The reference counts by summing the routing map (layer.py:278); the permutation plan
         # counts the same slots on the device as a by-product, and the dispatcher hands that
         # very plan to the experts a moment later, so neither the sum nor a second plan is run.
+        # A dispatcher that is not this package's own (anything that only implements the
+        # dispatch / combine protocol, token_dispatch.py:201-275) has no plan: the counts are then
+        # the column sums of the routing map, as in the reference.
         dispatcher = self.routed_experts.token_dispatcher
-        plan = dispatcher.plan(topk_expert_ids_TK)
-        num_tokens_per_expert_E = plan.counts_E
+        if _is_own_dispatcher(dispatcher):
+            num_tokens_per_expert_E = dispatcher.plan(topk_expert_ids_TK).counts_E
+        else:
+            num_tokens_per_expert_E = routing_map_TE.sum(dim=0)
         out_TD = self.routed_experts(tokens, topk_scores_TK, topk_expert_ids_TK, num_tokens_per_expert_E)
 
         if self.shared_experts is not None:
@@ -154,7 +159,7 @@ class MoE(nn.Module):
                 if padding_mask is None:
                     valid_counts_E = num_tokens_per_expert_E  # int32; add_ promotes inside its one kernel
                 else:
-                    keep = (~padding_mask).to(torch.float32).repeat_interleave(plan.top_k)
+                    keep = (~padding_mask).to(torch.float32).repeat_interleave(topk_expert_ids_TK.shape[-1])
                     valid_counts_E = torch.zeros_like(self.tokens_per_expert_E).scatter_add_(
                         0, topk_expert_ids_TK.reshape(-1), keep
                     )

@@ -91,7 +91,11 @@ class LocalTokenDispatcher:
         self.num_experts = num_experts
         self.top_k = top_k
         self.accumulate_in_fp32 = False
-        self._last_plan = None  # (weakref to the ids tensor, its version, the plan made for it)
+        # combine() of a record that carries only the reference's two fields checks that every
+        # token owns exactly top_k rows; the check reads one flag back from the device (a host
+        # synchronisation) and can be switched off by callers who build such records themselves
+        self.validate_foreign_records = True
+        self._last_plan = None  # (weakref to the ids tensor, its version, the plan made for it, its layout key)
 
     def set_ep_group(self, *, ep_group=None) -> None:
         """No-op: there is no expert-parallel group on one GPU."""
@@ -119,16 +123,36 @@ class LocalTokenDispatcher:
         and returned again for the very same tensor object (unchanged since): the block asks
         for the counts first and the experts for the layout right after."""
         ids = topk_expert_ids_TK
-        last = self._last_plan
-        if last is not None and last[0]() is ids and last[1] == ids._version:
-            return last[2]
         lo, hi = self._local_range()
+        layout = (self.num_experts, lo, hi, self._align())
+        last = self._last_plan
+        if last is not None and last[0]() is ids and last[1] == ids._version and last[3] == layout:
+            return last[2]
         plan = ops.permute_plan(ids, self.num_experts, lo, hi, self._align())
         try:
-            self._last_plan = (weakref.ref(ids), ids._version, plan)
+            self._last_plan = (weakref.ref(ids), ids._version, plan, layout)
         except TypeError:  # tensor subclasses without weak references: no memo
             self._last_plan = None
         return plan
+
+    def forget_plan(self) -> None:
+        """Drop the kept plan (its index arrays are N-sized); the next ``plan()`` builds anew."""
+        self._last_plan = None
+
+    def _permute_tokens(self, inputs, token_indices, expert_ids):
+        """Gather tokens into expert-major rows -- the hook of token_dispatch.py:197-199
+        ("backend adapters may own the repeated-index VJP").  This class's own gather is the
+        plan's row kernel, whose backward is the K-way row sum in a fixed order; it takes the
+        layout from the plan of ``expert_ids`` and does not read ``token_indices`` (``dispatch``
+        passes None here and the token of every row, int64 with -1 for padding rows, to an
+        override)."""
+        del token_indices
+        return Fn.permute_rows(inputs, self.plan(expert_ids))
+
+    def _gather_rows(self, x_TD, topk_expert_ids_TK, metadata: "LocalDispatchMetadata"):
+        overridden = type(self)._permute_tokens is not LocalTokenDispatcher._permute_tokens
+        token_indices = metadata.token_indices_experts_sorted_N if overridden else None
+        return self._permute_tokens(x_TD, token_indices, topk_expert_ids_TK)
 
     def _rows_for_combine(self, routed_output_RD, metadata: "LocalDispatchMetadata"):
         """(plan, scores_TK) for a record that only carries the reference's two fields: with
@@ -139,7 +163,8 @@ class LocalTokenDispatcher:
             raise ValueError("combine: the dispatch record does not hold top_k rows per token")
         T = tok.numel() // K
         order = torch.argsort(tok, stable=True)
-        if T > 0 and not bool((tok[order].view(T, K) == torch.arange(T, device=tok.device)[:, None]).all()):
+        if self.validate_foreign_records and T > 0 and not bool(
+                (tok[order].view(T, K) == torch.arange(T, device=tok.device)[:, None]).all()):
             raise ValueError("combine: the dispatch record does not hold top_k rows per token")
         row_of_slot = order.to(torch.int32)
         inv = torch.empty_like(row_of_slot)
@@ -154,8 +179,8 @@ class LocalTokenDispatcher:
     def dispatch(self, x_TD, topk_scores_TK, topk_expert_ids_TK, num_local_tokens_per_expert_E):
         self._check_routing(x_TD, topk_scores_TK, topk_expert_ids_TK)
         plan = self.plan(topk_expert_ids_TK)
-        rows = Fn.permute_rows(x_TD, plan)
         metadata = LocalDispatchMetadata(plan=plan, topk_scores_TK=topk_scores_TK)
+        rows = self._gather_rows(x_TD, topk_expert_ids_TK, metadata)
         return rows, num_local_tokens_per_expert_E, metadata
 
     def combine(self, routed_output_RD, metadata: LocalDispatchMetadata, x_TD):
@@ -182,12 +207,12 @@ class PaddedTokenDispatcher(LocalTokenDispatcher):
     def dispatch(self, x_TD, topk_scores_TK, topk_expert_ids_TK, num_local_tokens_per_expert_E):
         self._check_routing(x_TD, topk_scores_TK, topk_expert_ids_TK)
         plan = self.plan(topk_expert_ids_TK)
-        rows = Fn.permute_rows(x_TD, plan)
+        metadata = LocalDispatchMetadata(plan=plan, topk_scores_TK=topk_scores_TK)
+        rows = self._gather_rows(x_TD, topk_expert_ids_TK, metadata)
         # Resolving the covered size reads one int from the device, as the reference's
         # adapter does (torchao_dispatch.py:167).
         covered = int(plan.total_rows.item())
         padded_counts = (plan.seg_offsets[1:] - plan.seg_offsets[:-1]).to(torch.int64)
-        metadata = LocalDispatchMetadata(plan=plan, topk_scores_TK=topk_scores_TK)
         return rows[:covered], padded_counts, metadata
 
 
@@ -210,7 +235,7 @@ class LocalShareTokenDispatcher(LocalTokenDispatcher):
     def dispatch(self, x_TD, topk_scores_TK, topk_expert_ids_TK, num_local_tokens_per_expert_E):
         self._check_routing(x_TD, topk_scores_TK, topk_expert_ids_TK)
         plan = self.plan(topk_expert_ids_TK)
-        rows = Fn.permute_rows(x_TD, plan)
-        covered = int(plan.total_rows.item())
         metadata = LocalDispatchMetadata(plan=plan, topk_scores_TK=topk_scores_TK)
+        rows = self._gather_rows(x_TD, topk_expert_ids_TK, metadata)
+        covered = int(plan.total_rows.item())
         return rows[:covered], plan.seg_counts.to(torch.int64), metadata
