@@ -255,7 +255,9 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
 #pragma unroll
     for (int i = 0; i < NA; ++i) {
       const int r = max(min(kc_row + 64 * i, m.valid - 1), 0);
-      asrc[i] = GATHER ? min(max(p.a_src[m.row0 + r], 0), p.a_rows - 1) : r;
+      // (the index as loaded: it is clamped to [0, a_rows) where it is used, in setup(), a whole K
+      // loop later, so that nothing waits for this load here)
+      asrc[i] = GATHER ? p.a_src[m.row0 + r] : r;
     }
   };
   auto setup = [&](const TileMeta& m, const int (&asrc)[NA]) {
@@ -263,8 +265,10 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
     rsA0 = make_rsrc(p.a0 + arow);
     rsA1 = (MODE == RM_DX) ? make_rsrc(p.a1 + arow) : rsA0;
 #pragma unroll
-    for (int i = 0; i < NA; ++i)
-      voffA[i] = (static_cast<uint32_t>(asrc[i]) * static_cast<uint32_t>(lda) + static_cast<uint32_t>(kc_chunk * 8)) * 2u;
+    for (int i = 0; i < NA; ++i) {
+      const int src = GATHER ? min(max(asrc[i], 0), p.a_rows - 1) : asrc[i];
+      voffA[i] = (static_cast<uint32_t>(src) * static_cast<uint32_t>(lda) + static_cast<uint32_t>(kc_chunk * 8)) * 2u;
+    }
     const uint16_t* B0 = p.b0 + m.e * wsz;
     const uint16_t* B1 = (MODE == RM_GATEUP || MODE == RM_DX) ? p.b1 + m.e * wsz : B0;
     // KC: the tile's first weight row is n0; KS: its first column is n0
@@ -708,21 +712,26 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
   };
   // B row of this thread's chunk i in K step `step` of segment (s0, c): its own row, or
   // (gather) the source row from the index array.  Needs c > 0.
+  // (a gathered index is returned as loaded and clamped to [0, src_rows) only where it is used,
+  // a K step later: clamping here would make the wave wait for the index right away, and with it
+  // -- the load counter retires in order -- for every operand load requested before it)
   auto row_index = [&](int s0, int c, int step, int i) -> int {
     const int k = min(step * BK + ks_k + 16 * i, c - 1);
-    return GATHER ? min(max(p.b_src[s0 + k], 0), p.src_rows - 1) : k;
+    return GATHER ? p.b_src[s0 + k] : k;
   };
   // the same for the A row (its own row unless A is gathered too)
   auto a_row_index = [&](int s0, int c, int step, int i) -> int {
     const int k = min(step * BK + ks_k + 16 * i, c - 1);
-    return GATHER_A ? min(max(p.a_src[s0 + k], 0), p.src_rows - 1) : k;
+    return GATHER_A ? p.a_src[s0 + k] : k;
   };
+  auto clamp_src = [&](int r) -> int { return min(max(r, 0), p.src_rows - 1); };
   // Loads of one K step, unconditional: rows past the segment re-read its last row and
   // the A side is zeroed when it is parked, so the products vanish.  Needs cnt > 0.
   auto load_ab = [&](int step, int i, int brow, int arow_g) {
-    const int k = GATHER_A ? arow_g : min(step * BK + ks_k + 16 * i, cnt - 1);
+    const int k = GATHER_A ? clamp_src(arow_g) : min(step * BK + ks_k + 16 * i, cnt - 1);
+    const int kb = GATHER ? clamp_src(brow) : brow;
     ra[i] = *reinterpret_cast<const u32x4*>(a_base + static_cast<int64_t>(k) * M);
-    rb[i] = *reinterpret_cast<const u32x4*>(b_base + static_cast<int64_t>(brow) * N);
+    rb[i] = *reinterpret_cast<const u32x4*>(b_base + static_cast<int64_t>(kb) * N);
   };
   auto park = [&](int step, int i, uint16_t* An, uint16_t* Bn, int count) {
     const bool live = step * BK + ks_k + 16 * i < count;
@@ -733,13 +742,16 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
   int aidx[4];  // A rows likewise (used when A is gathered)
   set_bases();
   if (cnt > 0) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) load_ab(0, i, row_index(seg0, cnt, 0, i), a_row_index(seg0, cnt, 0, i));
+    // (requests always go out as operands, then the next index, chunk after chunk: the K loop's
+    // waits count the requests that follow the one they need along every way into the loop)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
+      __builtin_amdgcn_sched_barrier(0);
+      load_ab(0, i, row_index(seg0, cnt, 0, i), a_row_index(seg0, cnt, 0, i));
       bidx[i] = row_index(seg0, cnt, 1, i);
       aidx[i] = a_row_index(seg0, cnt, 1, i);
     }
+    __builtin_amdgcn_sched_barrier(0);
   }
   // expert and segment of the next tile, expert of the one after it (its segment is
   // looked up inside the loop, the expert after that too)
@@ -779,13 +791,17 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) park(0, i, smem, smem + WBM * BK, c_cnt);
       if (ksteps > 1) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) load_ab(1, i, bidx[i], aidx[i]);
+        // in the order of a K step of the loop below (operands, then the next index, chunk after
+        // chunk, and kept in that order): the loop's waits count the requests that follow the one
+        // they need, on both ways into the loop, so both ways must issue them alike
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
+          __builtin_amdgcn_sched_barrier(0);
+          load_ab(1, i, bidx[i], aidx[i]);
           bidx[i] = row_index(c_seg0, c_cnt, 2, i);
           aidx[i] = a_row_index(c_seg0, c_cnt, 2, i);
         }
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
     __syncthreads();
@@ -813,6 +829,14 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
 #pragma unroll
         for (int nj = 0; nj < 4; ++nj) bf[nj] = frag_ks<256>(Bs, wn + nj * 32, kk, lane);
         if constexpr (has_next) park(ks + 1, kk, An, Bn, c_cnt);
+        // Nothing is moved across this point: the requests below stay in their quarter of the K
+        // step (left alone, the compiler gathers all of a step's global loads at its end, where
+        // the data they fetch is parked a moment later instead of a whole step later, and the
+        // wave waits out the memory latency once per K step), and an index is clamped a whole
+        // step after it was requested.  What lies between two such points -- this quarter's
+        // requests and MFMAs, the next quarter's fragment reads and its park -- is still
+        // interleaved freely.
+        __builtin_amdgcn_sched_barrier(0);
         if constexpr (has_next2) {
           load_ab(ks + 2, kk, bidx[kk], aidx[kk]);
           bidx[kk] = row_index(c_seg0, c_cnt, ks + 3, kk);
@@ -844,12 +868,13 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
       set_bases();
       if (cnt > 0) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) load_ab(0, i, nidx[i], nidx_a[i]);
-#pragma unroll
         for (int i = 0; i < 4; ++i) {
+          __builtin_amdgcn_sched_barrier(0);
+          load_ab(0, i, nidx[i], nidx_a[i]);
           bidx[i] = row_index(seg0, cnt, 1, i);
           aidx[i] = a_row_index(seg0, cnt, 1, i);
         }
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
 
