@@ -957,6 +957,24 @@ template <int MODE, bool GATHER = false, bool SAVE_GU = true>
 static int launch_row(RowArgs& a, int64_t width, int64_t tile_capacity, hipStream_t s, const char* what) {
   constexpr int div = MODE == RM_GATEUP ? 2 : 1;
   a.n_tiles = (int)((width + 256 / div - 1) / (256 / div));
+  // A product with so few row tiles that 256-column tiles would leave a quarter of the CUs or more without work
+  // (the dH of one dense segment: 4096 rows x 2048 columns are 16 x 8 tiles) runs on 128-column
+  // tiles instead: twice the work items, each with the whole contraction.  Only where the
+  // epilogue does not depend on the tile width (the folded dH writes one partial per 128
+  // columns of a 256-column tile).
+  if constexpr (MODE == RM_DH && !GATHER) {
+    if (tile_capacity * a.n_tiles * 4 <= resident_blocks() * 3 && width >= 128) {  // (the capacity is an upper bound)
+      a.n_tiles = (int)((width + 127) / 128);
+      static PerDeviceOnce narrow_configured;
+      if (narrow_configured.needed()) {
+        if (int rc = set_lds(row_tiled_kernel<MODE, 2, GATHER, 4, SAVE_GU>, W_LDS_BYTES)) return rc;
+        narrow_configured.done();
+      }
+      const unsigned blocks = std::min(round8(tile_capacity * a.n_tiles), resident_blocks());
+      hipLaunchKernelGGL((row_tiled_kernel<MODE, 2, GATHER, 4, SAVE_GU>), dim3(blocks), dim3(NT), W_LDS_BYTES, s, a);
+      return check_launch(what);
+    }
+  }
   static PerDeviceOnce configured;  // one per kernel instantiation
   if (configured.needed()) {
     if (int rc = set_lds(row_tiled_kernel<MODE, 4, GATHER, 4, SAVE_GU>, W_LDS_BYTES)) return rc;

@@ -197,20 +197,31 @@ def _is_own_dispatcher(dispatcher) -> bool:
     ``plan`` and ``_permute_tokens`` as this package defines them (a subclass that overrides none
     of them included): only then may RoutedExperts.forward replace the three protocol calls by
     the planned / fused kernels, which compute the same thing."""
-    from . import token_dispatch as td
-
     cls = type(dispatcher)
-    if not isinstance(dispatcher, td.LocalTokenDispatcher):
-        return False
-    own_dispatch = {c.__dict__["dispatch"] for c in (td.LocalTokenDispatcher, td.PaddedTokenDispatcher,
-                                                     td.LocalShareTokenDispatcher)}
-    if getattr(cls, "dispatch", None) not in own_dispatch:
-        return False
-    base = td.LocalTokenDispatcher
-    if cls.combine is not base.combine or cls.plan is not base.plan or cls._permute_tokens is not base._permute_tokens:
+    seams = (getattr(cls, "dispatch", None), getattr(cls, "combine", None), getattr(cls, "plan", None),
+             getattr(cls, "_permute_tokens", None))
+    own = _OWN_DISPATCHER_CLASSES.get(seams)  # keyed by the functions themselves: a class patched later misses
+    if own is None:
+        from . import token_dispatch as td
+
+        base = td.LocalTokenDispatcher
+        own_dispatch = {c.__dict__["dispatch"] for c in (base, td.PaddedTokenDispatcher, td.LocalShareTokenDispatcher)}
+        own = (
+            issubclass(cls, base)
+            and getattr(cls, "dispatch", None) in own_dispatch
+            and cls.combine is base.combine
+            and cls.plan is base.plan
+            and cls._permute_tokens is base._permute_tokens
+        )
+        _OWN_DISPATCHER_CLASSES[seams] = own
+    if not own:
         return False
     # methods patched onto the instance count as overrides too
-    return not any(name in vars(dispatcher) for name in ("dispatch", "combine", "plan", "_permute_tokens"))
+    d = getattr(dispatcher, "__dict__", None)
+    return not d or not ("dispatch" in d or "combine" in d or "plan" in d or "_permute_tokens" in d)
+
+
+_OWN_DISPATCHER_CLASSES: dict = {}  # a class's four seam methods -> whether they are this package's own
 
 
 def _is_plain_grouped_experts(module: nn.Module) -> bool:

@@ -231,8 +231,46 @@ def _(dout, x, weights, w1, w3, w2, gate, up, token_of_row, slot_of_row, row_of_
 
 # ====================================================================== autograd formulas
 # Each differentiable operator's backward is the hand-written kernel for that stage.
+# The registration is what ``torch.library.register_autograd`` does -- a Python kernel for the
+# operator's Autograd dispatch key that wraps the call in an ``autograd.Function`` -- without
+# its per-call ``fill_defaults``: that helper re-reads ``schema.arguments`` (a fresh list of
+# wrapped argument objects) once per argument, about 18 us for our twenty-argument operators
+# and a fifth of the host time of a small step, to put back arguments that the dispatcher drops
+# when they equal their schema default.  None of these schemas declares a default, so nothing
+# is ever dropped.
+_AUTOGRAD_LIB = torch.library.Library("mi355_moe", "FRAGMENT")
+_AFTER_AUTOGRAD = torch._C._after_autograd_keyset
+_BELOW_AUTOGRAD = torch._C._AutoDispatchBelowAutograd
+_ANY_REQUIRES_GRAD = torch._C._any_requires_grad
+
+
 def _autograd(name, backward, setup):
-    torch.library.register_autograd(f"mi355_moe::{name}", backward, setup_context=setup)
+    op = getattr(torch.ops.mi355_moe, name).default
+    if any(a.has_default_value() for a in op._schema.arguments):
+        raise RuntimeError(f"mi355_moe::{name}: schema defaults would need torch.library.register_autograd")
+
+    def forward(ctx, *args):
+        keyset, args = args[-1], args[:-1]
+        with _BELOW_AUTOGRAD():
+            result = op.redispatch(keyset & _AFTER_AUTOGRAD, *args)
+        setup(ctx, args, result)
+        return result
+
+    def backward_(ctx, *grads):
+        ctx.needs_input_grad = ctx.needs_input_grad[:-1]  # the key set rides along as a last, non-tensor input
+        result = backward(ctx, *grads)
+        return (*result, None) if isinstance(result, tuple) else (result, None)
+
+    generated = type(f"GeneratedBackwardFor_mi355_moe_{name}", (torch.autograd.Function,),
+                     {"forward": staticmethod(forward), "backward": staticmethod(backward_)})
+
+    def autograd_kernel(keyset, *args):
+        if torch.is_grad_enabled() and _ANY_REQUIRES_GRAD(*args):
+            return generated.apply(*args, keyset)
+        with _BELOW_AUTOGRAD():
+            return op.redispatch(keyset & _AFTER_AUTOGRAD, *args)
+
+    _AUTOGRAD_LIB.impl(name, autograd_kernel, "Autograd", with_keyset=True)
 
 
 # -- router gate: dX in the input dtype, dW in the weight dtype (linear.py:133-151)
@@ -581,17 +619,11 @@ class PermutePlan:
 
 
 def _split_small(small, E, El, tile_cap):
-    o = 0
-    counts_E = None
-    if E:
-        counts_E = small[o:o + E]; o += E
-    seg_offsets = small[o:o + El + 1]; o += El + 1
-    # 2*El ints: the counts, then the experts by descending count
-    seg_counts = small[o:o + El]; expert_order = small[o + El:o + 2 * El]; o += 2 * El
-    tile_expert = small[o:o + tile_cap]; o += tile_cap
-    tile_row0 = small[o:o + tile_cap]; o += tile_cap
-    num_tiles = small[o:o + 1]
-    return counts_E, seg_offsets, seg_counts, expert_order, tile_expert, tile_row0, num_tiles
+    # one call for the seven views (sliced one by one they cost a microsecond of host time each);
+    # 2*El ints hold the counts, then the experts by descending count
+    sizes = [E, El + 1, El, El, tile_cap, tile_cap, 1]
+    counts_E, seg_offsets, seg_counts, expert_order, tile_expert, tile_row0, num_tiles = small[:sum(sizes)].split(sizes)
+    return (counts_E if E else None), seg_offsets, seg_counts, expert_order, tile_expert, tile_row0, num_tiles
 
 
 def permute_plan(ids_TK, num_experts, local_lo=0, local_hi=None, align=1) -> PermutePlan:
