@@ -81,6 +81,8 @@ def parse():
     ap.add_argument("--single-workload", dest="all_workloads", action="store_false",
                     help="measure --workload only (default: the other four configurations follow it, a short run "
                          "each, and are summarised under \"workloads\")")
+    ap.add_argument("--settle-steps", type=int, default=30,
+                    help="untimed steps before the warm-up that bring the card from its idle clocks to the ones it holds")
     ap.add_argument("--other-steps", type=int, default=20)
     ap.add_argument("--other-warmup", type=int, default=10)
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -583,6 +585,12 @@ def measure_workload(args, wl, steps, warmup, *, detail):
             with torch.no_grad():
                 block(x)
 
+    # The card leaves its idle clocks over the first fifteen or so steps of a process (at C3:
+    # 3.4, 3.1, 2.9, 2.75 ... ms, level from the fifteenth on), whatever the caller's warm-up
+    # count: settle first, untimed, then do the W warm-up steps and time exactly K.
+    for _ in range(args.settle_steps):
+        step()
+    torch.cuda.synchronize()
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
