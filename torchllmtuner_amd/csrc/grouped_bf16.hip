@@ -302,11 +302,19 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
   };
   auto kofs = [&](int ks) { return ks * BK; };
   // request every chunk of K step `step` of the fetch tile
+  // (chunk after chunk in the order of a K step of the loop below, and kept in that order: the
+  // loop's waits count the requests that follow the one they need along every way into the loop,
+  // so every way must issue them alike -- with all A chunks first the park of the first B chunk
+  // waited for five requests more than it needed)
   auto issue = [&](int step) {
 #pragma unroll
-    for (int i = 0; i < NA; ++i) ra[i] = load_a(kofs(step), i);
+    for (int q = 0; q < 4; ++q) {
+      __builtin_amdgcn_sched_barrier(0);
+      if (q < NA) ra[q] = load_a(kofs(step), q);
 #pragma unroll
-    for (int i = 0; i < NB; ++i) rb[i] = load_b(kofs(step), i);
+      for (int i = (q * NB) / 4; i < ((q + 1) * NB) / 4; ++i) rb[i] = load_b(kofs(step), i);
+    }
+    __builtin_amdgcn_sched_barrier(0);
   };
 
   TileMeta cur = load_meta(within);
