@@ -4,7 +4,7 @@
 tensor-level calls into ``libmi355moe.so`` (C ABI in ``include/mi355_moe.h``).
 """
 
-from . import _lib, functional, kernel_registry, moe, ops  # noqa: F401
+from . import _lib, kernel_registry, moe, ops  # noqa: F401
 from .moe import (  # noqa: F401
     DenseSwiGLU,
     GroupedExperts,

@@ -32,7 +32,7 @@ from typing import Any, TypeVar
 
 import torch
 
-from . import functional as F
+from . import ops as F
 from . import ops
 
 logger = logging.getLogger(__name__)

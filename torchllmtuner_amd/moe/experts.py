@@ -23,7 +23,7 @@ from typing import Protocol
 import torch
 import torch.nn as nn
 
-from .. import functional as Fn
+from .. import ops as Fn
 from .. import ops
 from .activation import SwiGLU
 

@@ -11,7 +11,7 @@ from __future__ import annotations
 import torch
 import torch.nn as nn
 
-from .. import functional as Fn
+from .. import ops as Fn
 
 __all__ = ["RouterGateLinear"]
 

@@ -20,7 +20,7 @@ from typing import Literal
 import torch
 import torch.nn as nn
 
-from .. import functional as Fn
+from .. import ops as Fn
 from .. import ops
 from .auxiliary_loss import in_checkpoint_recompute
 from .linear import RouterGateLinear

@@ -26,7 +26,7 @@ import weakref
 
 import torch
 
-from .. import functional as Fn
+from .. import ops as Fn
 from .. import ops
 
 __all__ = [
