@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define MI355_MOE_ABI_VERSION 2
+#define MI355_MOE_ABI_VERSION 3
 
 /* element types of activation / weight buffers */
 #define MI355_F32 0
@@ -448,6 +448,32 @@ int mi355_grouped_swiglu_stage(int stage, const void* dy, const void* rows,
                                int64_t tile_capacity, void* dgate, void* dup, void* drows,
                                void* dw1, void* dw3, void* dw2, int64_t El, int64_t D,
                                int64_t F, int64_t row_capacity, void* stream);
+
+/*
+ * One grouped linear map over expert-major rows, the reference's pluggable
+ * GroupedExperts._grouped_mm(x_TD, weight_EOI, offsets_E)
+ * (llmtuner/models/common/moe/experts.py:211-216, :256-285):
+ *   y[r] = x[r] . w[e(r)]^T      x (rows, I), w (El, O, I) row-major, y (rows, O)
+ * over the segments of a plan / of mi355_segments_from_counts, fp32 accumulation, one rounding
+ * to `dtype` (fp32 or bf16; x, w and y share it).  It is what GroupedExperts is built from when
+ * its gated activation is not SwiGLU (llmtuner/models/common/activation.py:40-64, SituGLU):
+ * gate = linear(x, w1), up = linear(x, w3), h = activation(gate, up), y = linear(h, w2).
+ * bf16 with I and O multiples of 64 (>= 384) runs the MFMA kernels of the SwiGLU path (the down
+ * projection's kernel forward, the dH product with a plain epilogue for dx, the dW2 kernel for
+ * dw); everything else the strided fp32-MFMA GEMM.  Rows outside the listed segments are not
+ * written.  The backward (autograd of the above): dx[r] = dy[r] . w[e(r)], dw[e] = sum over the
+ * segment of dy[r]^T x[r]; dx or dw may be NULL; an expert without rows gets a zero dw.
+ */
+int mi355_grouped_linear_fwd(const void* x, const void* w, int dtype, const int32_t* seg_offsets,
+                             const int32_t* seg_counts, const int32_t* tile_expert,
+                             const int32_t* tile_row0, const int32_t* num_tiles,
+                             int64_t tile_capacity, void* y, int64_t El, int64_t I, int64_t O,
+                             int64_t row_capacity, void* stream);
+int mi355_grouped_linear_bwd(const void* dy, const void* x, const void* w, int dtype,
+                             const int32_t* seg_offsets, const int32_t* seg_counts,
+                             const int32_t* tile_expert, const int32_t* tile_row0,
+                             const int32_t* num_tiles, int64_t tile_capacity, void* dx, void* dw,
+                             int64_t El, int64_t I, int64_t O, int64_t row_capacity, void* stream);
 
 /*
  * RMS normalisation over the last axis, the `rms_norm` entry of the reference's kernel

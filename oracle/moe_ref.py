@@ -26,6 +26,10 @@ Pinning status (tests/test_oracle.py holds the checks):
   permute_and_pad        pinned: invariants padded=c+(-c%m), rows==sum(padded),
                          equality with the local path after combine, analytic 2*sum(w)
   grouped_experts        pinned: per-segment hand reference, zero-count segments fp64
+  situ_glu               pinned: the explicit formula of the reference's own test
+                         (tests/unit_tests/cpu/models/test_situ_activation.py:31-45) for
+                         linear_beta None / 0 / 1.7, values and gradients; |out| <= beta*|up|
+                         and the small-argument limit gate*up/2
   combine                pinned: inverse-permute/reshape/sum reference, fp64 exactness
   moe_forward            pinned: analytic experts x(id+1), brute-force fp64 loop
   balance_loss           pinned: the paper formula, even-load value, scale and order invariance
@@ -62,6 +66,7 @@ __all__ = [
     "permute_and_pad",
     "unpermute_padded",
     "grouped_experts",
+    "situ_glu",
     "combine",
     "shared_expert",
     "balance_loss",
@@ -271,17 +276,30 @@ def _segment_linear(x_RI, w_EOI, counts):
     return out
 
 
-def grouped_experts(x_RD, counts_E, w1_EFD, w3_EFD, w2_EDF):
+def situ_glu(gate, up, beta=1.0, linear_beta=None):
+    """``SituGLU.forward`` (activation.py:58-64): fp32 arithmetic, result in the gate's dtype."""
+    g, u = gate.float(), up.float()
+    act = beta * torch.tanh(g / beta) * g.sigmoid()
+    if linear_beta not in (None, 0.0):
+        u = linear_beta * torch.tanh(u / linear_beta)
+    return (act * u).to(gate.dtype)
+
+
+def grouped_experts(x_RD, counts_E, w1_EFD, w3_EFD, w2_EDF, activation=None):
     """``GroupedExperts._compute`` (experts.py:204-209) on the loop path.
 
-    gate, up and the SwiGLU product are each materialised in the activation
-    dtype, which is where the reference's bf16 rounding points are.
+    gate, up and the activation's product are each materialised in the activation
+    dtype, which is where the reference's bf16 rounding points are.  ``activation``
+    is the ``(gate, up)`` function of experts.py:207; None is SwiGLU.
     """
     counts = [int(c) for c in counts_E.tolist()]
     assert sum(counts) == x_RD.shape[0]
     gate = _segment_linear(x_RD, w1_EFD, counts)
     up = _segment_linear(x_RD, w3_EFD, counts)
-    h = F.silu(gate) * up  # activation.py:36-37
+    if activation is None:
+        h = F.silu(gate) * up  # activation.py:36-37
+    else:
+        h = activation(gate, up)
     return _segment_linear(h, w2_EDF, counts).type_as(x_RD)
 
 
@@ -414,12 +432,14 @@ def moe_forward(
     pad_multiple: int | None = None,
     accumulate_in_fp32: bool = False,
     local_experts: tuple[int, int] | None = None,
+    activation=None,
 ):
     """``MoE.forward`` (layer.py:268-309) at EP=1.
 
     ``pad_multiple`` routes through the padded permute; ``local_experts=(lo, hi)``
     computes only experts ``[lo, hi)`` (weights given for those experts only) and
     drops the other assignments from compute while still counting them.
+    ``activation``: the experts' gated activation (None is SwiGLU).
     Returns ``(out, aux)`` where ``aux`` holds ids, scores, counts and the sorted
     token indices for parity checks.
     """
@@ -436,12 +456,12 @@ def moe_forward(
     rows, tok_l, s_l = rows[start:stop], tok[start:stop], s_sorted[start:stop]
     local_counts = counts_E[lo:hi]
     if pad_multiple is None:
-        y = grouped_experts(rows, local_counts, p.w1_EFD, p.w3_EFD, p.w2_EDF)
+        y = grouped_experts(rows, local_counts, p.w1_EFD, p.w3_EFD, p.w2_EDF, activation)
     else:
         ext_shape, padded_rows, pidx, padded_counts = permute_and_pad(
             rows, local_counts, pad_multiple
         )
-        y_pad = grouped_experts(padded_rows, padded_counts, p.w1_EFD, p.w3_EFD, p.w2_EDF)
+        y_pad = grouped_experts(padded_rows, padded_counts, p.w1_EFD, p.w3_EFD, p.w2_EDF, activation)
         y = unpermute_padded(y_pad, ext_shape, pidx)
     out = combine(y, tok_l, s_l, tokens, accumulate_in_fp32)
     if p.shared_gate_FD is not None:

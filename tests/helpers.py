@@ -74,7 +74,7 @@ def make_params(E, D, F, dtype, seed=0, std=0.02, shared_F=None, El=None):
 
 
 def build_block(p: R.MoEParams, spec: R.RouterSpec, D, F, dtype, device, *, dispatcher="local",
-                pad_multiple=None, local=None, load_balance_coeff=None):
+                pad_multiple=None, local=None, load_balance_coeff=None, activation=None):
     """The device MoE block holding exactly the oracle's parameters."""
     from torchllmtuner_amd import moe
 
@@ -94,7 +94,7 @@ def build_block(p: R.MoEParams, spec: R.RouterSpec, D, F, dtype, device, *, disp
     shared = None
     if p.shared_gate_FD is not None:
         shared = moe.DenseSwiGLU(D, p.shared_gate_FD.shape[0])
-    block = moe.MoE(E, moe.RoutedExperts(moe.GroupedExperts(D, F, El), disp), router,
+    block = moe.MoE(E, moe.RoutedExperts(moe.GroupedExperts(D, F, El, activation_fn=activation), disp), router,
                     load_balance_coeff=load_balance_coeff, shared_experts=shared)
     block = block.to(dtype)
     block.router.gate.float()  # router stays fp32 under bf16 experts

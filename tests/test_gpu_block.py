@@ -29,6 +29,8 @@ def _run_pair(p, spec, x, gout, dtype, D, F, **kw):
               if getattr(p, k) is not None}
     pr = R.MoEParams(expert_bias_E=p.expert_bias_E, router_logit_bias_E=p.router_logit_bias_E, **leaves)
     xr = x.clone().requires_grad_()
+    if kw.get("activation") is not None:  # the module itself is the oracle's (gate, up) function: plain torch on the CPU
+        oracle_kw["activation"] = kw["activation"]
     ref, aux = R.moe_forward(xr, pr, spec, **oracle_kw)
     ref.backward(gout)
     block = build_block(p, spec, D, F, dtype, DEV, load_balance_coeff=1e-3 if p.expert_bias_E is not None else None, **kw)
@@ -119,6 +121,61 @@ def test_qwen3_shape_bf16_forward_backward(dispatcher, T):
     for k in want:
         err = rel_l2(got[k], want[k])
         assert err < 2e-2, f"{k}: rel-L2 {err}"
+
+
+@pytest.mark.parametrize("dtype,T,D,E,K,F,dispatcher", [
+    (torch.float32, 300, 64, 8, 2, 96, "local"),
+    (torch.bfloat16, 700, 512, 16, 4, 384, "local"),
+    (torch.bfloat16, 900, 384, 16, 4, 640, "padded"),
+    (torch.bfloat16, 700, 512, 16, 4, 384, "share"),
+])
+def test_block_with_the_situ_activation_matches_the_oracle(dtype, T, D, E, K, F, dispatcher):
+    """Experts with SituGLU (activation.py:40-64) instead of SwiGLU: gate, up and down run as
+    grouped linear maps with the module's own torch arithmetic between them.  The oracle calls
+    the restated formula (oracle.moe_ref.situ_glu), not the package's module."""
+    from torchllmtuner_amd import moe
+
+    print(f"block situ {dtype} T={T} D={D} E={E} K={K} F={F} {dispatcher}", flush=True)
+    spec = R.RouterSpec(E, K, score_func="sigmoid", route_norm=True)
+    kw = {}
+    El = E
+    if dispatcher == "padded":
+        kw = dict(dispatcher="padded", pad_multiple=64)
+    elif dispatcher == "share":
+        kw = dict(dispatcher="share", local=(4, 12))
+        El = 8
+    p = make_params(E, D, F, dtype, seed=3, std=0.05, El=El)
+    x = torch.randn(T, D, generator=torch.Generator().manual_seed(0)).to(dtype)
+    gout = torch.randn(T, D, generator=torch.Generator().manual_seed(1)).to(dtype)
+    beta, linear_beta = 2.0, 1.7
+    leaves = {k: getattr(p, k).clone().requires_grad_() for k in ("router_w_ED", "w1_EFD", "w3_EFD", "w2_EDF")}
+    xr = x.clone().requires_grad_()
+    okw = {}
+    if dispatcher == "padded":
+        okw["pad_multiple"] = 64
+    if dispatcher == "share":
+        okw["local_experts"] = (4, 12)
+    ref, aux = R.moe_forward(xr, R.MoEParams(**leaves), spec,
+                             activation=lambda g, u: R.situ_glu(g, u, beta, linear_beta), **okw)
+    ref.backward(gout)
+    block = build_block(p, spec, D, F, dtype, DEV, activation=moe.SituGLU(beta, linear_beta), **kw)
+    assert not block.routed_experts.inner_experts.fuses_activation()
+    xd = x.to(DEV).requires_grad_()
+    out = block(xd)
+    out.backward(gout.to(DEV))
+    _check_routing(block, x.to(DEV), aux, spec, label="situ " + dispatcher)
+    ie = block.routed_experts.inner_experts
+    got = {"out": out, "dx": xd.grad, "router_w_ED": block.router.gate.weight.grad,
+           "w1_EFD": ie.w1_EFD.grad, "w3_EFD": ie.w3_EFD.grad, "w2_EDF": ie.w2_EDF.grad}
+    want = {"out": ref, "dx": xr.grad, **{k: v.grad for k, v in leaves.items()}}
+    for k in want:
+        if dtype == torch.float32:
+            assert rel_max(got[k], want[k]) < 1e-5, f"{k}: {rel_max(got[k], want[k])}"
+        else:
+            assert rel_l2(got[k], want[k]) < 2e-2, f"{k}: rel-L2 {rel_l2(got[k], want[k])}"
+    # and the same block with SwiGLU gives something else (the activation is really used)
+    swi = build_block(p, spec, D, F, dtype, DEV, **kw)
+    assert rel_l2(swi(x.to(DEV)), ref) > 5e-2
 
 
 def test_deepseek_shape_local_share_with_shared_expert():

@@ -401,6 +401,113 @@ def test_grouped_experts_bf16_mfma(ops, counts, D, Fd):
     _experts_case(ops, torch.bfloat16, counts, D, Fd, std=0.05)
 
 
+# ---------------------------------------------------------------- one grouped linear map
+def _linear_case(ops, dtype, counts, I, O, seed=0, extra_rows=0):
+    """y[segment e] = x[segment e] . w[e]^T and both gradients, against per-segment fp32 matrix
+    products of the same inputs (experts.py:272-285's loop, written out here)."""
+    g = torch.Generator().manual_seed(seed)
+    El, Rn = len(counts), sum(counts) + extra_rows
+    x = torch.randn(Rn, I, generator=g).to(dtype)
+    w = (torch.randn(El, O, I, generator=g) * 0.1).to(dtype)
+    gy = torch.randn(Rn, O, generator=g).to(dtype)
+    covered = sum(counts)
+    xs, gs = x[:covered].float().split(counts), gy[:covered].float().split(counts)
+    want_y = torch.cat([xs[e] @ w[e].float().T for e in range(El)]) if covered else torch.zeros(0, O)
+    want_dx = torch.cat([gs[e] @ w[e].float() for e in range(El)]) if covered else torch.zeros(0, I)
+    want_dw = torch.stack([gs[e].T @ xs[e] for e in range(El)])
+    plan = ops.segments_from_counts(torch.tensor(counts, dtype=torch.int32, device=DEV), Rn)
+    xd, wd = x.to(DEV).requires_grad_(), w.to(DEV).requires_grad_()
+    junk = torch.full((Rn + 1, max(I, O)), float("nan"), device=DEV, dtype=dtype)  # poison the free blocks
+    del junk
+    y = ops.grouped_linear(xd, wd, plan, zero_fill=extra_rows > 0)
+    assert y.shape == (Rn, O) and y.dtype == dtype
+    y.backward(gy.to(DEV))
+    # one rounding of an fp32-accumulated sum in bf16; fp32 sums within 1e-5 of the largest value
+    tol, metric = (1e-5, rel_max) if dtype == torch.float32 else (5e-3, rel_l2)
+    for name, got, want in (("y", y[:covered], want_y), ("dx", xd.grad[:covered], want_dx), ("dw", wd.grad, want_dw)):
+        assert got.shape == want.shape, name
+        if want.numel() == 0 or want.abs().max() == 0:
+            assert got.numel() == 0 or got.abs().max() == 0, name
+        else:
+            assert metric(got, want) < tol, f"{name} {metric(got, want)}"
+    if extra_rows:
+        assert not y[covered:].any() and not xd.grad[covered:].any()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("counts,I,O", [((5, 6, 4, 7), 16, 32), ((2, 0, 3), 4, 8), ((0, 5, 0), 8, 4), ((0, 0, 0), 4, 8),
+                                        ((130, 1, 64, 300), 72, 40), ((100, 0, 29), 40, 72)])
+def test_grouped_linear_generic(ops, dtype, counts, I, O):
+    print(f"grouped linear generic {dtype} {counts} I={I} O={O}", flush=True)
+    _linear_case(ops, dtype, counts, I, O)
+
+
+@pytest.mark.parametrize("counts,I,O", [
+    ((200, 0, 129), 384, 768), ((131, 260), 768, 384), ((1000,), 384, 512), ((3,), 384, 384),
+    ((513, 77, 0, 256, 255, 257, 1), 512, 448), ((0, 0, 0), 384, 384),
+    # few row tiles: the input gradient runs on 128-column tiles
+    ((4096,), 448, 2048), ((700, 900), 2048, 384),
+    ((300, 0, 5, 700, 1, 64, 65, 0, 128, 129, 2, 5, 4, 250, 0, 90, 17, 33, 640), 640, 384),
+])
+def test_grouped_linear_bf16_mfma(ops, counts, I, O):
+    print(f"grouped linear bf16 mfma {counts} I={I} O={O}", flush=True)
+    _linear_case(ops, torch.bfloat16, counts, I, O)
+
+
+@pytest.mark.parametrize("dtype,I,O", [(torch.float32, 16, 24), (torch.bfloat16, 384, 448)])
+def test_grouped_linear_zero_fills_rows_the_counts_do_not_cover(ops, dtype, I, O):
+    print(f"grouped linear uncovered rows {dtype}", flush=True)
+    _linear_case(ops, dtype, (10, 0, 20), I, O, extra_rows=10)
+
+
+def test_grouped_linear_needs_only_the_gradients_asked_for(ops):
+    print("grouped linear partial gradients", flush=True)
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(50, 384, generator=g).bfloat16().to(DEV)
+    w = (torch.randn(2, 448, 384, generator=g) * 0.1).bfloat16().to(DEV)
+    plan = ops.segments_from_counts(torch.tensor([20, 30], dtype=torch.int32, device=DEV), 50)
+    gy = torch.randn(50, 448, generator=g).bfloat16().to(DEV)
+    full = ops.grouped_linear_bwd(gy, x, w, plan)
+    only_dx = ops.grouped_linear_bwd(gy, x, w, plan, need_dw=False)
+    only_dw = ops.grouped_linear_bwd(gy, x, w, plan, need_dx=False)
+    assert torch.equal(only_dx[0], full[0]) and only_dx[1] is None
+    assert torch.equal(only_dw[1], full[1]) and only_dw[0] is None
+    assert ops.grouped_linear(x, w, plan).requires_grad is False
+
+
+@pytest.mark.parametrize("dtype,counts,D,Fd", [(torch.float32, (5, 6, 4, 7), 16, 32), (torch.bfloat16, (200, 0, 129), 384, 768),
+                                               (torch.bfloat16, (100, 0, 29), 72, 40)])
+def test_grouped_experts_module_with_the_situ_activation(ops, dtype, counts, D, Fd):
+    """GroupedExperts(activation_fn=SituGLU(...)) called with counts, as the reference's
+    dispatchers call it (experts.py:152-209), against the oracle with the restated formula."""
+    from torchllmtuner_amd import moe
+
+    print(f"experts situ {dtype} {counts} D={D} F={Fd}", flush=True)
+    g = torch.Generator().manual_seed(9)
+    El, Rn = len(counts), sum(counts)
+    x = torch.randn(Rn, D, generator=g).to(dtype)
+    ws = [(torch.randn(El, Fd, D, generator=g) * 0.1).to(dtype), (torch.randn(El, Fd, D, generator=g) * 0.1).to(dtype),
+          (torch.randn(El, D, Fd, generator=g) * 0.1).to(dtype)]
+    gy = torch.randn(Rn, D, generator=g).to(dtype)
+    ref_in = [t.clone().requires_grad_() for t in (x, *ws)]
+    ref = R.grouped_experts(ref_in[0], torch.tensor(counts), *ref_in[1:], lambda a, b: R.situ_glu(a, b, 1.5, None))
+    ref.backward(gy)
+    experts = moe.GroupedExperts(D, Fd, El, activation_fn=moe.SituGLU(1.5)).to(DEV).to(dtype)
+    with torch.no_grad():
+        for prm, t in zip((experts.w1_EFD, experts.w3_EFD, experts.w2_EDF), ws):
+            prm.copy_(t)
+    xd = x.to(DEV).requires_grad_()
+    y = experts(xd, torch.tensor(counts, device=DEV))
+    y.backward(gy.to(DEV))
+    tol, metric = (FP32_TOL, rel_max) if dtype == torch.float32 else (BF16_TOL, rel_l2)
+    for name, got, want in (("y", y, ref), ("dx", xd.grad, ref_in[0].grad), ("dw1", experts.w1_EFD.grad, ref_in[1].grad),
+                            ("dw3", experts.w3_EFD.grad, ref_in[2].grad), ("dw2", experts.w2_EDF.grad, ref_in[3].grad)):
+        if want.abs().max() == 0:
+            assert got.abs().max() == 0, name
+        else:
+            assert metric(got, want) < tol, f"{name} {metric(got, want)}"
+
+
 # ---------------------------------------------------------------- balance loss
 @pytest.mark.parametrize("seed", [0, 1])
 def test_grouped_experts_bf16_mfma_random_segments(ops, seed):

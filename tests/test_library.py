@@ -28,7 +28,7 @@ def test_library_loads_and_exports_every_declared_symbol():
         assert hasattr(raw, name), f"{name} is declared in mi355_moe.h but not exported"
         assert name in _lib.SIGNATURES, f"{name} has no ctypes prototype"
     assert set(_lib.SIGNATURES) == set(names)
-    assert lib.mi355_moe_abi_version() == _lib.ABI_VERSION == 2
+    assert lib.mi355_moe_abi_version() == _lib.ABI_VERSION == 3
     assert lib.mi355_grouped_tile_m(1) == 256 and lib.mi355_grouped_tile_m(0) == 256
 
 

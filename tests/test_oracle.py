@@ -254,6 +254,54 @@ def test_bf16_rounding_points_are_per_op():
     torch.testing.assert_close(got.float(), want.float(), rtol=2e-2, atol=1e-3)
 
 
+@pytest.mark.parametrize("linear_beta", [None, 0.0, 1.7])
+def test_situ_glu_matches_the_reference_tests_explicit_formula(linear_beta):
+    # tests/unit_tests/cpu/models/test_situ_activation.py:31-45: bounded gate over (1 + e^-gate),
+    # times the (optionally bounded) up; values and both gradients
+    torch.manual_seed(5)
+    gate = torch.randn(2, 5, requires_grad=True)
+    up = torch.randn(2, 5, requires_grad=True)
+    got = R.situ_glu(gate, up, 2.0, linear_beta)
+    bounded_gate = 2 * torch.tanh(gate / 2)
+    bounded_up = up if not linear_beta else linear_beta * torch.tanh(up / linear_beta)
+    want = bounded_gate / (1 + (-gate).exp()) * bounded_up
+    torch.testing.assert_close(got, want)
+    for a, b_ in zip(torch.autograd.grad(got.sum(), (gate, up)), torch.autograd.grad(want.sum(), (gate, up))):
+        torch.testing.assert_close(a, b_)
+
+
+def test_situ_glu_bounds_small_argument_limit_and_dtype():
+    torch.manual_seed(6)
+    g, u = torch.randn(64, 8, dtype=torch.float64) * 6, torch.randn(64, 8, dtype=torch.float64) * 6
+    out = R.situ_glu(g.float(), u.float(), 1.5, 0.75)
+    # |beta tanh| <= beta, sigmoid <= 1, |linear_beta tanh| <= linear_beta (equal once fp32 saturates)
+    assert out.abs().max() <= 1.5 * 0.75
+    # the sign is the sign of gate * up (tanh is odd, sigmoid positive)
+    assert torch.equal(out.sign(), (g * u).sign().float())
+    # near zero: tanh(x/b) b -> x, sigmoid -> 1/2
+    eps = torch.full((4,), 1e-4, dtype=torch.float64)
+    torch.testing.assert_close(R.situ_glu(eps.float(), eps.float(), 2.0, 1.0).double(), eps * eps / 2, rtol=1e-3, atol=0)
+    # huge gate: beta * up exactly (both saturate), and a bf16 input comes back as bf16
+    big = R.situ_glu(torch.tensor([40.0]), torch.tensor([0.5]), 3.0, None)
+    assert big.item() == 1.5
+    assert R.situ_glu(torch.ones(2).bfloat16(), torch.ones(2).bfloat16()).dtype is torch.bfloat16
+
+
+def test_grouped_experts_with_a_callers_activation_uses_it_between_the_projections():
+    # experts.py:204-209: gate, up, activation(gate, up), down -- per segment by hand
+    torch.manual_seed(8)
+    w1, w3 = torch.randn(3, 12, 8) * 0.3, torch.randn(3, 12, 8) * 0.3
+    w2 = torch.randn(3, 8, 12) * 0.3
+    x = torch.randn(9, 8)
+    counts = (4, 0, 5)
+    act = lambda g, u: R.situ_glu(g, u, 2.0, 1.7)
+    want = torch.cat([act(sx @ w1[e].T, sx @ w3[e].T) @ w2[e].T for e, sx in enumerate(x.split(counts))])
+    got = R.grouped_experts(x, torch.tensor(counts), w1, w3, w2, act)
+    torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-6)
+    # and it is not SwiGLU
+    assert not torch.allclose(got, R.grouped_experts(x, torch.tensor(counts), w1, w3, w2), atol=1e-3)
+
+
 # ---- combine ----------------------------------------------------------------
 def test_combine_fp64_exact():
     # test_moe_token_dispatch.py:84-99

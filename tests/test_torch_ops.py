@@ -39,7 +39,8 @@ def test_every_operator_is_registered_with_a_fake_kernel_and_propagates_shapes()
         "quantile_observe", "quantile_estimate", "rms_norm_fwd", "rms_norm_bwd", "balance_loss_fwd",
         "balance_loss_bwd", "permute_plan", "segments_from_counts", "permute_rows_fwd", "permute_rows_bwd",
         "combine_fwd", "combine_bwd", "combine_row_scale", "combine_scores_bwd", "grouped_swiglu_fwd",
-        "grouped_swiglu_bwd", "gather_experts_combine_fwd", "gather_experts_combine_bwd",
+        "grouped_swiglu_bwd", "grouped_linear_fwd", "grouped_linear_bwd", "gather_experts_combine_fwd",
+        "gather_experts_combine_bwd",
     }
     tile_cap = N // ops.TILE_M + El + 1
     small = E + (El + 1) + 2 * El + 2 * tile_cap + 1
@@ -78,6 +79,8 @@ def test_every_operator_is_registered_with_a_fake_kernel_and_propagates_shapes()
                                    [((N, D), BF), ((N, F), BF), ((N, F), BF), ((N, F), BF)]),
             "grouped_swiglu_bwd": (O.grouped_swiglu_bwd(rows, rows, None, w1, w3, w2, rf, rf, rf, *seg, True, True, False),
                                    [((N, D), BF), ((El, F, D), BF), ((El, F, D), BF), ((El, D, F), BF)]),
+            "grouped_linear_fwd": (O.grouped_linear_fwd(rows, w1, *seg, False), [((N, F), BF)]),
+            "grouped_linear_bwd": (O.grouped_linear_bwd(rf, rows, w1, *seg, True, False, False), [((N, D), BF), ((0,), BF)]),
             "gather_experts_combine_fwd": (
                 O.gather_experts_combine_fwd(x, wts, w1, w3, w2, tok, sor, ros, *seg, K, N, True, True),
                 [((T, D), BF), ((N, F), BF), ((N, F), BF)]),
@@ -127,6 +130,54 @@ def test_block_calls_its_submodules_through_their_hooks():
             lambda m, a, out: seen.__setitem__("inner", _shapes(a) + _shapes(out)))
         block(x)
         assert seen["inner"] == [((N, D), BF), ((E,), I32), ((N, D), BF)]
+
+
+def test_situ_activation_matches_the_explicit_formula_and_validates_its_arguments():
+    """The formula and gradient check of tests/unit_tests/cpu/models/test_situ_activation.py:31-45
+    and the constructor errors of llmtuner/models/common/activation.py:47-54."""
+    for linear_beta in (None, 0.0, 1.7):
+        torch.manual_seed(0)
+        gate = torch.randn(2, 5, requires_grad=True)
+        up = torch.randn(2, 5, requires_grad=True)
+        actual = moe.SituGLU(2.0, linear_beta)(gate, up)
+        bounded_up = up if not linear_beta else linear_beta * torch.tanh(up / linear_beta)
+        expected = 2 * torch.tanh(gate / 2) / (1 + (-gate).exp()) * bounded_up
+        torch.testing.assert_close(actual, expected)
+        for a, b in zip(torch.autograd.grad(actual.sum(), (gate, up)), torch.autograd.grad(expected.sum(), (gate, up))):
+            torch.testing.assert_close(a, b)
+    assert moe.SituGLU()(torch.ones(3).bfloat16(), torch.ones(3).bfloat16()).dtype is BF
+    for bad in (0.0, -1.0, float("inf"), float("nan")):
+        with pytest.raises(ValueError, match="beta must be finite and positive"):
+            moe.SituGLU(bad)
+    for bad in (-0.5, float("inf")):
+        with pytest.raises(ValueError, match="linear_beta must be finite and nonnegative"):
+            moe.SituGLU(1.0, bad)
+    assert issubclass(moe.SituGLU, moe.ActivationFn) and issubclass(moe.SwiGLU, moe.ActivationFn)
+    with pytest.raises(TypeError):
+        moe.ActivationFn()  # abstract
+
+
+def test_a_block_with_another_activation_runs_three_grouped_linear_maps():
+    """Only SwiGLU itself is evaluated inside the gate/up kernel: SituGLU, a caller's own module and a
+    subclass of SwiGLU (which may compute anything) all run between grouped linear maps, with the
+    reference's shapes (experts.py:204-209)."""
+    class Mine(moe.SwiGLU):
+        def forward(self, gate, up):
+            calls.append((tuple(gate.shape), tuple(up.shape)))
+            return gate * up
+
+    calls = []
+    with FakeTensorMode(), torch.device("cuda"):
+        block = _fake_block()
+        ie = block.routed_experts.inner_experts
+        assert ie.fuses_activation()
+        x = torch.empty(T, D, dtype=BF)
+        for act in (moe.SituGLU(2.0, 1.0), Mine()):
+            ie.activation_fn = act
+            assert not ie.fuses_activation()
+            assert _shapes(block(x)) == [((T, D), BF)]
+            assert _shapes(ie(torch.empty(N, D, dtype=BF), torch.empty(E, dtype=I64))) == [((N, D), BF)]
+    assert calls == [((N, F), (N, F))] * 2
 
 
 def test_a_routed_experts_subclass_that_replaces_forward_is_honoured():

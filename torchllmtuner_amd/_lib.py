@@ -57,6 +57,8 @@ SIGNATURES = {
         I,
         [I, P, P, P, L, P, P, P, P, P, P, P, P, P, P, P, P, L, P, P, P, P, P, P, L, L, L, L, P],
     ),
+    "mi355_grouped_linear_fwd": (I, [P, P, I, P, P, P, P, P, L, P, L, L, L, L, P]),
+    "mi355_grouped_linear_bwd": (I, [P, P, P, I, P, P, P, P, P, L, P, P, L, L, L, L, P]),
     "mi355_grouped_combine_bwd_slots": (L, [I, L, L]),
     "mi355_grouped_swiglu_combine_bwd": (
         I,
@@ -70,7 +72,7 @@ SIGNATURES = {
     ),
 }
 
-ABI_VERSION = 2  # MI355_MOE_ABI_VERSION of include/mi355_moe.h
+ABI_VERSION = 3  # MI355_MOE_ABI_VERSION of include/mi355_moe.h
 
 _lib = None
 

@@ -21,6 +21,9 @@ int bf16_grouped_fwd(const void* rows, const int32_t* token_of_row, int64_t num_
                      int64_t tile_capacity, void* gate, void* up, void* h, void* y, int64_t D,
                      int64_t F, int stages, hipStream_t s);
 int bf16_fused_dot_slots(int64_t F);
+int bf16_grouped_linear_dx(const void* dy, const void* w, const int32_t* seg_offsets, const int32_t* seg_counts,
+                           const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* num_tiles,
+                           int64_t tile_capacity, void* dx, int64_t O, int64_t I, hipStream_t s);
 int bf16_grouped_bwd(const void* dy, const void* rows, const int32_t* token_of_row, int64_t num_tokens,
                      const void* w1, const void* w3, const void* w2, const void* gate, const void* up,
                      const void* h, const float* row_scale, float* dot_partial,
@@ -250,6 +253,57 @@ extern "C" int mi355_grouped_swiglu_stage(int stage, const void* dy, const void*
   return bf16_grouped_bwd(
       dy, rows, token_of_row, num_tokens, w1, w3, w2, gate, up, h, nullptr, nullptr, seg_offsets, seg_counts,
       tile_expert, tile_row0, num_tiles, tile_capacity, dgate, dup, drows, dw1, dw3, dw2, El, D, F, stage, s);
+}
+
+// ---- one grouped linear map: y[r] = x[r] . w[e(r)]^T (the reference's GroupedExperts._grouped_mm) ----
+extern "C" int mi355_grouped_linear_fwd(const void* x, const void* w, int dtype, const int32_t* seg_offsets,
+                                        const int32_t* seg_counts, const int32_t* tile_expert,
+                                        const int32_t* tile_row0, const int32_t* num_tiles, int64_t tile_capacity,
+                                        void* y, int64_t El, int64_t I, int64_t O, int64_t row_capacity,
+                                        void* stream) {
+  if (int rc = check_common("grouped_linear_fwd", dtype, El, O, I, row_capacity, tile_capacity)) return rc;
+  if (row_capacity == 0 || tile_capacity == 0) return MI355_OK;
+  MI355_REQUIRE(x && w && y && seg_offsets && seg_counts && tile_expert && tile_row0 && num_tiles,
+                "grouped_linear_fwd: null pointer");
+  hipStream_t s = as_stream(stream);
+  if (dtype == MI355_BF16 && bf16_fast_path_ok(O, I))
+    // the down projection's kernel is this product: rows (R, I) . w[e] (O, I)^T
+    return bf16_grouped_fwd(nullptr, nullptr, 0, nullptr, nullptr, w, seg_offsets, seg_counts, tile_expert, tile_row0,
+                            num_tiles, tile_capacity, nullptr, nullptr, const_cast<void*>(x), y, O, I, 2, s);
+  const Seg sg{seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles, tile_capacity};
+  // B(k=i, n=o) = w[e][o][i]
+  return rowseg(sg, x, I, w, 1, I, O * I, y, O, I, dtype, 0, s);
+}
+
+extern "C" int mi355_grouped_linear_bwd(const void* dy, const void* x, const void* w, int dtype,
+                                        const int32_t* seg_offsets, const int32_t* seg_counts,
+                                        const int32_t* tile_expert, const int32_t* tile_row0,
+                                        const int32_t* num_tiles, int64_t tile_capacity, void* dx, void* dw,
+                                        int64_t El, int64_t I, int64_t O, int64_t row_capacity, void* stream) {
+  if (int rc = check_common("grouped_linear_bwd", dtype, El, O, I, row_capacity, tile_capacity)) return rc;
+  MI355_REQUIRE(seg_offsets && seg_counts && num_tiles, "grouped_linear_bwd: null plan pointer");
+  const bool rows = row_capacity > 0 && tile_capacity > 0;
+  MI355_REQUIRE(!rows || (dy && x && w && tile_expert && tile_row0), "grouped_linear_bwd: null pointer");
+  hipStream_t s = as_stream(stream);
+  const Seg sg{seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles, tile_capacity};
+  if (dtype == MI355_BF16 && bf16_fast_path_ok(O, I) && rows) {
+    if (dx)
+      if (int rc = bf16_grouped_linear_dx(dy, w, seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles,
+                                          tile_capacity, dx, O, I, s))
+        return rc;
+    // dw[e] (O, I) = dy[segment]^T . x[segment]: the dW2 product of the SwiGLU backward
+    if (dw)
+      return bf16_grouped_bwd(dy, nullptr, nullptr, 0, nullptr, nullptr, nullptr, nullptr, nullptr, x, nullptr, nullptr,
+                              seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles, tile_capacity, nullptr,
+                              nullptr, nullptr, nullptr, nullptr, dw, El, O, I, 16, s);
+    return MI355_OK;
+  }
+  // dx = dy . w[e]: B(k=o, n=i) = w[e][o][i]
+  if (dx && rows)
+    if (int rc = rowseg(sg, dy, O, w, I, 1, O * I, dx, I, O, dtype, 0, s)) return rc;
+  // the weight gradient also covers the no-rows case: every expert's gradient is written (zeros)
+  if (dw) return kseg(sg, dy, x, dw, O, I, El, dtype, s);
+  return MI355_OK;
 }
 
 extern "C" int64_t mi355_grouped_combine_bwd_slots(int dtype, int64_t D, int64_t F) {

@@ -77,7 +77,9 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base) {
 // int32 data that no kernel of this file writes (the plan's arrays), for uniform lookups
 typedef const int32_t __attribute__((address_space(4))) * const_i32;
 
-enum RowMode { RM_GATEUP = 0, RM_DOWN = 1, RM_DH = 2, RM_DX = 3 };
+// RM_DLIN: the product of RM_DH (rows . w[e], the weight's contraction axis strided) with a plain epilogue:
+// the input gradient of one grouped linear map
+enum RowMode { RM_GATEUP = 0, RM_DOWN = 1, RM_DH = 2, RM_DX = 3, RM_DLIN = 4 };
 
 struct RowArgs {
   const uint16_t* a0;  // GATEUP rows | DOWN h | DH dy | DX dgate
@@ -133,7 +135,8 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
   constexpr int NA = TBM / 64;             // 16-byte A chunks staged per thread and K step
   constexpr int NB = BNT / 64;             // the same for B
   constexpr int STAGE = (TBM + BNT) * BK;  // elements per LDS stage
-  constexpr bool B_KS = (MODE == RM_DH || MODE == RM_DX);
+  constexpr bool DH_LIKE = (MODE == RM_DH || MODE == RM_DLIN);  // same operands, different epilogue
+  constexpr bool B_KS = (DH_LIKE || MODE == RM_DX);
   static_assert(!GATHER || MODE == RM_GATEUP || MODE == RM_DH, "only gate/up and dH gather their rows");
   static_assert(!(GATHER && MODE == RM_DH) || NJ == 4, "the fused dH epilogue reduces over 16 lanes per row");
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
@@ -142,9 +145,9 @@ __global__ __launch_bounds__(NT, 2) void row_tiled_kernel(RowArgs p) {
   const int wm = (wave / WN) * 64, wn = wave % WN;
   const int wave_m = __builtin_amdgcn_readfirstlane(wm);  // the same value, known to be wave-uniform
   const int D = p.D, F = p.F;
-  const int Kdim = (MODE == RM_GATEUP || MODE == RM_DH) ? D : (MODE == RM_DOWN ? F : 2 * F);
-  const int lda = (MODE == RM_GATEUP || MODE == RM_DH) ? D : F;
-  const int Ncols = (MODE == RM_GATEUP || MODE == RM_DH) ? F : D;  // output width
+  const int Kdim = (MODE == RM_GATEUP || DH_LIKE) ? D : (MODE == RM_DOWN ? F : 2 * F);
+  const int lda = (MODE == RM_GATEUP || DH_LIKE) ? D : F;
+  const int Ncols = (MODE == RM_GATEUP || DH_LIKE) ? F : D;  // output width
   const int64_t wsz = static_cast<int64_t>(D) * F;
   const int ksteps = Kdim / BK;
 
@@ -970,7 +973,7 @@ static int launch_row(RowArgs& a, int64_t width, int64_t tile_capacity, hipStrea
   // tiles instead: twice the work items, each with the whole contraction.  Only where the
   // epilogue does not depend on the tile width (the folded dH writes one partial per 128
   // columns of a 256-column tile).
-  if constexpr (MODE == RM_DH && !GATHER) {
+  if constexpr ((MODE == RM_DH || MODE == RM_DLIN) && !GATHER) {
     if (tile_capacity * a.n_tiles * 4 <= resident_blocks() * 3 && width >= 128) {  // (the capacity is an upper bound)
       a.n_tiles = (int)((width + 127) / 128);
       static PerDeviceOnce narrow_configured;
@@ -1023,6 +1026,17 @@ int bf16_grouped_fwd(const void* rows, const int32_t* token_of_row, int64_t num_
     if (int rc = launch_row<RM_DOWN>(b, D, tile_capacity, s, "grouped down")) return rc;
   }
   return MI355_OK;
+}
+
+// dx = dy . w[e] over the listed segments: dy (rows, O), w (El, O, I), dx (rows, I)
+int bf16_grouped_linear_dx(const void* dy, const void* w, const int32_t* seg_offsets, const int32_t* seg_counts,
+                           const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* num_tiles,
+                           int64_t tile_capacity, void* dx, int64_t O, int64_t I, hipStream_t s) {
+  RowArgs a{};
+  a.seg_offsets = seg_offsets; a.seg_counts = seg_counts; a.tile_expert = tile_expert;
+  a.tile_row0 = tile_row0; a.num_tiles = num_tiles; a.D = (int)O; a.F = (int)I;
+  a.a0 = (const uint16_t*)dy; a.b0 = (const uint16_t*)w; a.o0 = (uint16_t*)dx;
+  return launch_row<RM_DLIN>(a, I, tile_capacity, s, "grouped linear dx");
 }
 
 int bf16_fused_dot_slots(int64_t F) {

@@ -439,6 +439,44 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> grouped_swiglu_bwd(
   return {drows, dw1, dw3, dw2};
 }
 
+// y[r] = x[r] . w[e(r)]^T over the plan's segments (GroupedExperts._grouped_mm of the reference)
+Tensor grouped_linear_fwd(const Tensor& x_, const Tensor& w_, const Tensor& seg_offsets, const Tensor& seg_counts,
+                          const Tensor& tile_expert, const Tensor& tile_row0, const Tensor& num_tiles,
+                          bool zero_fill) {
+  Launch L(x_);
+  const Tensor x = x_.contiguous(), w = w_.contiguous();
+  TORCH_CHECK_VALUE(x.dim() == 2 && w.dim() == 3 && w.size(2) == x.size(1), "grouped weight ", w.sizes(),
+                    " does not match rows ", x.sizes());
+  TORCH_CHECK_TYPE(w.scalar_type() == x.scalar_type(), "grouped weight and rows must share one dtype");
+  const int64_t R = x.size(0), I = x.size(1), El = w.size(0), O = w.size(1);
+  const Plan p = plan_of(seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles);
+  Tensor y = zero_fill ? at::zeros({R, O}, x.options()) : at::empty({R, O}, x.options());
+  check(mi355_grouped_linear_fwd(ptr(x), ptr(w), dtype_code(x), p.seg_offsets, p.seg_counts, p.tile_expert,
+                                 p.tile_row0, p.num_tiles, p.tile_capacity, ptr(y), El, I, O, R, L.stream),
+        "grouped_linear_fwd");
+  return y;
+}
+
+std::tuple<Tensor, Tensor> grouped_linear_bwd(const Tensor& dy_, const Tensor& x_, const Tensor& w_,
+                                              const Tensor& seg_offsets, const Tensor& seg_counts,
+                                              const Tensor& tile_expert, const Tensor& tile_row0,
+                                              const Tensor& num_tiles, bool need_dx, bool need_dw, bool zero_fill) {
+  Launch L(x_);
+  const Tensor x = x_.contiguous(), w = w_.contiguous();
+  const Tensor dy = (dy_.scalar_type() == x.scalar_type() ? dy_ : dy_.to(x.scalar_type())).contiguous();
+  const int64_t R = x.size(0), I = x.size(1), El = w.size(0), O = w.size(1);
+  TORCH_CHECK_VALUE(dy.dim() == 2 && dy.size(0) == R && dy.size(1) == O, "grouped_linear_bwd: gradient ", dy.sizes(),
+                    " does not match (", R, ", ", O, ")");
+  const Plan p = plan_of(seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles);
+  Tensor dx = !need_dx ? none_like(x) : (zero_fill ? at::zeros({R, I}, x.options()) : at::empty({R, I}, x.options()));
+  Tensor dw = need_dw ? at::empty_like(w) : none_like(w);
+  check(mi355_grouped_linear_bwd(ptr(dy), ptr(x), ptr(w), dtype_code(x), p.seg_offsets, p.seg_counts, p.tile_expert,
+                                 p.tile_row0, p.num_tiles, p.tile_capacity, need_dx ? ptr(dx) : nullptr,
+                                 need_dw ? ptr(dw) : nullptr, El, I, O, R, L.stream),
+        "grouped_linear_bwd");
+  return {dx, dw};
+}
+
 // out[t] = sum_k weights[t,k] * experts(x)[row(t,k)]: gathered expert product, then the combine.
 // Returns (out, gate, up); y and h are dropped (the fused backward recomputes h).  save_gate_up = false
 // (nobody will differentiate): gate and up are not written at all and come back empty.
@@ -570,6 +608,12 @@ TORCH_LIBRARY(mi355_moe, m) {
       "Tensor tile_row0, Tensor num_tiles, bool need_drows, bool need_dw, bool zero_fill) -> "
       "(Tensor, Tensor, Tensor, Tensor)");
   m.def(
+      "grouped_linear_fwd(Tensor x, Tensor w, Tensor seg_offsets, Tensor seg_counts, Tensor tile_expert, "
+      "Tensor tile_row0, Tensor num_tiles, bool zero_fill) -> Tensor");
+  m.def(
+      "grouped_linear_bwd(Tensor dy, Tensor x, Tensor w, Tensor seg_offsets, Tensor seg_counts, Tensor tile_expert, "
+      "Tensor tile_row0, Tensor num_tiles, bool need_dx, bool need_dw, bool zero_fill) -> (Tensor, Tensor)");
+  m.def(
       "gather_experts_combine_fwd(Tensor x, Tensor weights, Tensor w1, Tensor w3, Tensor w2, Tensor token_of_row, "
       "Tensor slot_of_row, Tensor row_of_slot, Tensor seg_offsets, Tensor seg_counts, Tensor tile_expert, Tensor tile_row0, "
       "Tensor num_tiles, int top_k, int row_capacity, bool round_terms, bool save_gate_up) -> (Tensor, Tensor, Tensor)");
@@ -602,6 +646,8 @@ TORCH_LIBRARY_IMPL(mi355_moe, CUDA, m) {
   m.impl("combine_scores_bwd", combine_scores_bwd);
   m.impl("grouped_swiglu_fwd", grouped_swiglu_fwd);
   m.impl("grouped_swiglu_bwd", grouped_swiglu_bwd);
+  m.impl("grouped_linear_fwd", grouped_linear_fwd);
+  m.impl("grouped_linear_bwd", grouped_linear_bwd);
   m.impl("gather_experts_combine_fwd", gather_experts_combine_fwd);
   m.impl("gather_experts_combine_bwd", gather_experts_combine_bwd);
 }

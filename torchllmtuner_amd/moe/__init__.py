@@ -1,6 +1,6 @@
 """The native MoE block (router, dispatchers, grouped experts) on MI355X kernels."""
 
-from .activation import SwiGLU
+from .activation import ActivationFn, SituGLU, SwiGLU
 from .auxiliary_loss import AuxLoss, MicrobatchWiseLoadBalanceLoss
 from .bias_update import (
     collect_moe_layers,
@@ -44,6 +44,8 @@ __all__ = [
     "QuantileBalancer",
     "RoutedExperts",
     "RouterGateLinear",
+    "ActivationFn",
+    "SituGLU",
     "SwiGLU",
     "TokenChoiceTopKRouter",
     "collect_moe_layers",

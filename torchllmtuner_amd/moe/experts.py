@@ -1,4 +1,4 @@
-"""Expert weights and the routed-expert module, on the grouped SwiGLU kernels.
+"""Expert weights and the routed-expert module, on the grouped expert kernels.
 
 Constructor surface, parameter names and validation of
 llmtuner/models/common/moe/experts.py:73-343 (``GroupedExperts``,
@@ -75,10 +75,6 @@ class GroupedExperts(nn.Module):
                 raise ValueError(f"{name} must be positive integer, got {value!r}")
         if use_grouped_mm is not None and not isinstance(use_grouped_mm, bool):
             raise TypeError("use_grouped_mm must be bool or None")
-        if activation_fn is not None and not isinstance(activation_fn, SwiGLU):
-            raise NotImplementedError(
-                "the grouped expert kernels fuse SwiGLU; other activations are not implemented"
-            )
         self.num_experts = num_experts
         self.hidden_dim = hidden_dim
         self.dim = dim
@@ -125,9 +121,30 @@ class GroupedExperts(nn.Module):
         plan = ops.segments_from_counts(num_tokens_per_expert_E, x_RD.shape[0])
         return self.compute_planned(x_RD, plan, zero_fill=True)
 
+    def _grouped_mm(self, x_RI, weight_EOI, plan: ops.PermutePlan, zero_fill: bool = False):
+        """``x . weight[e]^T`` per expert segment (experts.py:211-216).  The reference passes the
+        cumulative offsets; here the segments travel as the plan they were counted into."""
+        return Fn.grouped_linear(x_RI, weight_EOI, plan, zero_fill=zero_fill)
+
+    def fuses_activation(self) -> bool:
+        """SwiGLU exactly (not a subclass that may compute something else) is evaluated inside
+        the gate/up kernel; any other gated activation, and any subclass that brings its own
+        ``_grouped_mm``, runs as three grouped linear maps with the activation between them."""
+        if type(self)._grouped_mm is not GroupedExperts._grouped_mm:
+            return False  # a subclass's own grouped product must be the one that runs
+        cls = type(self.activation_fn)
+        # (the reference's own class, llmtuner.models.common.activation.SwiGLU, is the same function)
+        return cls is SwiGLU or (cls.__name__ == "SwiGLU" and cls.__module__.endswith("models.common.activation"))
+
     def compute_planned(self, x_RD, plan: ops.PermutePlan, zero_fill: bool = False):
         w1, w3, w2 = self._weights_as(x_RD.dtype)
-        return Fn.grouped_swiglu(x_RD, w1, w3, w2, plan, zero_fill=zero_fill)
+        if self.fuses_activation():
+            return Fn.grouped_swiglu(x_RD, w1, w3, w2, plan, zero_fill=zero_fill)
+        # experts.py:204-209 with the caller's activation: gate, up, activation(gate, up), down
+        gate = self._grouped_mm(x_RD, w1, plan, zero_fill=zero_fill)
+        up = self._grouped_mm(x_RD, w3, plan, zero_fill=zero_fill)
+        h = self.activation_fn(gate, up)
+        return self._grouped_mm(h, w2, plan, zero_fill=zero_fill).type_as(x_RD)
 
 
 class RoutedExperts(nn.Module):
@@ -164,6 +181,7 @@ class RoutedExperts(nn.Module):
         round_terms = not dispatcher.accumulate_in_fp32
         fused = (
             _is_plain_grouped_experts(experts)  # hooks on, or a subclass of, the inner module must run
+            and experts.fuses_activation()
             and ops.gather_supported(x_TD, experts.hidden_dim)
             and x_TD.is_contiguous()
             and ops.combine_bwd_slots(x_TD.dtype, x_TD.shape[-1], experts.hidden_dim) > 0

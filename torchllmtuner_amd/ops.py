@@ -213,6 +213,16 @@ def _(dy, rows, token_of_row, w1, w3, w2, gate, up, h, seg_offsets, seg_counts, 
     return drows, g(w1), g(w3), g(w2)
 
 
+@_fake("grouped_linear_fwd")
+def _(x, w, seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles, zero_fill):
+    return x.new_empty((x.shape[0], w.shape[1]))
+
+
+@_fake("grouped_linear_bwd")
+def _(dy, x, w, seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles, need_dx, need_dw, zero_fill):
+    return (torch.empty_like(x) if need_dx else _e0(x)), (torch.empty_like(w) if need_dw else _e0(w))
+
+
 @_fake("gather_experts_combine_fwd")
 def _(x, weights, w1, w3, w2, token_of_row, slot_of_row, row_of_slot, seg_offsets, seg_counts, tile_expert,
       tile_row0, num_tiles, top_k, row_capacity, round_terms, save_gate_up):
@@ -426,6 +436,26 @@ def _gs_backward(ctx, dy, _dgate, _dup, _dh):
 
 
 _autograd("grouped_swiglu_fwd", _gs_backward, _gs_setup)
+
+
+# -- one grouped linear map (the reference's GroupedExperts._grouped_mm)
+def _gl_setup(ctx, inputs, output):
+    x, w, so, sc, te, tr, nt, zero_fill = inputs
+    ctx.save_for_backward(x, w, so, sc, te, tr, nt)
+    ctx.zero_fill = zero_fill
+    ctx.set_materialize_grads(False)
+
+
+def _gl_backward(ctx, dy):
+    x, w, so, sc, te, tr, nt = ctx.saved_tensors
+    need = ctx.needs_input_grad
+    if dy is None or not (need[0] or need[1]):
+        return (None,) * 8
+    dx, dw = _O.grouped_linear_bwd(dy, x, w, so, sc, te, tr, nt, need[0], need[1], ctx.zero_fill)
+    return ((dx if need[0] else None), (dw if need[1] else None)) + (None,) * 6
+
+
+_autograd("grouped_linear_fwd", _gl_backward, _gl_setup)
 
 
 # -- gathered experts + combine: one backward for both halves
@@ -732,6 +762,32 @@ def grouped_swiglu_bwd(dy_RD, rows_RD, w1_EFD, w3_EFD, w2_EDF, gate, up, h, plan
     drows, dw1, dw3, dw2 = _O.grouped_swiglu_bwd(dy_RD, rows_RD, tok, w1_EFD, w3_EFD, w2_EDF, gate, up, h,
                                                  *plan.segments(), bool(need_drows), bool(need_dw), bool(zero_fill))
     return _opt(drows, need_drows), _opt(dw1, need_dw), _opt(dw3, need_dw), _opt(dw2, need_dw)
+
+
+def grouped_linear(x_RI, w_EOI, plan: PermutePlan, zero_fill=False):
+    """y[r] = x[r] . w[e(r)]^T over the plan's expert segments -- the reference's pluggable
+    ``GroupedExperts._grouped_mm(x_TD, weight_EOI, offsets_E)``
+    (llmtuner/models/common/moe/experts.py:211-216).  Differentiable in the rows and the weight;
+    bf16 with both widths multiples of 64 (>= 384) runs the MFMA kernels, anything else the
+    strided fp32-MFMA GEMM.  ``zero_fill``: rows the plan does not cover come back as zeros."""
+    _dev(x_RI, w_EOI)
+    _dt(x_RI)
+    if x_RI.ndim != 2 or w_EOI.ndim != 3 or w_EOI.shape[2] != x_RI.shape[1]:
+        raise ValueError(f"grouped weight {tuple(w_EOI.shape)} does not match rows {tuple(x_RI.shape)}")
+    if w_EOI.dtype != x_RI.dtype:
+        raise TypeError("grouped weight and rows must share one dtype")
+    if w_EOI.shape[0] != plan.num_local_experts:
+        raise ValueError(f"plan covers {plan.num_local_experts} experts, weights hold {w_EOI.shape[0]}")
+    return _O.grouped_linear_fwd(x_RI, w_EOI, *plan.segments(), bool(zero_fill))
+
+
+def grouped_linear_bwd(dy_RO, x_RI, w_EOI, plan: PermutePlan, need_dx=True, need_dw=True, zero_fill=False):
+    """Both gradients of ``grouped_linear``: dx[r] = dy[r] . w[e(r)] and dw[e] = dy[segment e]^T .
+    x[segment e] (zeros for an expert without rows).  A gradient that is not asked for is not
+    computed and comes back as None."""
+    _dev(dy_RO, x_RI, w_EOI)
+    dx, dw = _O.grouped_linear_bwd(dy_RO, x_RI, w_EOI, *plan.segments(), bool(need_dx), bool(need_dw), bool(zero_fill))
+    return _opt(dx, need_dx), _opt(dw, need_dw)
 
 
 def combine_bwd_slots(dtype, D, F):
