@@ -27,9 +27,17 @@ extern "C" {
 
 #define MI355_MOE_ABI_VERSION 3
 
-/* element types of activation / weight buffers */
+/* element types of activation / weight buffers.
+ * MI355_F64 is accepted where the reference's fp64 runs pass through this boundary
+ * (tests/unit_tests/cpu/test_expert_compile_segments.py:13-40 runs the experts in fp64):
+ * the row movers, the combine, the grouped experts and grouped linear maps compute in fp64
+ * throughout; the router gate takes fp64 tokens and weights and converts them to fp32 on
+ * the way in, as RouterGateLinearFunction does (linear.py:123-125), and writes its
+ * gradients back in the operands' types.  Every other entry point takes fp32 or bf16
+ * and returns MI355_EINVAL for fp64. */
 #define MI355_F32 0
 #define MI355_BF16 1
+#define MI355_F64 2
 
 /* score functions: llmtuner/models/common/moe/routing.py:270-277 */
 #define MI355_SCORE_SIGMOID 0
@@ -287,7 +295,7 @@ int mi355_permute_rows_fwd(const void* x, int dtype, const int32_t* row_of_slot,
 
 /*
  * dx[t] = sum_k drows[row_of_slot[t*K+k]] (slots with row -1 contribute nothing),
- * summed in fp32 in ascending k, written in `dtype`.  This is the backward of the
+ * summed in fp32 (fp64 rows: in fp64) in ascending k, written in `dtype`.  This is the backward of the
  * row gather (autograd's index_put accumulate for token_dispatch.py:199; the
  * duplicate-row contract is tests/unit_tests/cpu/kernel/test_kernel_contracts.py:
  * 114-127).
@@ -455,7 +463,7 @@ int mi355_grouped_swiglu_stage(int stage, const void* dy, const void* rows,
  * (llmtuner/models/common/moe/experts.py:211-216, :256-285):
  *   y[r] = x[r] . w[e(r)]^T      x (rows, I), w (El, O, I) row-major, y (rows, O)
  * over the segments of a plan / of mi355_segments_from_counts, fp32 accumulation, one rounding
- * to `dtype` (fp32 or bf16; x, w and y share it).  It is what GroupedExperts is built from when
+ * to `dtype` (fp32, bf16 or fp64; x, w and y share it).  It is what GroupedExperts is built from when
  * its gated activation is not SwiGLU (llmtuner/models/common/activation.py:40-64, SituGLU):
  * gate = linear(x, w1), up = linear(x, w3), h = activation(gate, up), y = linear(h, w2).
  * bf16 with I and O multiples of 64 (>= 384) runs the MFMA kernels of the SwiGLU path (the down

@@ -650,7 +650,7 @@ def test_gathered_experts_combine_autograd_matches_the_explicit_backward(ops):
 
 
 @pytest.mark.parametrize("counts", [(2, 0, 3), (0, 5, 0), (0, 0, 0)])
-@pytest.mark.parametrize("dtype,D,Fd", [(torch.float32, 4, 8), (torch.bfloat16, 384, 384)])
+@pytest.mark.parametrize("dtype,D,Fd", [(torch.float32, 4, 8), (torch.float64, 4, 8), (torch.bfloat16, 384, 384)])
 def test_grouped_experts_under_torch_compile(counts, dtype, D, Fd):
     """GroupedExperts traced whole (aot_eager, fullgraph) equals eager, forward and gradients, for
     the zero-count segment cases of tests/unit_tests/cpu/test_expert_compile_segments.py:13-40:

@@ -92,7 +92,10 @@ def test_ops_refuse_cpu_tensors():
     with pytest.raises(RuntimeError, match="no CPU implementation"):
         ops.router_gate_fwd(torch.zeros(2, 4), torch.zeros(3, 4))
     with pytest.raises(TypeError, match="float32 and bfloat16"):
-        ops._dt(torch.zeros(1, dtype=torch.float64))
+        ops._dt(torch.zeros(1, dtype=torch.float16))
+    assert ops._dt(torch.zeros(1, dtype=torch.float64)) == 2  # MI355_F64
+    with pytest.raises(TypeError, match="float32 and bfloat16, got torch.float64"):
+        ops._dt(torch.zeros(1, dtype=torch.float64), fp64=False)  # kernels without an fp64 form (rms_norm)
 
 
 def test_module_surface_matches_the_reference_block():

@@ -250,6 +250,78 @@ __global__ __launch_bounds__(256) void combine_bwd_kernel(
   if (lane < K && dweights) dweights[s0 + lane] = my_dot;
 }
 
+// ---- fp64 rows: every product and sum in fp64 (the scores stay fp32 and are widened), one wave
+// per token, lanes along D; the terms are added in ascending row order like the kernels above
+__global__ __launch_bounds__(256) void combine_fwd_f64_kernel(
+    const double* __restrict__ y, const float* __restrict__ weights, const int32_t* __restrict__ row_of_slot,
+    double* __restrict__ out, int T_, int D, int K) {
+  const int lane = threadIdx.x & 63;
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= T_) return;
+  const int64_t s0 = static_cast<int64_t>(t) * K;
+  const int row = lane < K ? row_of_slot[s0 + lane] : -1;
+  const float w = lane < K ? weights[s0 + lane] : 0.0f;
+  int pos = 0;
+  for (int j = 0; j < K; ++j) {
+    const int rj = __shfl(row, j, kWave);
+    pos += (rj >= 0 && (rj < row || (rj == row && j < lane))) ? 1 : 0;
+  }
+  const int nvalid = __popcll(__ballot(row >= 0));
+  const int to = (row >= 0 ? pos : 63) << 2;
+  int o_row = __builtin_amdgcn_ds_permute(to, row);
+  float o_w = __int_as_float(__builtin_amdgcn_ds_permute(to, __float_as_int(w)));
+  if (lane >= nvalid) { o_row = -1; o_w = 0.0f; }
+  double* dst = out + static_cast<int64_t>(t) * D;
+  for (int base = 0; base < D; base += kWave) {  // uniform trip count: the shuffles need every lane
+    const int i = base + lane;
+    double a = 0.0;
+    for (int p = 0; p < nvalid; ++p) {
+      const int r = __shfl(o_row, p, kWave);
+      const double ww = static_cast<double>(__shfl(o_w, p, kWave));
+      if (i < D) a += y[static_cast<int64_t>(r) * D + i] * ww;
+    }
+    if (i < D) dst[i] = a;
+  }
+}
+
+__global__ __launch_bounds__(256) void combine_bwd_f64_kernel(
+    const double* __restrict__ dout, const double* __restrict__ y, const float* __restrict__ weights,
+    const int32_t* __restrict__ row_of_slot, const int32_t* __restrict__ slot_of_row,
+    const int32_t* __restrict__ total_rows, double* __restrict__ dy, float* __restrict__ dweights, int T_, int D,
+    int K, int token_blocks, int row_capacity) {
+  const int lane = threadIdx.x & 63;
+  if (static_cast<int>(blockIdx.x) >= token_blocks) {
+    const int r = (blockIdx.x - token_blocks) * 4 + (threadIdx.x >> 6);
+    if (r >= row_capacity || r >= *total_rows || slot_of_row[r] >= 0) return;
+    double* dst = dy + static_cast<int64_t>(r) * D;
+    for (int i = lane; i < D; i += kWave) dst[i] = 0.0;
+    return;
+  }
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= T_) return;
+  const int64_t s0 = static_cast<int64_t>(t) * K;
+  const double* g = dout + static_cast<int64_t>(t) * D;
+  for (int k = 0; k < K; ++k) {
+    const int r = row_of_slot[s0 + k];  // wave-uniform
+    if (r < 0) {
+      if (lane == 0 && dweights) dweights[s0 + k] = 0.0f;
+      continue;
+    }
+    const double ww = static_cast<double>(weights[s0 + k]);
+    const double* yr = y + static_cast<int64_t>(r) * D;
+    double* dr = dy + static_cast<int64_t>(r) * D;
+    double dot = 0.0;
+    for (int i = lane; i < D; i += kWave) {
+      const double gv = g[i];
+      dot += yr[i] * gv;
+      dr[i] = gv * ww;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) dot += __shfl_xor(dot, o, kWave);
+    if (lane == 0 && dweights) dweights[s0 + k] = static_cast<float>(dot);
+  }
+}
+
 }  // namespace
 }  // namespace mi355
 
@@ -273,6 +345,9 @@ extern "C" int mi355_combine_fwd(const void* y, int dtype, const float* weights,
   } else if (dtype == MI355_BF16) {
     if (K <= 8) launch(combine_fwd_kernel<uint16_t, true>, static_cast<const uint16_t*>(y), static_cast<uint16_t*>(out));
     else launch(combine_fwd_kernel<uint16_t, false>, static_cast<const uint16_t*>(y), static_cast<uint16_t*>(out));
+  } else if (dtype == MI355_F64) {
+    hipLaunchKernelGGL(combine_fwd_f64_kernel, grid, dim3(256), 0, as_stream(stream), static_cast<const double*>(y),
+                       weights, row_of_slot, static_cast<double*>(out), (int)T, (int)D, (int)K);
   } else
     return fail(MI355_EINVAL, "combine_fwd: unknown dtype %d", dtype);
   return check_launch("combine_fwd");
@@ -304,6 +379,11 @@ extern "C" int mi355_combine_bwd(const void* dout, const void* y, int dtype, con
                        static_cast<const uint16_t*>(dout), static_cast<const uint16_t*>(y), weights,
                        row_of_slot, slot_of_row, total_rows, static_cast<uint16_t*>(dy), dweights,
                        (int)T, (int)D, (int)K, token_blocks, (int)row_capacity, stream_stores);
+  else if (dtype == MI355_F64)
+    hipLaunchKernelGGL(combine_bwd_f64_kernel, grid, dim3(256), 0, as_stream(stream),
+                       static_cast<const double*>(dout), static_cast<const double*>(y), weights, row_of_slot,
+                       slot_of_row, total_rows, static_cast<double*>(dy), dweights, (int)T, (int)D, (int)K,
+                       token_blocks, (int)row_capacity);
   else
     return fail(MI355_EINVAL, "combine_bwd: unknown dtype %d", dtype);
   return check_launch("combine_bwd");

@@ -97,6 +97,9 @@ template <>
 __device__ __forceinline__ float load_as_f32<float>(const float* p) { return *p; }
 template <>
 __device__ __forceinline__ float load_as_f32<uint16_t>(const uint16_t* p) { return bf16_to_f32(*p); }
+// fp64 storage read by a kernel that computes in fp32 (the router: `.float()` of its operands)
+template <>
+__device__ __forceinline__ float load_as_f32<double>(const double* p) { return static_cast<float>(*p); }
 
 template <typename T>
 __device__ __forceinline__ void store_from_f32(T* p, float v);
@@ -104,6 +107,8 @@ template <>
 __device__ __forceinline__ void store_from_f32<float>(float* p, float v) { *p = v; }
 template <>
 __device__ __forceinline__ void store_from_f32<uint16_t>(uint16_t* p, float v) { *p = f32_to_bf16(v); }
+template <>
+__device__ __forceinline__ void store_from_f32<double>(double* p, float v) { *p = static_cast<double>(v); }
 
 // ---- wave reductions ---------------------------------------------------------
 __device__ __forceinline__ float wave_sum(float v) {

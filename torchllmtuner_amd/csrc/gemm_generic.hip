@@ -6,22 +6,48 @@
 // per-lane operand of the MFMA (one A(m,k), one B(k,n)) is a conflict-free
 // ds_read_b32 whatever the global layout was.  Global loads pick the lane mapping
 // that walks the operand's contiguous axis.
+//
+// fp64 storage: an fp64 operand or result next to fp32 ones is converted on the way in and
+// out (the router, which computes in fp32 whatever it is given).  With A, B and C all fp64
+// (fp64 experts) the same kernel computes in fp64: each wave's 32x32 quadrant is then 2 x 2
+// tiles of v_mfma_f64_16x16x4_f64.
 #include "gemm_generic.h"
 
 #include <cstdint>
+#include <type_traits>
 
 namespace mi355 {
 
 namespace {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef double f64x4 __attribute__((ext_vector_type(4)));
+
+// the arithmetic type of a product: fp64 only when everything is fp64
+template <typename TA, typename TB, typename TC>
+struct ComputeOf { using type = float; };
+template <>
+struct ComputeOf<double, double, double> { using type = double; };
+
+template <typename CT, typename T>
+__device__ __forceinline__ CT load_op(const T* p) {
+  if constexpr (std::is_same_v<CT, double>) return *p;  // (T is double here)
+  else return load_as_f32(p);
+}
+template <typename CT, typename T>
+__device__ __forceinline__ void store_op(T* p, CT v) {
+  if constexpr (std::is_same_v<CT, double>) *p = v;
+  else store_from_f32(p, v);
+}
 
 constexpr int TM = 64, TN = 64, TK = 16, PITCH = 65;
 
 template <typename TA, typename TB, typename TC>
 __global__ __launch_bounds__(256) void ggemm_kernel(GemmArgs g) {
-  __shared__ float As[TK][PITCH];
-  __shared__ float Bs[TK][PITCH];
+  using CT = typename ComputeOf<TA, TB, TC>::type;
+  constexpr bool F64 = std::is_same_v<CT, double>;
+  __shared__ CT As[TK][PITCH];
+  __shared__ CT Bs[TK][PITCH];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -83,24 +109,31 @@ __global__ __launch_bounds__(256) void ggemm_kernel(GemmArgs g) {
     if (b_nc) { bn[j] = i % TN; bk[j] = i / TN; } else { bk[j] = i % TK; bn[j] = i / TK; }
   }
 
-  float ra[4], rb[4];
+  CT ra[4], rb[4];
   auto load_slab = [&](int k0) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int k = k0 + ak[j];
       ra[j] = (am[j] < m_valid && k < k_end)
-                  ? load_as_f32(A + (a_row0 + am[j]) * g.a_rs + static_cast<int64_t>(k) * g.a_cs)
-                  : 0.0f;
+                  ? load_op<CT>(A + (a_row0 + am[j]) * g.a_rs + static_cast<int64_t>(k) * g.a_cs)
+                  : CT(0);
       const int kb = k0 + bk[j];
       rb[j] = (bn[j] < n_valid && kb < k_end)
-                  ? load_as_f32(B + static_cast<int64_t>(kb) * g.b_rs + static_cast<int64_t>(n0 + bn[j]) * g.b_cs)
-                  : 0.0f;
+                  ? load_op<CT>(B + static_cast<int64_t>(kb) * g.b_rs + static_cast<int64_t>(n0 + bn[j]) * g.b_cs)
+                  : CT(0);
     }
   };
 
-  f32x16 acc;
+  f32x16 acc;       // fp32: one 32x32 tile
+  f64x4 acc64[2][2];  // fp64: 2 x 2 tiles of 16x16
 #pragma unroll
   for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc64[i][j][v] = 0.0;
 
   if (k_begin < k_end) load_slab(k_begin);
   for (int k0 = k_begin; k0 < k_end; k0 += TK) {
@@ -111,13 +144,52 @@ __global__ __launch_bounds__(256) void ggemm_kernel(GemmArgs g) {
     }
     __syncthreads();
     if (k0 + TK < k_end) load_slab(k0 + TK);
+    if constexpr (F64) {
+      // lane l supplies A(m = l % 16, k = l / 16) and B(k = l / 16, n = l % 16) of a 16x16x4 step
 #pragma unroll
-    for (int kk = 0; kk < TK; kk += 2) {
-      const float a = As[kk + (lane >> 5)][wm + (lane & 31)];
-      const float b = Bs[kk + (lane >> 5)][wn + (lane & 31)];
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc, 0, 0, 0);
+      for (int kk = 0; kk < TK; kk += 4) {
+        double a[2], b[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          a[i] = As[kk + (lane >> 4)][wm + 16 * i + (lane & 15)];
+          b[i] = Bs[kk + (lane >> 4)][wn + 16 * i + (lane & 15)];
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+            acc64[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[i], b[j], acc64[i][j], 0, 0, 0);
+      }
+    } else {
+#pragma unroll
+      for (int kk = 0; kk < TK; kk += 2) {
+        const float a = As[kk + (lane >> 5)][wm + (lane & 31)];
+        const float b = Bs[kk + (lane >> 5)][wn + (lane & 31)];
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc, 0, 0, 0);
+      }
     }
     __syncthreads();
+  }
+
+  if constexpr (F64) {
+    // register v of tile (i, j) holds row 16 i + 4 v + l / 16, column 16 j + l % 16 (probed on the card)
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int n = wn + 16 * j + (lane & 15);
+        if (n >= n_valid) continue;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const int m = wm + 16 * i + 4 * v + (lane >> 4);
+          if (m >= m_valid) continue;
+          const int64_t off = (a_row0 + m) * g.ldc + n0 + n;
+          double r = acc64[i][j][v];
+          if (g.accumulate) r += load_op<CT>(C + off);
+          store_op<CT>(C + off, r);
+        }
+      }
+    return;
   }
 
   const int n = wn + (lane & 31);
@@ -253,9 +325,18 @@ template <typename TA, typename TB>
 int launch_c(const GemmArgs& a, int c_dtype, dim3 grid, hipStream_t s) {
   if (c_dtype == MI355_F32 || a.ksplit > 1)
     hipLaunchKernelGGL((ggemm_kernel<TA, TB, float>), grid, dim3(256), 0, s, a);
+  else if (c_dtype == MI355_F64)
+    hipLaunchKernelGGL((ggemm_kernel<TA, TB, double>), grid, dim3(256), 0, s, a);
   else
     hipLaunchKernelGGL((ggemm_kernel<TA, TB, uint16_t>), grid, dim3(256), 0, s, a);
   return check_launch("ggemm");
+}
+
+template <typename TA>
+int launch_b(const GemmArgs& a, int b_dtype, int c_dtype, dim3 grid, hipStream_t s) {
+  if (b_dtype == MI355_F32) return launch_c<TA, float>(a, c_dtype, grid, s);
+  if (b_dtype == MI355_BF16) return launch_c<TA, uint16_t>(a, c_dtype, grid, s);
+  return launch_c<TA, double>(a, c_dtype, grid, s);
 }
 
 }  // namespace
@@ -283,6 +364,7 @@ int launch_vec_layout(const GemmArgs& a, int av, int bv, int c_dtype, dim3 grid,
 // 4-element aligned along a unit-stride axis.
 bool vec_layout(const GemmArgs& a, int a_dtype, int b_dtype, int* av, int* bv) {
   if (a.mode != GEMM_DENSE || a.accumulate) return false;
+  if (a_dtype == MI355_F64 || b_dtype == MI355_F64) return false;
   const int64_t asz = a_dtype == MI355_F32 ? 4 : 2, bsz = b_dtype == MI355_F32 ? 4 : 2;
   if (reinterpret_cast<uintptr_t>(a.A) % (4 * asz) || reinterpret_cast<uintptr_t>(a.B) % (4 * bsz)) return false;
   if (a.K % 4) return false;
@@ -305,17 +387,20 @@ int launch_gemm(const GemmArgs& a, int a_dtype, int b_dtype, int c_dtype, dim3 g
                 hipStream_t s) {
   if (grid.x == 0 || grid.y == 0 || grid.z == 0) return MI355_OK;
   int av = 0, bv = 0;
-  if (vec_layout(a, a_dtype, b_dtype, &av, &bv)) {
+  if (c_dtype != MI355_F64 && vec_layout(a, a_dtype, b_dtype, &av, &bv)) {
     if (a_dtype == MI355_F32 && b_dtype == MI355_F32) return launch_vec_layout<float, float>(a, av, bv, c_dtype, grid, s);
     if (a_dtype == MI355_BF16 && b_dtype == MI355_F32) return launch_vec_layout<uint16_t, float>(a, av, bv, c_dtype, grid, s);
     if (a_dtype == MI355_F32 && b_dtype == MI355_BF16) return launch_vec_layout<float, uint16_t>(a, av, bv, c_dtype, grid, s);
     if (a_dtype == MI355_BF16 && b_dtype == MI355_BF16) return launch_vec_layout<uint16_t, uint16_t>(a, av, bv, c_dtype, grid, s);
   }
-  if (a_dtype == MI355_F32 && b_dtype == MI355_F32) return launch_c<float, float>(a, c_dtype, grid, s);
-  if (a_dtype == MI355_BF16 && b_dtype == MI355_F32) return launch_c<uint16_t, float>(a, c_dtype, grid, s);
-  if (a_dtype == MI355_F32 && b_dtype == MI355_BF16) return launch_c<float, uint16_t>(a, c_dtype, grid, s);
-  if (a_dtype == MI355_BF16 && b_dtype == MI355_BF16) return launch_c<uint16_t, uint16_t>(a, c_dtype, grid, s);
-  return fail(MI355_EINVAL, "gemm: unknown dtype %d/%d", a_dtype, b_dtype);
+  auto known = [](int d) { return d == MI355_F32 || d == MI355_BF16 || d == MI355_F64; };
+  if (!known(a_dtype) || !known(b_dtype) || !known(c_dtype))
+    return fail(MI355_EINVAL, "gemm: unknown dtype %d/%d/%d", a_dtype, b_dtype, c_dtype);
+  if (a.ksplit > 1 && a_dtype == MI355_F64 && b_dtype == MI355_F64 && c_dtype == MI355_F64)
+    return fail(MI355_EUNSUP, "gemm: fp64 products are not split along K");
+  if (a_dtype == MI355_F32) return launch_b<float>(a, b_dtype, c_dtype, grid, s);
+  if (a_dtype == MI355_BF16) return launch_b<uint16_t>(a, b_dtype, c_dtype, grid, s);
+  return launch_b<double>(a, b_dtype, c_dtype, grid, s);
 }
 
 dim3 gemm_grid_dense(int M, int N, int ksplit) {
@@ -335,6 +420,9 @@ int launch_splitk_reduce(const float* partial, void* out, int out_dtype, int64_t
   if (out_dtype == MI355_F32)
     hipLaunchKernelGGL(splitk_reduce_kernel<float>, dim3(blocks), dim3(256), 0, s, partial,
                        static_cast<float*>(out), MN, ksplit);
+  else if (out_dtype == MI355_F64)
+    hipLaunchKernelGGL(splitk_reduce_kernel<double>, dim3(blocks), dim3(256), 0, s, partial,
+                       static_cast<double*>(out), MN, ksplit);
   else
     hipLaunchKernelGGL(splitk_reduce_kernel<uint16_t>, dim3(blocks), dim3(256), 0, s, partial,
                        static_cast<uint16_t*>(out), MN, ksplit);

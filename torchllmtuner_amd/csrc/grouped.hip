@@ -1,7 +1,7 @@
 // Grouped SwiGLU experts: C entry points and the generic (any dtype, any shape)
 // path.  bf16 problems whose D and F are multiples of 64 go to the MFMA kernels of
-// grouped_bf16.hip; everything else (fp32, odd shapes) runs the strided fp32-MFMA
-// GEMM plus two small elementwise kernels.
+// grouped_bf16.hip; everything else (fp32, fp64, odd shapes) runs the strided GEMM of
+// gemm_generic.hip (fp32 MFMA; fp64 MFMA for fp64) plus two small elementwise kernels.
 #include <cstdlib>
 
 #include "common.h"
@@ -75,6 +75,30 @@ __global__ void swiglu_bwd_kernel(const T* __restrict__ gate, const T* __restric
   }
 }
 
+// the same two in fp64, for fp64 experts (every step of the reference's fp64 path is fp64)
+__global__ void swiglu_fwd_f64_kernel(const double* __restrict__ gate, const double* __restrict__ up,
+                                      double* __restrict__ h, const int32_t* __restrict__ total_rows, int F) {
+  const int64_t n = static_cast<int64_t>(*total_rows) * F;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const double g = gate[i];
+    h[i] = g / (1.0 + exp(-g)) * up[i];
+  }
+}
+
+__global__ void swiglu_bwd_f64_kernel(const double* __restrict__ gate, const double* __restrict__ up,
+                                      double* __restrict__ dgate, double* __restrict__ dup,
+                                      const int32_t* __restrict__ total_rows, int F) {
+  const int64_t n = static_cast<int64_t>(*total_rows) * F;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const double dh = dgate[i], g = gate[i], u = up[i];
+    const double sig = 1.0 / (1.0 + exp(-g));
+    dup[i] = dh * (g * sig);
+    dgate[i] = dh * u * (sig * (1.0 + g * (1.0 - sig)));
+  }
+}
+
 struct Seg {
   const int32_t *seg_offsets, *seg_counts, *tile_expert, *tile_row0, *num_tiles;
   int64_t tile_capacity;
@@ -107,7 +131,7 @@ int kseg(const Seg& sg, const void* A, const void* B, void* C, int64_t M, int64_
 
 int check_common(const char* who, int dtype, int64_t El, int64_t D, int64_t F, int64_t row_capacity,
                  int64_t tile_capacity) {
-  MI355_REQUIRE(dtype == MI355_F32 || dtype == MI355_BF16, "%s: unknown dtype %d", who, dtype);
+  MI355_REQUIRE(dtype == MI355_F32 || dtype == MI355_BF16 || dtype == MI355_F64, "%s: unknown dtype %d", who, dtype);
   MI355_REQUIRE(El >= 1 && D >= 1 && F >= 1, "%s: bad shape El=%lld D=%lld F=%lld", who, (long long)El,
                 (long long)D, (long long)F);
   MI355_REQUIRE(D < (1ll << 24) && F < (1ll << 24) && D * F < (1ll << 31), "%s: D*F exceeds int32", who);
@@ -173,6 +197,9 @@ extern "C" int mi355_grouped_swiglu_fwd(const void* rows, const int32_t* token_o
   if (dtype == MI355_F32)
     hipLaunchKernelGGL(swiglu_fwd_kernel<float>, dim3(blocks), dim3(256), 0, s, (const float*)gate,
                        (const float*)up, (float*)h, seg_offsets + El, (int)F);
+  else if (dtype == MI355_F64)
+    hipLaunchKernelGGL(swiglu_fwd_f64_kernel, dim3(blocks), dim3(256), 0, s, (const double*)gate,
+                       (const double*)up, (double*)h, seg_offsets + El, (int)F);
   else
     hipLaunchKernelGGL(swiglu_fwd_kernel<uint16_t>, dim3(blocks), dim3(256), 0, s,
                        (const uint16_t*)gate, (const uint16_t*)up, (uint16_t*)h, seg_offsets + El, (int)F);
@@ -215,6 +242,9 @@ extern "C" int mi355_grouped_swiglu_bwd(const void* dy, const void* rows,
     if (dtype == MI355_F32)
       hipLaunchKernelGGL(swiglu_bwd_kernel<float>, dim3(blocks), dim3(256), 0, s, (const float*)gate,
                          (const float*)up, (float*)dgate, (float*)dup, seg_offsets + El, (int)F);
+    else if (dtype == MI355_F64)
+      hipLaunchKernelGGL(swiglu_bwd_f64_kernel, dim3(blocks), dim3(256), 0, s, (const double*)gate,
+                         (const double*)up, (double*)dgate, (double*)dup, seg_offsets + El, (int)F);
     else
       hipLaunchKernelGGL(swiglu_bwd_kernel<uint16_t>, dim3(blocks), dim3(256), 0, s,
                          (const uint16_t*)gate, (const uint16_t*)up, (uint16_t*)dgate, (uint16_t*)dup,

@@ -453,6 +453,25 @@ __global__ __launch_bounds__(256) void permute_rows_bwd_kernel(
   }
 }
 
+// fp64 rows: the K-way sum in fp64, ascending k, one wave per token
+__global__ __launch_bounds__(256) void permute_rows_bwd_f64_kernel(
+    const double* __restrict__ drows, const int32_t* __restrict__ row_of_slot, double* __restrict__ dx,
+    int T_, int D, int K) {
+  const int lane = threadIdx.x & 63;
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= T_) return;
+  const int64_t s0 = static_cast<int64_t>(t) * K;
+  double* dst = dx + static_cast<int64_t>(t) * D;
+  for (int i = lane; i < D; i += kWave) {
+    double a = 0.0;
+    for (int k = 0; k < K; ++k) {
+      const int row = row_of_slot[s0 + k];  // wave-uniform
+      if (row >= 0) a += drows[static_cast<int64_t>(row) * D + i];
+    }
+    dst[i] = a;
+  }
+}
+
 }  // namespace
 }  // namespace mi355
 
@@ -584,6 +603,12 @@ extern "C" int mi355_permute_rows_fwd(const void* x, int dtype, const int32_t* r
                     row_capacity < (1ll << 31) && D < (1ll << 31),
                 "permute_rows_fwd: bad shape");
   if (row_capacity == 0) return MI355_OK;
+  if (dtype == MI355_F64) {
+    // a copy moves bytes: an fp64 row is an fp32 row of twice the length
+    MI355_REQUIRE(D < (1ll << 30), "permute_rows_fwd: bad shape");
+    dtype = MI355_F32;
+    D *= 2;
+  }
   MI355_REQUIRE(rows && (T == 0 || (x && row_of_slot)), "permute_rows_fwd: null pointer");
   MI355_REQUIRE(!slot_of_row || total_rows, "permute_rows_fwd: total_rows required with slot_of_row");
   const int token_blocks = (int)((T + 3) / 4);
@@ -623,6 +648,10 @@ extern "C" int mi355_permute_rows_bwd(const void* drows, int dtype, const int32_
     hipLaunchKernelGGL(permute_rows_bwd_kernel<uint16_t>, grid, dim3(256), 0, as_stream(stream),
                        static_cast<const uint16_t*>(drows), row_of_slot,
                        static_cast<uint16_t*>(dx), (int)T, (int)D, (int)K);
+  else if (dtype == MI355_F64)
+    hipLaunchKernelGGL(permute_rows_bwd_f64_kernel, grid, dim3(256), 0, as_stream(stream),
+                       static_cast<const double*>(drows), row_of_slot, static_cast<double*>(dx), (int)T, (int)D,
+                       (int)K);
   else
     return fail(MI355_EINVAL, "permute_rows_bwd: unknown dtype %d", dtype);
   return check_launch("permute_rows_bwd");

@@ -32,7 +32,8 @@ using OptTensor = std::optional<Tensor>;
 int dtype_code(const Tensor& t) {
   if (t.scalar_type() == at::kFloat) return MI355_F32;
   if (t.scalar_type() == at::kBFloat16) return MI355_BF16;
-  TORCH_CHECK_TYPE(false, "MI355 MoE kernels support float32 and bfloat16, got ", t.scalar_type());
+  if (t.scalar_type() == at::kDouble) return MI355_F64;
+  TORCH_CHECK_TYPE(false, "MI355 MoE kernels support float32, bfloat16 and float64, got ", t.scalar_type());
 }
 
 void* ptr(const Tensor& t) { return (t.defined() && t.numel() > 0) ? t.data_ptr() : nullptr; }

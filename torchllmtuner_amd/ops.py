@@ -24,18 +24,21 @@ from . import _lib
 _lib.load_torch_ops()  # fails loudly when the library is not built
 _O = torch.ops.mi355_moe
 
-_DT = {torch.float32: 0, torch.bfloat16: 1}
+_DT = {torch.float32: 0, torch.bfloat16: 1, torch.float64: 2}
 SCORE_FUNCS = {"sigmoid": 0, "softmax": 1, "sqrtsoftplus": 2}
 SELECT_TOPK, SELECT_FIXED, SELECT_BALANCED = 0, 1, 2
 # most rows an entry of a plan's tile list covers: the library's row-tile height
 TILE_M = int(_lib.load().mi355_grouped_tile_m(_DT[torch.bfloat16]))
 
 
-def _dt(t: torch.Tensor) -> int:
-    try:
-        return _DT[t.dtype]
-    except KeyError:
-        raise TypeError(f"MI355 MoE kernels support float32 and bfloat16, got {t.dtype}") from None
+def _dt(t: torch.Tensor, fp64: bool = True) -> int:
+    """The library's code for the tensor's dtype.  fp64 passes through the router gate (converted
+    to fp32 on the way in, as the reference does), the row movers, the combine and the grouped
+    experts (fp64 arithmetic throughout); ``fp64=False`` is for the kernels that have no fp64 form."""
+    code = _DT.get(t.dtype)
+    if code is None or (code == 2 and not fp64):
+        raise TypeError(f"MI355 MoE kernels support float32 and bfloat16{' (and float64)' if fp64 else ''}, got {t.dtype}")
+    return code
 
 
 def _dev(*tensors: torch.Tensor | None) -> torch.device:
@@ -565,7 +568,7 @@ def rms_norm_fwd(x, weight, epsilon):
     _dev(x, weight)
     if x.dtype != weight.dtype:
         raise TypeError(f"rms_norm: input ({x.dtype}) and weight ({weight.dtype}) must share a dtype")
-    _dt(x)
+    _dt(x, fp64=False)
     return _O.rms_norm_fwd(x, weight, float(epsilon))
 
 
