@@ -649,6 +649,42 @@ def test_gathered_experts_combine_autograd_matches_the_explicit_backward(ops):
     assert torch.equal(x2.grad, dx)
 
 
+def test_fused_backward_forks_and_joins_on_the_callers_stream(ops):
+    """The fused backward runs its weight gradients on a second stream and joins before it
+    returns: on a caller's own stream, several times in a row, with the gradients consumed by the
+    very next launch, every gradient equals the first run's bit for bit (a missing join would let
+    the consumer read weight gradients that are still being written)."""
+    print("gather_experts_combine on a caller's stream", flush=True)
+    T, K, E, D, Fd = 2048, 4, 8, 512, 768
+    g = torch.Generator().manual_seed(11)
+    ids = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(T)]).to(DEV)
+    wts = torch.rand(T, K, generator=g).to(DEV)
+    x = torch.randn(T, D, generator=g).bfloat16().to(DEV)
+    dout = torch.randn(T, D, generator=g).bfloat16().to(DEV)
+    mk = lambda *s: (torch.randn(*s, generator=g) * 0.05).bfloat16().to(DEV)
+    w1, w3, w2 = mk(E, Fd, D), mk(E, Fd, D), mk(E, D, Fd)
+    plan = ops.permute_plan(ids, E)
+
+    def grads():
+        leaves = [t.detach().clone().requires_grad_() for t in (x, wts, w1, w3, w2)]
+        ops.gather_experts_combine(*leaves, plan).backward(dout)
+        # consumed at once, on the same stream
+        return [t.grad.clone() for t in leaves], torch.stack([t.grad.float().sum() for t in leaves])
+
+    first, first_sums = grads()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for it in range(5):
+            again, sums = grads()
+            for a, b in zip(again, first):
+                assert torch.equal(a, b), f"iteration {it}"
+            assert torch.equal(sums, first_sums), f"iteration {it}"
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+
+
 @pytest.mark.parametrize("counts", [(2, 0, 3), (0, 5, 0), (0, 0, 0)])
 @pytest.mark.parametrize("dtype,D,Fd", [(torch.float32, 4, 8), (torch.float64, 4, 8), (torch.bfloat16, 384, 384)])
 def test_grouped_experts_under_torch_compile(counts, dtype, D, Fd):

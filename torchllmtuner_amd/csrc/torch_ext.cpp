@@ -19,12 +19,56 @@
 #include <c10/core/DeviceGuard.h>
 #include <torch/library.h>
 
+#include <hip/hip_runtime_api.h>
+
+#include <mutex>
 #include <optional>
 #include <tuple>
 
 #include "../../include/mi355_moe.h"
 
 namespace {
+
+// A second stream per device (default priority, not synchronising with the null stream) and the
+// two events of a fork / join around it.  The backward's weight gradients do not depend on its
+// input gradient: launched there, their workgroups fill the CUs that the last, partly filled
+// round of the other product's tiles leaves idle, and the bandwidth-bound row sum runs beside
+// matrix work instead of between two launches.  Created on first use; never under stream
+// capture (a caller who captures first runs a step uncaptured, as for every lazily built state);
+// nullptr means "stay on one stream".
+struct SideStream {
+  hipStream_t stream = nullptr;
+  hipEvent_t fork = nullptr, join = nullptr;
+  std::mutex order;  // an event is recorded and waited for as one step: host threads share the pair
+
+  // `to` waits for everything enqueued on `from` so far
+  bool chain(hipEvent_t event, hipStream_t from, hipStream_t to) {
+    std::lock_guard<std::mutex> lock(order);
+    return hipEventRecord(event, from) == hipSuccess && hipStreamWaitEvent(to, event, 0) == hipSuccess;
+  }
+};
+
+SideStream* side_stream(int device, hipStream_t current) {
+  static std::mutex mu;
+  static SideStream per_device[64];
+  static bool tried[64];
+  if (device < 0 || device >= 64) return nullptr;
+  std::lock_guard<std::mutex> lock(mu);
+  SideStream& s = per_device[device];
+  if (!tried[device]) {
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(current, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone)
+      return nullptr;  // not now: try again on a later, uncaptured call
+    tried[device] = true;
+    if (hipStreamCreateWithFlags(&s.stream, hipStreamNonBlocking) != hipSuccess ||
+        hipEventCreateWithFlags(&s.fork, hipEventDisableTiming) != hipSuccess ||
+        hipEventCreateWithFlags(&s.join, hipEventDisableTiming) != hipSuccess) {
+      (void)hipGetLastError();
+      s.stream = nullptr;
+    }
+  }
+  return s.stream ? &s : nullptr;
+}
 
 using at::Tensor;
 using OptTensor = std::optional<Tensor>;
@@ -534,29 +578,48 @@ std::tuple<Tensor, Tensor, Tensor, Tensor, Tensor> gather_experts_combine_bwd(
   Tensor dw1 = need_dw ? at::empty_like(w1) : none_like(w1);
   Tensor dw3 = need_dw ? at::empty_like(w3) : none_like(w3);
   Tensor dw2 = need_dw ? at::empty_like(w2) : none_like(w2);
-  auto run = [&](int stages) {
+  auto run = [&](int stages, void* stream) {
     check(mi355_grouped_swiglu_combine_bwd(
               ptr(dout), ptr(x), iptr(token_of_row), T, fptr(row_scale), ptr(w1), ptr(w3), ptr(w2), ptr(gate),
               ptr(up), dtype_code(x), p.seg_offsets, p.seg_counts, p.tile_expert, p.tile_row0, p.num_tiles,
               p.tile_capacity, ptr(dgate), ptr(dup), ptr(hs), static_cast<float*>(ptr(partial)),
               need_dx ? ptr(drows) : nullptr, need_dw ? ptr(dw1) : nullptr, need_dw ? ptr(dw3) : nullptr,
-              need_dw ? ptr(dw2) : nullptr, El, D, F, R, stages, L.stream),
+              need_dw ? ptr(dw2) : nullptr, El, D, F, R, stages, stream),
           "grouped_swiglu_combine_bwd");
   };
   Tensor dx = need_dx ? at::empty({T, D}, x.options()) : none_like(x);
   Tensor dweights = at::empty({T, K}, w.options());
-  if (R > 0) {
-    run(MI355_STAGE_DH | (need_dx ? MI355_STAGE_DX : 0));
+  auto sums = [&]() {
+    if (need_dx)
+      check(mi355_permute_rows_bwd(ptr(drows), dtype_code(x), iptr(row_of_slot), ptr(dx), T, D, K, L.stream),
+            "permute_rows_bwd");
+    check(mi355_combine_scores_bwd(fptr(partial), slots, iptr(row_of_slot), static_cast<float*>(ptr(dweights)), T, K,
+                                   R, L.stream),
+          "combine_scores_bwd");
+  };
+  const hipStream_t main = static_cast<hipStream_t>(L.stream);
+  SideStream* side = (R > 0 && need_dw && need_dx) ? side_stream(x.device().index(), main) : nullptr;
+  if (R == 0) {
+    run(0, L.stream);  // no rows: only the zero weight gradients remain to be written
+    sums();
+  } else if (!side) {
+    run(MI355_STAGE_DH | (need_dx ? MI355_STAGE_DX : 0), L.stream);
+    sums();
+    if (need_dw) run(MI355_STAGE_DW2 | MI355_STAGE_DW1 | MI355_STAGE_DW3, L.stream);
   } else {
-    run(0);  // no rows: only the zero weight gradients remain to be written
+    // Everything after dH reads what dH wrote and nothing else of this call: the weight gradients
+    // go to the side stream; the input gradient, its row sum and the score gradient stay here;
+    // this stream waits for the other before the operator returns, so that whatever the caller
+    // enqueues next, and the allocator's reuse of these buffers, is ordered behind both.
+    run(MI355_STAGE_DH, L.stream);
+    TORCH_CHECK(side->chain(side->fork, main, side->stream),
+                "gather_experts_combine_bwd: cannot fork to the side stream: ", hipGetErrorString(hipGetLastError()));
+    run(MI355_STAGE_DW2 | MI355_STAGE_DW1 | MI355_STAGE_DW3, side->stream);
+    run(MI355_STAGE_DX, L.stream);
+    sums();
+    TORCH_CHECK(side->chain(side->join, side->stream, main),
+                "gather_experts_combine_bwd: cannot join the side stream: ", hipGetErrorString(hipGetLastError()));
   }
-  if (need_dx)
-    check(mi355_permute_rows_bwd(ptr(drows), dtype_code(x), iptr(row_of_slot), ptr(dx), T, D, K, L.stream),
-          "permute_rows_bwd");
-  check(mi355_combine_scores_bwd(fptr(partial), slots, iptr(row_of_slot), static_cast<float*>(ptr(dweights)), T, K, R,
-                                 L.stream),
-        "combine_scores_bwd");
-  if (R > 0 && need_dw) run(MI355_STAGE_DW2 | MI355_STAGE_DW1 | MI355_STAGE_DW3);
   return {dx, dw1, dw3, dw2, dweights};
 }
 
