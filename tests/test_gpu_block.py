@@ -285,18 +285,21 @@ def test_forward_without_gradients_skips_gate_and_up_and_returns_the_same_bits()
     assert torch.isfinite(xin.grad.float()).all() and float(xin.grad.float().abs().sum()) > 0
 
 
-@pytest.mark.parametrize("dtype,D,F,dispatcher", [(torch.float32, 256, 512, "local"), (torch.bfloat16, 512, 384, "local"),
-                                                   (torch.bfloat16, 384, 512, "padded")])
-def test_block_step_replays_from_a_hip_graph(dtype, D, F, dispatcher):
+@pytest.mark.parametrize("dtype,D,F,dispatcher,shared_F", [
+    (torch.float32, 256, 512, "local", None), (torch.bfloat16, 512, 384, "local", None),
+    (torch.bfloat16, 384, 512, "padded", None),
+    # with a shared expert: it runs on the library's second stream, a fork and join inside the graph
+    (torch.bfloat16, 512, 384, "local", 448), (torch.float32, 128, 192, "local", 64)])
+def test_block_step_replays_from_a_hip_graph(dtype, D, F, dispatcher, shared_F):
     """Forward + backward of the block captured once as a HIP graph: no kernel of the path
     synchronises the host, reads a size back or allocates outside PyTorch's allocator, so the
     whole step captures as it is.  Every replay -- with eager steps and synchronisations between
     them, and with new token values in the captured input buffer -- must reproduce the eager
     step's output and gradients bit for bit (the kernels use no atomics)."""
-    print(f"block under a HIP graph {dtype} D={D} F={F} {dispatcher}", flush=True)
+    print(f"block under a HIP graph {dtype} D={D} F={F} {dispatcher} shared={shared_F}", flush=True)
     T, E, K = 600, 16, 4
     spec = R.RouterSpec(E, K, score_func="softmax", route_norm=True)
-    p = make_params(E, D, F, dtype, seed=31)
+    p = make_params(E, D, F, dtype, seed=31, shared_F=shared_F)
     kw = dict(pad_multiple=64) if dispatcher == "padded" else {}
     block = build_block(p, spec, D, F, dtype, DEV, dispatcher=dispatcher, **kw)
     block.train()
@@ -327,6 +330,53 @@ def test_block_step_replays_from_a_hip_graph(dtype, D, F, dispatcher):
         torch.cuda.synchronize()
         for got, want in zip(captured, eager):
             assert torch.equal(got, want), f"replay {rep} differs from the eager step"
+
+
+def test_shared_expert_on_the_second_stream_gives_the_one_stream_results():
+    """A block with a shared expert, run with the shared expert on the library's second stream and
+    with everything on the caller's stream: the same output and parameter gradients bit for bit
+    (the input gradient sums its three parts in another order: one bf16 rounding), several steps in
+    a row, also on a caller's own stream, with the results consumed at once."""
+    print("block shared expert on a second stream", flush=True)
+    T, D, E, K, F, Fs = 1500, 512, 16, 4, 384, 640
+    spec = R.RouterSpec(E, K, score_func="sigmoid", route_norm=True)
+    p = make_params(E, D, F, torch.bfloat16, seed=5, std=0.05, shared_F=Fs)
+    block = build_block(p, spec, D, F, torch.bfloat16, DEV)
+    block.train()
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn(T, D, generator=g).bfloat16().to(DEV)
+    gout = torch.randn(T, D, generator=g).bfloat16().to(DEV)
+    params = [q for q in block.parameters() if q.requires_grad]
+
+    def step():
+        xin = x.detach().clone().requires_grad_()
+        out = block(xin)
+        grads = torch.autograd.grad(out, [xin] + params, gout)
+        # (detached: a graph kept alive would keep the parameters' gradient accumulators of this
+        # step, with this step's stream, for the next one)
+        return [out.detach()] + [t.clone() for t in grads]
+
+    block.overlap_shared_experts = False
+    want = step()
+    torch.cuda.synchronize()
+    block.overlap_shared_experts = True
+    from torchllmtuner_amd import ops
+    assert ops.aux_stream(x.device) is not None
+    mine = torch.cuda.Stream()
+    for stream in (torch.cuda.current_stream(), mine):
+        stream.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(stream):
+            for it in range(4):
+                got = step()
+                assert torch.equal(got[0], want[0]), f"out, step {it}"
+                assert rel_l2(got[1], want[1]) < 4e-3, f"dx, step {it}"
+                for a, b in zip(got[2:], want[2:]):
+                    assert torch.equal(a, b), f"parameter gradient, step {it}"
+        torch.cuda.current_stream().wait_stream(stream)
+    torch.cuda.synchronize()
+    # without gradients too
+    with torch.no_grad():
+        assert torch.equal(block(x), want[0])
 
 
 def _random_case(rng):

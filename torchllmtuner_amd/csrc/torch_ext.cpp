@@ -48,13 +48,16 @@ struct SideStream {
   }
 };
 
-SideStream* side_stream(int device, hipStream_t current) {
+// which: 0 the weight gradients of the fused backward, 1 the shared expert (handed to the Python
+// layer as a raw pointer, see aux_stream below)
+SideStream* side_stream(int device, hipStream_t current, int which = 0) {
   static std::mutex mu;
-  static SideStream per_device[64];
-  static bool tried[64];
-  if (device < 0 || device >= 64) return nullptr;
+  static SideStream streams[2][64];
+  static bool attempted[2][64];
+  if (device < 0 || device >= 64 || which < 0 || which > 1) return nullptr;
   std::lock_guard<std::mutex> lock(mu);
-  SideStream& s = per_device[device];
+  SideStream& s = streams[which][device];
+  bool* tried = attempted[which];
   if (!tried[device]) {
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(current, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone)
@@ -623,9 +626,20 @@ std::tuple<Tensor, Tensor, Tensor, Tensor, Tensor> gather_experts_combine_bwd(
   return {dx, dw1, dw3, dw2, dweights};
 }
 
+// The address of this library's stream for work that runs beside the current stream (a
+// hipStream_t as an integer, for torch.cuda.ExternalStream), or 0 when there is none (yet): it is
+// created on the first call per device that is not under stream capture.
+int64_t aux_stream(int64_t device) {
+  c10::DeviceGuard guard(c10::Device(c10::DeviceType::CUDA, static_cast<c10::DeviceIndex>(device)));
+  const hipStream_t current = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(static_cast<c10::DeviceIndex>(device)).stream();
+  SideStream* s = side_stream(static_cast<int>(device), current, 1);
+  return s ? static_cast<int64_t>(reinterpret_cast<intptr_t>(s->stream)) : 0;
+}
+
 }  // namespace
 
 TORCH_LIBRARY(mi355_moe, m) {
+  m.def("aux_stream(int device) -> int", aux_stream);
   m.def("router_gate_fwd(Tensor x, Tensor w, Tensor? logit_bias) -> Tensor");
   m.def("router_gate_bwd(Tensor dlogits, Tensor x, Tensor w, bool need_dx, bool need_dw) -> (Tensor, Tensor)");
   m.def(

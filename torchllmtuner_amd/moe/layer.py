@@ -18,6 +18,7 @@ from numbers import Real
 import torch
 import torch.nn as nn
 
+from .. import ops
 from .auxiliary_loss import in_checkpoint_recompute
 from .experts import RoutedExperts, _is_own_dispatcher
 from .routing import QuantileBalancedTopKRouter, TokenChoiceTopKRouter
@@ -87,6 +88,11 @@ class MoE(nn.Module):
         )
         self._pending_padding_mask: torch.Tensor | None = None
         self.returns_router_logits = False
+        # The shared expert reads nothing but the tokens: it runs on a second stream beside the
+        # router, the plan and the routed experts (their small kernels and memory-bound tiles
+        # leave most of the matrix cores idle), and autograd runs its backward there as well.
+        # Set to False to keep everything on the caller's stream.
+        self.overlap_shared_experts = True
 
     # The two statistics buffers stay fp32 when the block is cast to bf16
     # (llmtuner/parallel/expert_parallel/block_conversion.py:61-79).
@@ -116,6 +122,31 @@ class MoE(nn.Module):
         self.expert_bias_E.add_(delta_E - delta_E.mean())
         self.tokens_per_expert_E.zero_()
 
+    def _start_shared_experts(self, tokens: torch.Tensor):
+        """Launch the shared expert on the library's second stream, behind everything the
+        caller's stream holds so far.  Returns ``(output, stream)``, or ``(None, None)`` when the
+        shared expert is to run in place (none, switched off, not a real device tensor, under a
+        tracing compiler, or no second stream yet -- its first use must not be under capture)."""
+        if (
+            self.shared_experts is None
+            or not self.overlap_shared_experts
+            or not tokens.is_cuda
+            or isinstance(tokens, torch._subclasses.FakeTensor)
+            or torch.compiler.is_compiling()
+        ):
+            return None, None
+        stream = ops.aux_stream(tokens.device)
+        if stream is None:
+            return None, None
+        stream.wait_stream(torch.cuda.current_stream(tokens.device))
+        if tokens.is_leaf and tokens.requires_grad:
+            # a leaf's gradient accumulator belongs to the stream of the leaf's first use: make
+            # that the caller's stream (a view, no kernel), not the second one
+            tokens = tokens.view_as(tokens)
+        with torch.cuda.stream(stream):
+            shared_TD = self.shared_experts(tokens)
+        return shared_TD, stream
+
     def set_padding_mask(self, padding_mask: torch.Tensor | None) -> None:
         self._pending_padding_mask = padding_mask
 
@@ -135,6 +166,8 @@ class MoE(nn.Module):
                     f"got {tuple(padding_mask.shape)} for {tokens.shape[0]} tokens."
                 )
 
+        shared_TD, shared_stream = self._start_shared_experts(tokens)
+
         topk_scores_TK, topk_expert_ids_TK, routing_map_TE = self.router(
             tokens, self.expert_bias_E, padding_mask_T=padding_mask
         )
@@ -151,7 +184,14 @@ class MoE(nn.Module):
             num_tokens_per_expert_E = routing_map_TE.sum(dim=0)
         out_TD = self.routed_experts(tokens, topk_scores_TK, topk_expert_ids_TK, num_tokens_per_expert_E)
 
-        if self.shared_experts is not None:
+        if shared_stream is not None:
+            # join: the caller's stream waits for the shared expert, whose output (allocated on
+            # the other stream) is marked as used here so that its memory is not handed out early
+            main = torch.cuda.current_stream(tokens.device)
+            main.wait_stream(shared_stream)
+            shared_TD.record_stream(main)
+            out_TD = out_TD + shared_TD
+        elif self.shared_experts is not None:
             out_TD = out_TD + self.shared_experts(tokens)
         # Commit this block's observations only after both expert paths succeeded.
         if self.training and not in_checkpoint_recompute.get():

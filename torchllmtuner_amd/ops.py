@@ -75,6 +75,23 @@ def _opt(t: torch.Tensor, wanted: bool):
     return t if wanted else None
 
 
+_AUX_STREAMS: dict = {}
+
+
+def aux_stream(device: torch.device):
+    """The library's stream for work that may run beside the current stream of ``device`` (the
+    shared expert of a block), as a ``torch.cuda.ExternalStream`` of default priority, or None
+    when there is none: it is created on the first call that is not under stream capture."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    stream = _AUX_STREAMS.get(index)
+    if stream is None:
+        address = _O.aux_stream(index)
+        if not address:
+            return None
+        stream = _AUX_STREAMS[index] = torch.cuda.ExternalStream(address, device=torch.device("cuda", index))
+    return stream
+
+
 # ====================================================================== fake kernels
 # Shape / dtype propagation for tracing.  Skipped outputs are empty (0,) tensors.
 def _fake(name):
