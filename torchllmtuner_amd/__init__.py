@@ -14,6 +14,8 @@ from .moe import (  # noqa: F401
     PaddedTokenDispatcher,
     RoutedExperts,
     RouterGateLinear,
+    SituGLU,
+    SwiGLU,
     TokenChoiceTopKRouter,
 )
 
