@@ -180,6 +180,22 @@ def test_a_block_with_another_activation_runs_three_grouped_linear_maps():
     assert calls == [((N, F), (N, F))] * 2
 
 
+def test_a_block_with_a_shared_expert_traces_without_touching_a_stream():
+    """Under fake tensors (no device behind them) the shared expert runs in place: the second
+    stream is for real device tensors only."""
+    with FakeTensorMode(), torch.device("cuda"):
+        block = _fake_block()
+        torch.set_default_dtype(BF)
+        try:
+            block.shared_experts = moe.DenseSwiGLU(D, 2 * F)
+        finally:
+            torch.set_default_dtype(F32)
+        assert block.overlap_shared_experts
+        x = torch.empty(2, T // 2, D, dtype=BF)
+        assert _shapes(block(x)) == [((2, T // 2, D), BF)]
+        assert block._start_shared_experts(x.reshape(-1, D)) == (None, None)
+
+
 def test_a_routed_experts_subclass_that_replaces_forward_is_honoured():
     """The seam the reference names at experts.py:307-311 (DominoRoutedExperts, MC2RoutedExperts,
     KimiRoutedExperts replace ``forward`` wholesale)."""
