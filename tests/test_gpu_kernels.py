@@ -508,6 +508,50 @@ def test_grouped_experts_module_with_the_situ_activation(ops, dtype, counts, D, 
             assert metric(got, want) < tol, f"{name} {metric(got, want)}"
 
 
+def test_a_subclass_with_its_own_grouped_mm_gets_the_reference_arguments(ops):
+    """``GroupedExperts._grouped_mm(x, weight_EOI, offsets_E)`` is the reference's pluggable product
+    (experts.py:211-216): an override is called for all three projections -- SwiGLU included, which
+    then runs as the activation module between them -- with the cumulative int32 end offsets the
+    reference passes, and the result equals the built-in kernels'."""
+    from torchllmtuner_amd import moe
+
+    print("experts with an overridden _grouped_mm", flush=True)
+    seen = []
+
+    class LoopExperts(moe.GroupedExperts):
+        def _grouped_mm(self, x_TD, weight_EOI, offsets_E):
+            seen.append((tuple(x_TD.shape), tuple(weight_EOI.shape), offsets_E.dtype, offsets_E.cpu().tolist()))
+            out = x_TD.new_zeros(x_TD.shape[0], weight_EOI.shape[1])
+            start = 0
+            for e, end in enumerate(offsets_E.cpu().tolist()):  # the loop path of experts.py:272-285
+                out[start:end] = F.linear(x_TD[start:end], weight_EOI[e])
+                start = end
+            return out
+
+    torch.manual_seed(4)
+    counts, D, Fd = (37, 0, 90, 1), 384, 448
+    mine = LoopExperts(D, Fd, len(counts)).to(DEV).to(torch.bfloat16)
+    builtin = moe.GroupedExperts(D, Fd, len(counts)).to(DEV).to(torch.bfloat16)
+    with torch.no_grad():
+        for p in mine.parameters():
+            p.normal_(0, 0.05)
+        builtin.load_state_dict(mine.state_dict())
+    assert builtin.fuses_activation() and not mine.fuses_activation()
+    x = torch.randn(sum(counts), D, device=DEV).bfloat16()
+    cnt = torch.tensor(counts, device=DEV)
+    xa, xb = x.clone().requires_grad_(), x.clone().requires_grad_()
+    ya, yb = mine(xa, cnt), builtin(xb, cnt)
+    assert [s[:3] for s in seen] == [((128, D), (4, Fd, D), torch.int32)] * 2 + [((128, Fd), (4, D, Fd), torch.int32)]
+    assert all(s[3] == [37, 37, 127, 128] for s in seen)
+    assert rel_l2(ya, yb) < BF16_TOL
+    gy = torch.randn_like(ya)
+    ya.backward(gy)
+    yb.backward(gy)
+    assert rel_l2(xa.grad, xb.grad) < BF16_TOL
+    for pa, pb in zip(mine.parameters(), builtin.parameters()):
+        assert rel_l2(pa.grad, pb.grad) < BF16_TOL
+
+
 # ---------------------------------------------------------------- balance loss
 @pytest.mark.parametrize("seed", [0, 1])
 def test_grouped_experts_bf16_mfma_random_segments(ops, seed):

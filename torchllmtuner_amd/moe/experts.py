@@ -81,6 +81,7 @@ class GroupedExperts(nn.Module):
         # Kept for interface parity; the device path always runs the grouped kernels.
         self.use_grouped_mm = True if use_grouped_mm is None else use_grouped_mm
         self.activation_fn = activation_fn if activation_fn is not None else SwiGLU()
+        self._call_plan = None  # (plan, zero_fill) while compute_planned runs its grouped products
         self.w1_EFD = nn.Parameter(torch.empty(num_experts, hidden_dim, dim))
         self.w3_EFD = nn.Parameter(torch.empty(num_experts, hidden_dim, dim))
         self.w2_EDF = nn.Parameter(torch.empty(num_experts, dim, hidden_dim))
@@ -121,10 +122,14 @@ class GroupedExperts(nn.Module):
         plan = ops.segments_from_counts(num_tokens_per_expert_E, x_RD.shape[0])
         return self.compute_planned(x_RD, plan, zero_fill=True)
 
-    def _grouped_mm(self, x_RI, weight_EOI, plan: ops.PermutePlan, zero_fill: bool = False):
-        """``x . weight[e]^T`` per expert segment (experts.py:211-216).  The reference passes the
-        cumulative offsets; here the segments travel as the plan they were counted into."""
-        return Fn.grouped_linear(x_RI, weight_EOI, plan, zero_fill=zero_fill)
+    def _grouped_mm(self, x_TD, weight_EOI, offsets_E):
+        """``x . weight[e]^T`` per expert segment: the reference's pluggable product, with its
+        signature (experts.py:211-216).  ``offsets_E`` are the segments' end offsets (int32), the
+        cumulative counts the reference passes to ``torch._grouped_mm``; this implementation
+        reads the same segments from the plan of the call in progress, which also carries the
+        tile list the kernels walk.  An override receives exactly the reference's arguments."""
+        plan, zero_fill = self._call_plan
+        return Fn.grouped_linear(x_TD, weight_EOI, plan, zero_fill=zero_fill)
 
     def fuses_activation(self) -> bool:
         """SwiGLU exactly (not a subclass that may compute something else) is evaluated inside
@@ -141,10 +146,15 @@ class GroupedExperts(nn.Module):
         if self.fuses_activation():
             return Fn.grouped_swiglu(x_RD, w1, w3, w2, plan, zero_fill=zero_fill)
         # experts.py:204-209 with the caller's activation: gate, up, activation(gate, up), down
-        gate = self._grouped_mm(x_RD, w1, plan, zero_fill=zero_fill)
-        up = self._grouped_mm(x_RD, w3, plan, zero_fill=zero_fill)
-        h = self.activation_fn(gate, up)
-        return self._grouped_mm(h, w2, plan, zero_fill=zero_fill).type_as(x_RD)
+        offsets_E = plan.seg_offsets[1:]
+        self._call_plan = (plan, zero_fill)  # (one call at a time per module, like any forward)
+        try:
+            gate = self._grouped_mm(x_RD, w1, offsets_E)
+            up = self._grouped_mm(x_RD, w3, offsets_E)
+            h = self.activation_fn(gate, up)
+            return self._grouped_mm(h, w2, offsets_E).type_as(x_RD)
+        finally:
+            self._call_plan = None
 
 
 class RoutedExperts(nn.Module):
