@@ -552,6 +552,38 @@ def test_a_subclass_with_its_own_grouped_mm_gets_the_reference_arguments(ops):
         assert rel_l2(pa.grad, pb.grad) < BF16_TOL
 
 
+@pytest.mark.parametrize("dtype,D,Fd,align", [(torch.float32, 96, 160, 1), (torch.bfloat16, 72, 40, 8), (torch.float64, 24, 40, 1),
+                                              (torch.bfloat16, 384, 448, 1)])
+def test_rows_experts_combine_is_the_three_stages_in_one_operator(ops, dtype, D, Fd, align):
+    """The one-operator form of scatter -> experts -> combine (what the module layer runs where the
+    folded kernels do not apply) gives the output and every gradient of the three differentiable
+    stages composed by hand, bit for bit."""
+    print(f"rows_experts_combine {dtype} D={D} F={Fd} align={align}", flush=True)
+    T, K, E = 300, 4, 8
+    g = torch.Generator().manual_seed(13)
+    ids = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(T)]).to(DEV)
+    mk = lambda *s: (torch.randn(*s, generator=g, dtype=torch.float64) * 0.1).to(dtype).to(DEV)
+    leaves_a = [torch.randn(T, D, generator=g, dtype=torch.float64).to(dtype).to(DEV), torch.rand(T, K, generator=g).to(DEV),
+                mk(E, Fd, D), mk(E, Fd, D), mk(E, D, Fd)]
+    leaves_b = [t.clone() for t in leaves_a]
+    for t in leaves_a + leaves_b:
+        t.requires_grad_()
+    dout = torch.randn(T, D, generator=g, dtype=torch.float64).to(dtype).to(DEV)
+    plan = ops.permute_plan(ids, E, 0, E, align)
+    one = ops.rows_experts_combine(*leaves_a, plan)
+    x, wts, w1, w3, w2 = leaves_b
+    three = ops.combine(ops.grouped_swiglu(ops.permute_rows(x, plan), w1, w3, w2, plan), wts, plan)
+    assert torch.equal(one, three)
+    one.backward(dout)
+    three.backward(dout)
+    for a, b in zip(leaves_a, leaves_b):
+        assert torch.equal(a.grad, b.grad)
+    # only the scores ask for a gradient
+    w_only = leaves_a[1].detach().clone().requires_grad_()
+    ops.rows_experts_combine(leaves_a[0].detach(), w_only, *(t.detach() for t in leaves_a[2:]), plan).backward(dout)
+    assert torch.equal(w_only.grad, leaves_b[1].grad)
+
+
 # ---------------------------------------------------------------- balance loss
 @pytest.mark.parametrize("seed", [0, 1])
 def test_grouped_experts_bf16_mfma_random_segments(ops, seed):

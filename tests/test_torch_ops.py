@@ -40,7 +40,7 @@ def test_every_operator_is_registered_with_a_fake_kernel_and_propagates_shapes()
         "balance_loss_bwd", "permute_plan", "segments_from_counts", "permute_rows_fwd", "permute_rows_bwd",
         "combine_fwd", "combine_bwd", "combine_row_scale", "combine_scores_bwd", "grouped_swiglu_fwd",
         "grouped_swiglu_bwd", "grouped_linear_fwd", "grouped_linear_bwd", "gather_experts_combine_fwd",
-        "gather_experts_combine_bwd",
+        "gather_experts_combine_bwd", "rows_experts_combine_fwd", "rows_experts_combine_bwd",
     }
     tile_cap = N // ops.TILE_M + El + 1
     small = E + (El + 1) + 2 * El + 2 * tile_cap + 1
@@ -81,6 +81,13 @@ def test_every_operator_is_registered_with_a_fake_kernel_and_propagates_shapes()
                                    [((N, D), BF), ((El, F, D), BF), ((El, F, D), BF), ((El, D, F), BF)]),
             "grouped_linear_fwd": (O.grouped_linear_fwd(rows, w1, *seg, False), [((N, F), BF)]),
             "grouped_linear_bwd": (O.grouped_linear_bwd(rf, rows, w1, *seg, True, False, False), [((N, D), BF), ((0,), BF)]),
+            "rows_experts_combine_fwd": (
+                O.rows_experts_combine_fwd(x, wts, w1, w3, w2, ros, None, seg[4], *seg, K, N, True),
+                [((T, D), BF), ((N, D), BF), ((N, F), BF), ((N, F), BF), ((N, F), BF), ((N, D), BF)]),
+            "rows_experts_combine_bwd": (
+                O.rows_experts_combine_bwd(x, rows, wts, w1, w3, w2, rf, rf, rf, rows, ros, None, seg[4], *seg, T, K,
+                                           True, True),
+                [((T, D), BF), ((El, F, D), BF), ((El, F, D), BF), ((El, D, F), BF), ((T, K), F32)]),
             "gather_experts_combine_fwd": (
                 O.gather_experts_combine_fwd(x, wts, w1, w3, w2, tok, sor, ros, *seg, K, N, True, True),
                 [((T, D), BF), ((N, F), BF), ((N, F), BF)]),

@@ -626,6 +626,39 @@ std::tuple<Tensor, Tensor, Tensor, Tensor, Tensor> gather_experts_combine_bwd(
   return {dx, dw1, dw3, dw2, dweights};
 }
 
+// The three stages of the routed path that has no folded form (fp32, fp64, shapes off the bf16
+// MFMA path) as ONE operator each way: row scatter, grouped SwiGLU experts and combine going
+// forward; combine, experts and K-way row sum going back.  Nothing new is computed -- these call
+// the stage operators above in order -- but a step then crosses the dispatcher and the autograd
+// engine once per direction instead of three times, which is what a small step's time is made of.
+// Returns (out, rows, gate, up, h, y): everything but `out` is kept for the backward.
+std::tuple<Tensor, Tensor, Tensor, Tensor, Tensor, Tensor> rows_experts_combine_fwd(
+    const Tensor& x, const Tensor& weights, const Tensor& w1, const Tensor& w3, const Tensor& w2,
+    const Tensor& row_of_slot, const OptTensor& slot_of_row, const Tensor& total_rows, const Tensor& seg_offsets,
+    const Tensor& seg_counts, const Tensor& tile_expert, const Tensor& tile_row0, const Tensor& num_tiles, int64_t K,
+    int64_t row_capacity, bool round_terms) {
+  Tensor rows = permute_rows_fwd(x, row_of_slot, slot_of_row, total_rows, K, row_capacity);
+  auto [y, gate, up, h] = grouped_swiglu_fwd(rows, std::nullopt, w1, w3, w2, seg_offsets, seg_counts, tile_expert,
+                                             tile_row0, num_tiles, row_capacity, false);
+  Tensor out = combine_fwd(y, weights, row_of_slot, slot_of_row, total_rows, x.size(0), K, round_terms);
+  return {out, rows, gate, up, h, y};
+}
+
+// Returns (dx, dw1, dw3, dw2, dweights).
+std::tuple<Tensor, Tensor, Tensor, Tensor, Tensor> rows_experts_combine_bwd(
+    const Tensor& dout, const Tensor& rows, const Tensor& weights, const Tensor& w1, const Tensor& w3,
+    const Tensor& w2, const Tensor& gate, const Tensor& up, const Tensor& h, const Tensor& y,
+    const Tensor& row_of_slot, const OptTensor& slot_of_row, const Tensor& total_rows, const Tensor& seg_offsets,
+    const Tensor& seg_counts, const Tensor& tile_expert, const Tensor& tile_row0, const Tensor& num_tiles, int64_t T,
+    int64_t K, bool need_dx, bool need_dw) {
+  auto [dy, dweights] = combine_bwd(dout, y, weights, row_of_slot, slot_of_row, total_rows, K);
+  auto [drows, dw1, dw3, dw2] = grouped_swiglu_bwd(dy, rows, std::nullopt, w1, w3, w2, gate, up, h, seg_offsets,
+                                                   seg_counts, tile_expert, tile_row0, num_tiles, need_dx, need_dw,
+                                                   false);
+  Tensor dx = need_dx ? permute_rows_bwd(drows, row_of_slot, T, K) : none_like(rows);
+  return {dx, dw1, dw3, dw2, dweights};
+}
+
 // The address of this library's stream for work that runs beside the current stream (a
 // hipStream_t as an integer, for torch.cuda.ExternalStream), or 0 when there is none (yet): it is
 // created on the first call per device that is not under stream capture.
@@ -692,6 +725,16 @@ TORCH_LIBRARY(mi355_moe, m) {
       "grouped_linear_bwd(Tensor dy, Tensor x, Tensor w, Tensor seg_offsets, Tensor seg_counts, Tensor tile_expert, "
       "Tensor tile_row0, Tensor num_tiles, bool need_dx, bool need_dw, bool zero_fill) -> (Tensor, Tensor)");
   m.def(
+      "rows_experts_combine_fwd(Tensor x, Tensor weights, Tensor w1, Tensor w3, Tensor w2, Tensor row_of_slot, "
+      "Tensor? slot_of_row, Tensor total_rows, Tensor seg_offsets, Tensor seg_counts, Tensor tile_expert, "
+      "Tensor tile_row0, Tensor num_tiles, int top_k, int row_capacity, bool round_terms) -> "
+      "(Tensor, Tensor, Tensor, Tensor, Tensor, Tensor)");
+  m.def(
+      "rows_experts_combine_bwd(Tensor dout, Tensor rows, Tensor weights, Tensor w1, Tensor w3, Tensor w2, "
+      "Tensor gate, Tensor up, Tensor h, Tensor y, Tensor row_of_slot, Tensor? slot_of_row, Tensor total_rows, "
+      "Tensor seg_offsets, Tensor seg_counts, Tensor tile_expert, Tensor tile_row0, Tensor num_tiles, int num_tokens, "
+      "int top_k, bool need_dx, bool need_dw) -> (Tensor, Tensor, Tensor, Tensor, Tensor)");
+  m.def(
       "gather_experts_combine_fwd(Tensor x, Tensor weights, Tensor w1, Tensor w3, Tensor w2, Tensor token_of_row, "
       "Tensor slot_of_row, Tensor row_of_slot, Tensor seg_offsets, Tensor seg_counts, Tensor tile_expert, Tensor tile_row0, "
       "Tensor num_tiles, int top_k, int row_capacity, bool round_terms, bool save_gate_up) -> (Tensor, Tensor, Tensor)");
@@ -726,6 +769,8 @@ TORCH_LIBRARY_IMPL(mi355_moe, CUDA, m) {
   m.impl("grouped_swiglu_bwd", grouped_swiglu_bwd);
   m.impl("grouped_linear_fwd", grouped_linear_fwd);
   m.impl("grouped_linear_bwd", grouped_linear_bwd);
+  m.impl("rows_experts_combine_fwd", rows_experts_combine_fwd);
+  m.impl("rows_experts_combine_bwd", rows_experts_combine_bwd);
   m.impl("gather_experts_combine_fwd", gather_experts_combine_fwd);
   m.impl("gather_experts_combine_bwd", gather_experts_combine_bwd);
 }

@@ -205,13 +205,27 @@ class RoutedExperts(nn.Module):
                 w1, w3, w2 = experts._weights_as(x_TD.dtype)
                 out = Fn.gather_experts_combine(x_TD, topk_scores_TK, w1, w3, w2, plan, round_terms)
                 return out.to(x_TD.dtype)
+            if _is_plain_grouped_experts(experts) and experts.fuses_activation():
+                # the same three stages as below as one operator each way: one trip through the
+                # dispatcher and one autograd node, which is most of a small step's time
+                with observe:
+                    plan = dispatcher.plan(topk_expert_ids_TK)
+                w1, w3, w2 = experts._weights_as(x_TD.dtype)
+                out = Fn.rows_experts_combine(x_TD, topk_scores_TK, w1, w3, w2, plan, round_terms)
+                return out.to(x_TD.dtype)
             with observe:
                 plan = dispatcher.plan(topk_expert_ids_TK)
                 rows = Fn.permute_rows(x_TD, plan)
-            # rows per local expert as laid out (padding included), the counts the reference hands
-            # to its inner module; rows past the last segment are not covered and come back as zeros
-            covered = plan.seg_offsets[1:] - plan.seg_offsets[:-1]
-            y = experts(rows, covered)
+            if _is_plain_grouped_experts(experts):
+                # nothing hangs on the inner module's call: the experts run on the dispatcher's own
+                # plan (no second plan from counts, no count arithmetic; padding rows belong to no
+                # segment, are not computed and are never read by the combine)
+                y = experts.compute_planned(rows, plan)
+            else:
+                # rows per local expert as laid out (padding included), the counts the reference hands
+                # to its inner module; rows past the last segment are not covered and come back as zeros
+                covered = plan.seg_offsets[1:] - plan.seg_offsets[:-1]
+                y = experts(rows, covered)
             out = Fn.combine(y, topk_scores_TK, plan, round_terms)
             return out.to(x_TD.dtype)
         finally:

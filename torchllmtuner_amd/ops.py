@@ -243,6 +243,22 @@ def _(dy, x, w, seg_offsets, seg_counts, tile_expert, tile_row0, num_tiles, need
     return (torch.empty_like(x) if need_dx else _e0(x)), (torch.empty_like(w) if need_dw else _e0(w))
 
 
+@_fake("rows_experts_combine_fwd")
+def _(x, weights, w1, w3, w2, row_of_slot, slot_of_row, total_rows, seg_offsets, seg_counts, tile_expert, tile_row0,
+      num_tiles, top_k, row_capacity, round_terms):
+    F = w1.shape[1]
+    mk = lambda n: x.new_empty((row_capacity, n))
+    return torch.empty_like(x), mk(x.shape[1]), mk(F), mk(F), mk(F), mk(x.shape[1])
+
+
+@_fake("rows_experts_combine_bwd")
+def _(dout, rows, weights, w1, w3, w2, gate, up, h, y, row_of_slot, slot_of_row, total_rows, seg_offsets, seg_counts,
+      tile_expert, tile_row0, num_tiles, num_tokens, top_k, need_dx, need_dw):
+    g = lambda w: torch.empty_like(w) if need_dw else _e0(w)
+    dx = rows.new_empty((num_tokens, rows.shape[1])) if need_dx else _e0(rows)
+    return dx, g(w1), g(w3), g(w2), rows.new_empty((num_tokens, top_k), dtype=torch.float32)
+
+
 @_fake("gather_experts_combine_fwd")
 def _(x, weights, w1, w3, w2, token_of_row, slot_of_row, row_of_slot, seg_offsets, seg_counts, tile_expert,
       tile_row0, num_tiles, top_k, row_capacity, round_terms, save_gate_up):
@@ -476,6 +492,31 @@ def _gl_backward(ctx, dy):
 
 
 _autograd("grouped_linear_fwd", _gl_backward, _gl_setup)
+
+
+# -- row scatter + experts + combine as one node (the path without a folded form)
+def _rec_setup(ctx, inputs, output):
+    x, weights, w1, w3, w2, ros, sor, total, so, sc, te, tr, nt, top_k, _cap, _round = inputs
+    _out, rows, gate, up, h, y = output
+    ctx.save_for_backward(rows, weights, w1, w3, w2, gate, up, h, y, ros, sor, total, so, sc, te, tr, nt)
+    ctx.top_k, ctx.num_tokens = top_k, x.shape[0]
+    ctx.set_materialize_grads(False)
+
+
+def _rec_backward(ctx, dout, *_unused):
+    rows, weights, w1, w3, w2, gate, up, h, y, ros, sor, total, so, sc, te, tr, nt = ctx.saved_tensors
+    need = ctx.needs_input_grad
+    if dout is None:
+        return (None,) * 16
+    need_dw = need[2] or need[3] or need[4]
+    dx, dw1, dw3, dw2, dweights = _O.rows_experts_combine_bwd(
+        dout, rows, weights, w1, w3, w2, gate, up, h, y, ros, sor, total, so, sc, te, tr, nt, ctx.num_tokens,
+        ctx.top_k, need[0], need_dw)
+    return ((dx if need[0] else None), (dweights.to(weights.dtype) if need[1] else None),
+            (dw1 if need[2] else None), (dw3 if need[3] else None), (dw2 if need[4] else None)) + (None,) * 11
+
+
+_autograd("rows_experts_combine_fwd", _rec_backward, _rec_setup)
 
 
 # -- gathered experts + combine: one backward for both halves
@@ -838,6 +879,18 @@ def gather_experts_combine(x_TD, weights_TK, w1_EFD, w3_EFD, w2_EDF, plan: Permu
         x_TD, weights_TK, w1_EFD, w3_EFD, w2_EDF, plan.token_of_row, plan.slot_of_row, plan.row_of_slot,
         *plan.segments(), plan.top_k, plan.row_capacity, bool(round_terms), differentiable)
     return out
+
+
+def rows_experts_combine(x_TD, weights_TK, w1_EFD, w3_EFD, w2_EDF, plan: PermutePlan, round_terms=True):
+    """The same function as ``gather_experts_combine`` for every dtype and shape, in stages: the
+    plan's row scatter, the grouped SwiGLU experts, the combine -- as one operator each way (one
+    trip through the dispatcher and one autograd node instead of three).  What the module layer
+    runs where the folded kernels do not apply (fp32, fp64, widths off the bf16 MFMA path)."""
+    _dev(x_TD, weights_TK, w1_EFD, w3_EFD, w2_EDF)
+    _check_experts(x_TD, w1_EFD, w3_EFD, w2_EDF, plan)
+    return _O.rows_experts_combine_fwd(
+        x_TD, weights_TK, w1_EFD, w3_EFD, w2_EDF, plan.row_of_slot, plan.pad_index(), plan.total_rows_1(),
+        *plan.segments(), plan.top_k, plan.row_capacity, bool(round_terms))[0]
 
 
 def combine_row_scale(weights_TK, plan: PermutePlan):
