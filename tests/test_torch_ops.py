@@ -268,3 +268,20 @@ def test_dispatcher_reuses_the_plan_for_the_same_ids_tensor_only():
         p2 = disp.plan(ids2)
         ids2.add_(1)  # changed in place: a new plan
         assert disp.plan(ids2) is not p2
+
+
+def test_exit_hook_is_idle_without_a_gpu():
+    """The package's exit hook (it lets the autograd engine's thread take the GIL once more before the
+    interpreter finalises) costs nothing in a process that never initialised the GPU."""
+    import atexit
+    import time
+
+    from torchllmtuner_amd import ops
+
+    assert callable(ops._let_autograd_threads_finish)
+    atexit.unregister(ops._let_autograd_threads_finish)  # (what import registered; put back below)
+    atexit.register(ops._let_autograd_threads_finish)
+    if not torch.cuda.is_initialized():
+        t0 = time.perf_counter()
+        ops._let_autograd_threads_finish()
+        assert time.perf_counter() - t0 < 0.02

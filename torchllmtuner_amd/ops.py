@@ -15,6 +15,8 @@ pre-allocated buffers) go straight to the C ABI through ``ctypes``.
 
 from __future__ import annotations
 
+import atexit
+import time
 from dataclasses import dataclass
 
 import torch
@@ -90,6 +92,19 @@ def aux_stream(device: torch.device):
             return None
         stream = _AUX_STREAMS[index] = torch.cuda.ExternalStream(address, device=torch.device("cuda", index))
     return stream
+
+
+def _let_autograd_threads_finish():
+    """Runs at interpreter exit.  After a backward pass the autograd engine's device thread may still be
+    releasing that pass's results; for the ones Python holds a wrapper of it needs the GIL, and CPython
+    ends a thread that asks for the GIL once finalisation has begun, which aborts the process (status
+    134, after all work is done) when the script exits within milliseconds of its last backward pass.
+    Giving up the GIL for a moment before finalisation begins lets that thread finish."""
+    if torch.cuda.is_initialized():
+        time.sleep(0.05)
+
+
+atexit.register(_let_autograd_threads_finish)
 
 
 # ====================================================================== fake kernels
