@@ -6,8 +6,9 @@
 // host, and turns a negative return code into a Python exception (MI355_EINVAL ->
 // ValueError, anything else -> RuntimeError) carrying mi355_moe_last_error().  Nothing is
 // computed here: argument validation that mirrors the reference's messages lives in the
-// Python host layer, shape propagation for tracing (fake tensors) and the autograd formulas
-// in torchllmtuner_amd/ops.py, and the arithmetic in the HIP kernels behind the C ABI.
+// Python host layer, shape propagation for tracing (fake tensors) in torchllmtuner_amd/ops.py,
+// the autograd formulas there and in torch_autograd.cpp, and the arithmetic in the HIP kernels
+// behind the C ABI.
 //
 // Plan tensors.  A permutation plan travels as plain int32 tensors: `small` packs
 // counts_E (E) | seg_offsets (El+1) | seg_counts (El) | expert_order (El) |

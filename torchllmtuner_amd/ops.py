@@ -291,7 +291,11 @@ def _(dout, x, weights, w1, w3, w2, gate, up, token_of_row, slot_of_row, row_of_
 
 
 # ====================================================================== autograd formulas
-# Each differentiable operator's backward is the hand-written kernel for that stage.
+# Each differentiable operator's backward is the hand-written kernel for that stage.  The operators on a
+# block's own path (router_gate_fwd, router_select_fwd, grouped_swiglu_fwd, rows_experts_combine_fwd,
+# gather_experts_combine_fwd; linear.py:133-151 is the gate's formula) have theirs as C++ autograd nodes
+# in csrc/torch_autograd.cpp, which run on the engine's thread without the interpreter lock; the formulas
+# below are those of the remaining building blocks.
 # The registration is what ``torch.library.register_autograd`` does -- a Python kernel for the
 # operator's Autograd dispatch key that wraps the call in an ``autograd.Function`` -- without
 # its per-call ``fill_defaults``: that helper re-reads ``schema.arguments`` (a fresh list of
@@ -332,47 +336,6 @@ def _autograd(name, backward, setup):
             return op.redispatch(keyset & _AFTER_AUTOGRAD, *args)
 
     _AUTOGRAD_LIB.impl(name, autograd_kernel, "Autograd", with_keyset=True)
-
-
-# -- router gate: dX in the input dtype, dW in the weight dtype (linear.py:133-151)
-def _rg_setup(ctx, inputs, output):
-    x, w, bias = inputs
-    ctx.save_for_backward(x, w)
-    ctx.bias_dtype = None if bias is None else bias.dtype
-
-
-def _rg_backward(ctx, grad_TE):
-    x, w = ctx.saved_tensors
-    need = ctx.needs_input_grad
-    dx = dw = None
-    if need[0] or need[1]:
-        dx, dw = _O.router_gate_bwd(grad_TE, x, w, need[0], need[1])
-    db = grad_TE.float().sum(dim=0).to(ctx.bias_dtype) if (ctx.bias_dtype is not None and need[2]) else None
-    return (dx if need[0] else None), (dw if need[1] else None), db
-
-
-_autograd("router_gate_fwd", _rg_backward, _rg_setup)
-
-
-# -- select: gather / norm / scale / score VJP per token; ids and the map are not differentiable
-def _rs_setup(ctx, inputs, output):
-    logits, _bias, _k, score_func, route_norm, route_scale, _g, _l, mode, want_scores, _m = inputs
-    ctx.save_for_backward(logits, output[1])
-    ctx.cfg = (score_func, route_norm, route_scale, mode, want_scores)
-    ctx.set_materialize_grads(False)
-
-
-def _rs_backward(ctx, dweights, _dids, dscores, _dmap):
-    logits, ids = ctx.saved_tensors
-    score_func, route_norm, route_scale, mode, want_scores = ctx.cfg
-    dlogits = None
-    if ctx.needs_input_grad[0]:
-        dlogits = _O.router_select_bwd(logits, ids, dweights, dscores if want_scores else None, score_func,
-                                       route_norm, route_scale, mode)
-    return (dlogits,) + (None,) * 10
-
-
-_autograd("router_select_fwd", _rs_backward, _rs_setup)
 
 
 def _rsc_setup(ctx, inputs, output):
@@ -460,35 +423,6 @@ def _cb_backward(ctx, dout):
 _autograd("combine_fwd", _cb_backward, _cb_setup)
 
 
-# -- grouped experts
-def _gs_setup(ctx, inputs, output):
-    rows, tok, w1, w3, w2, so, sc, te, tr, nt, _cap, zero_fill = inputs
-    _y, gate, up, h = output
-    ctx.gathered = tok is not None
-    ctx.save_for_backward(rows, w1, w3, w2, gate, up, h, so, sc, te, tr, nt)
-    ctx.zero_fill = zero_fill
-    ctx.set_materialize_grads(False)
-
-
-def _gs_backward(ctx, dy, _dgate, _dup, _dh):
-    if ctx.gathered:
-        raise NotImplementedError(
-            "grouped_swiglu_fwd with a token gather is differentiated through gather_experts_combine_fwd"
-        )
-    rows, w1, w3, w2, gate, up, h, so, sc, te, tr, nt = ctx.saved_tensors
-    need = ctx.needs_input_grad
-    if dy is None:
-        return (None,) * 12
-    need_dw = need[2] or need[3] or need[4]
-    drows, dw1, dw3, dw2 = _O.grouped_swiglu_bwd(dy, rows, None, w1, w3, w2, gate, up, h, so, sc, te, tr, nt,
-                                                 need[0], need_dw, ctx.zero_fill)
-    return ((drows if need[0] else None), None, (dw1 if need[2] else None), (dw3 if need[3] else None),
-            (dw2 if need[4] else None)) + (None,) * 7
-
-
-_autograd("grouped_swiglu_fwd", _gs_backward, _gs_setup)
-
-
 # -- one grouped linear map (the reference's GroupedExperts._grouped_mm)
 def _gl_setup(ctx, inputs, output):
     x, w, so, sc, te, tr, nt, zero_fill = inputs
@@ -507,57 +441,6 @@ def _gl_backward(ctx, dy):
 
 
 _autograd("grouped_linear_fwd", _gl_backward, _gl_setup)
-
-
-# -- row scatter + experts + combine as one node (the path without a folded form)
-def _rec_setup(ctx, inputs, output):
-    x, weights, w1, w3, w2, ros, sor, total, so, sc, te, tr, nt, top_k, _cap, _round = inputs
-    _out, rows, gate, up, h, y = output
-    ctx.save_for_backward(rows, weights, w1, w3, w2, gate, up, h, y, ros, sor, total, so, sc, te, tr, nt)
-    ctx.top_k, ctx.num_tokens = top_k, x.shape[0]
-    ctx.set_materialize_grads(False)
-
-
-def _rec_backward(ctx, dout, *_unused):
-    rows, weights, w1, w3, w2, gate, up, h, y, ros, sor, total, so, sc, te, tr, nt = ctx.saved_tensors
-    need = ctx.needs_input_grad
-    if dout is None:
-        return (None,) * 16
-    need_dw = need[2] or need[3] or need[4]
-    dx, dw1, dw3, dw2, dweights = _O.rows_experts_combine_bwd(
-        dout, rows, weights, w1, w3, w2, gate, up, h, y, ros, sor, total, so, sc, te, tr, nt, ctx.num_tokens,
-        ctx.top_k, need[0], need_dw)
-    return ((dx if need[0] else None), (dweights.to(weights.dtype) if need[1] else None),
-            (dw1 if need[2] else None), (dw3 if need[3] else None), (dw2 if need[4] else None)) + (None,) * 11
-
-
-_autograd("rows_experts_combine_fwd", _rec_backward, _rec_setup)
-
-
-# -- gathered experts + combine: one backward for both halves
-def _gec_setup(ctx, inputs, output):
-    x, weights, w1, w3, w2, tok, sor, ros, so, sc, te, tr, nt, top_k, _cap, _round, saved = inputs
-    if not saved:
-        raise RuntimeError("gather_experts_combine_fwd was run without its gate / up outputs and cannot be differentiated")
-    _out, gate, up = output
-    ctx.save_for_backward(x, weights, w1, w3, w2, gate, up, tok, sor, ros, so, sc, te, tr, nt)
-    ctx.top_k = top_k
-    ctx.set_materialize_grads(False)
-
-
-def _gec_backward(ctx, dout, _dgate, _dup):
-    x, weights, w1, w3, w2, gate, up, tok, sor, ros, so, sc, te, tr, nt = ctx.saved_tensors
-    need = ctx.needs_input_grad
-    if dout is None:
-        return (None,) * 17
-    need_dw = need[2] or need[3] or need[4]
-    dx, dw1, dw3, dw2, dweights = _O.gather_experts_combine_bwd(
-        dout, x, weights, w1, w3, w2, gate, up, tok, sor, ros, so, sc, te, tr, nt, ctx.top_k, need[0], need_dw)
-    return ((dx if need[0] else None), (dweights.to(weights.dtype) if need[1] else None),
-            (dw1 if need[2] else None), (dw3 if need[3] else None), (dw2 if need[4] else None)) + (None,) * 12
-
-
-_autograd("gather_experts_combine_fwd", _gec_backward, _gec_setup)
 
 
 # ====================================================================== router
