@@ -876,3 +876,64 @@ def test_balance_loss_hook_injects_the_reference_gradient(score_func, with_paddi
     xd2 = x.to(DEV).requires_grad_()
     block(xd2).backward(gout.to(DEV))
     assert rel_max(block.router.gate.weight.grad, leaves["router_w_ED"].grad) > 1e-4
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,D,F", [(torch.float32, 64, 96), (torch.bfloat16, 384, 384)])
+def test_partial_gradient_requests_give_the_same_gradients_and_skip_the_rest(dtype, D, F):
+    """Frozen parameters, an input that needs no gradient and a trainable gate bias: every gradient that
+    is asked for equals the one of the run where everything is trainable (bit for bit: the same kernels
+    run), and nothing is returned for what was not asked.  (The autograd nodes of the block's operators
+    index needs_input_grad by tensor argument; linear.py:133-151 has the gate's three gradients.)"""
+    T, E, K = 200, 8, 2
+    spec = R.RouterSpec(E, K, score_func="sigmoid", route_norm=True)
+    p = make_params(E, D, F, dtype, seed=3, std=0.1, shared_F=F)
+    p.router_logit_bias_E = torch.linspace(-0.2, 0.2, E)
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(T, D, generator=g).to(dtype).to(DEV)
+    gout = torch.randn(T, D, generator=g).to(dtype).to(DEV)
+
+    def run(frozen=(), x_grad=True, bias_grad=False):
+        block = build_block(p, spec, D, F, dtype, DEV)
+        block.train()
+        block.router.gate.bias.requires_grad_(bias_grad)
+        named = dict(block.named_parameters())
+        for name in frozen:
+            named[name].requires_grad_(False)
+        xin = x.clone().requires_grad_(x_grad)
+        block(xin).backward(gout)
+        grads = {n: q.grad for n, q in named.items()}
+        grads["x"] = xin.grad
+        return grads
+
+    full = run(bias_grad=True)
+    assert all(v is not None for v in full.values())
+    # the gate bias gradient against the oracle's, with the bias as a leaf of the oracle's graph
+    leaves = {k: getattr(p, k).clone() for k in
+              ("router_w_ED", "w1_EFD", "w3_EFD", "w2_EDF", "shared_gate_FD", "shared_up_FD", "shared_down_DF")}
+    bias_leaf = p.router_logit_bias_E.clone().requires_grad_()
+    ref, _ = R.moe_forward(x.cpu(), R.MoEParams(expert_bias_E=None, router_logit_bias_E=bias_leaf, **leaves), spec)
+    ref.backward(gout.cpu())
+    tol, metric = (1e-5, rel_max) if dtype == torch.float32 else (2e-2, rel_l2)
+    assert full["router.gate.bias"].shape == (E,)
+    assert metric(full["router.gate.bias"], bias_leaf.grad) < tol, metric(full["router.gate.bias"], bias_leaf.grad)
+    cases = [
+        dict(frozen=("routed_experts.inner_experts.w1_EFD",)),
+        dict(frozen=("routed_experts.inner_experts.w3_EFD", "routed_experts.inner_experts.w2_EDF")),
+        dict(frozen=("router.gate.weight",), bias_grad=True),
+        dict(frozen=("shared_experts.up_proj.weight",), x_grad=False),
+        dict(frozen=tuple(n for n in full if n not in ("x", "router.gate.bias")), x_grad=True),
+        dict(x_grad=False, bias_grad=True),
+    ]
+    for case in cases:
+        got = run(**case)
+        skipped = set(case.get("frozen", ()))
+        if not case.get("x_grad", True):
+            skipped.add("x")
+        if not case.get("bias_grad", False):
+            skipped.add("router.gate.bias")
+        for name, want in full.items():
+            if name in skipped:
+                assert got[name] is None, (case, name)
+            else:
+                assert got[name] is not None and torch.equal(got[name], want), (case, name)
