@@ -909,8 +909,12 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(WgradArgs p) {
       // whole tiles only: the stores are unconditional, so the compiler knows how many follow
       // the operand loads requested above and the next tile's wait for those loads does not
       // also wait for these stores (one counter serves both)
-      *reinterpret_cast<u32x4*>(C + static_cast<int64_t>(m) * N + n) =
-          *reinterpret_cast<const u32x4*>(st + (idx >> 4) * S::PITCH + (idx & 15) * 8);
+      // (non-temporal: a weight gradient is several times the size of L2 and is read next by the
+      // optimizer; written through the cache as ordinary stores, an expert's 30-60 MB of results push
+      // its own operands out of L2 between two of its tiles -- with few rows per expert, where the
+      // product is bound by these writes, the gathered rows were fetched from memory several times over)
+      __builtin_nontemporal_store(*reinterpret_cast<const u32x4*>(st + (idx >> 4) * S::PITCH + (idx & 15) * 8),
+                                  reinterpret_cast<u32x4*>(C + static_cast<int64_t>(m) * N + n));
     }
     // staging regions are free again before the next tile's operands are parked; only
     // the LDS traffic is waited for, the tile's stores keep draining
