@@ -4,8 +4,9 @@
 thin C++ layer that allocates outputs with PyTorch's allocator and calls the C ABI of
 ``include/mi355_moe.h`` on the current HIP stream.  This module adds what the dispatcher
 needs around them -- shape propagation for fake / meta tensors (so the operators trace
-under ``torch.compile``) and the autograd formulas, whose backward passes are again
-operators of the same library -- plus Python wrappers that validate arguments the way the
+under ``torch.compile``) and the autograd formulas of the public building blocks, whose backward
+passes are again operators of the same library (the operators on a block's own path have theirs
+as C++ autograd nodes inside ``libmi355moe_torch.so``) -- plus Python wrappers that validate arguments the way the
 reference's modules do and carry the permutation plan as one object.
 
 Every function requires device tensors and raises if given CPU tensors: the kernels are the
