@@ -4,9 +4,8 @@
 thin C++ layer that allocates outputs with PyTorch's allocator and calls the C ABI of
 ``include/mi355_moe.h`` on the current HIP stream.  This module adds what the dispatcher
 needs around them -- shape propagation for fake / meta tensors (so the operators trace
-under ``torch.compile``) and the autograd formulas of the public building blocks, whose backward
-passes are again operators of the same library (the operators on a block's own path have theirs
-as C++ autograd nodes inside ``libmi355moe_torch.so``) -- plus Python wrappers that validate arguments the way the
+under ``torch.compile``; the autograd formulas are C++ nodes inside ``libmi355moe_torch.so`` whose
+backward passes are again operators of the same library) -- plus Python wrappers that validate arguments the way the
 reference's modules do and carry the permutation plan as one object.
 
 Every function requires device tensors and raises if given CPU tensors: the kernels are the
@@ -292,156 +291,11 @@ def _(dout, x, weights, w1, w3, w2, gate, up, token_of_row, slot_of_row, row_of_
 
 
 # ====================================================================== autograd formulas
-# Each differentiable operator's backward is the hand-written kernel for that stage.  The operators on a
-# block's own path (router_gate_fwd, router_select_fwd, grouped_swiglu_fwd, rows_experts_combine_fwd,
-# gather_experts_combine_fwd; linear.py:133-151 is the gate's formula) have theirs as C++ autograd nodes
-# in csrc/torch_autograd.cpp, which run on the engine's thread without the interpreter lock; the formulas
-# below are those of the remaining building blocks.
-# The registration is what ``torch.library.register_autograd`` does -- a Python kernel for the
-# operator's Autograd dispatch key that wraps the call in an ``autograd.Function`` -- without
-# its per-call ``fill_defaults``: that helper re-reads ``schema.arguments`` (a fresh list of
-# wrapped argument objects) once per argument, about 18 us for our twenty-argument operators
-# and a fifth of the host time of a small step, to put back arguments that the dispatcher drops
-# when they equal their schema default.  None of these schemas declares a default, so nothing
-# is ever dropped.
-_AUTOGRAD_LIB = torch.library.Library("mi355_moe", "FRAGMENT")
-_AFTER_AUTOGRAD = torch._C._after_autograd_keyset
-_BELOW_AUTOGRAD = torch._C._AutoDispatchBelowAutograd
-_ANY_REQUIRES_GRAD = torch._C._any_requires_grad
-
-
-def _autograd(name, backward, setup):
-    op = getattr(torch.ops.mi355_moe, name).default
-    if any(a.has_default_value() for a in op._schema.arguments):
-        raise RuntimeError(f"mi355_moe::{name}: schema defaults would need torch.library.register_autograd")
-
-    def forward(ctx, *args):
-        keyset, args = args[-1], args[:-1]
-        with _BELOW_AUTOGRAD():
-            result = op.redispatch(keyset & _AFTER_AUTOGRAD, *args)
-        setup(ctx, args, result)
-        return result
-
-    def backward_(ctx, *grads):
-        ctx.needs_input_grad = ctx.needs_input_grad[:-1]  # the key set rides along as a last, non-tensor input
-        result = backward(ctx, *grads)
-        return (*result, None) if isinstance(result, tuple) else (result, None)
-
-    generated = type(f"GeneratedBackwardFor_mi355_moe_{name}", (torch.autograd.Function,),
-                     {"forward": staticmethod(forward), "backward": staticmethod(backward_)})
-
-    def autograd_kernel(keyset, *args):
-        if torch.is_grad_enabled() and _ANY_REQUIRES_GRAD(*args):
-            return generated.apply(*args, keyset)
-        with _BELOW_AUTOGRAD():
-            return op.redispatch(keyset & _AFTER_AUTOGRAD, *args)
-
-    _AUTOGRAD_LIB.impl(name, autograd_kernel, "Autograd", with_keyset=True)
-
-
-def _rsc_setup(ctx, inputs, output):
-    logits, _bias, _k, score_func, route_norm, route_scale = inputs
-    ctx.save_for_backward(logits, output[1])
-    ctx.cfg = (score_func, route_norm, route_scale)
-    ctx.set_materialize_grads(False)  # no dense zero gradient for an unused score map
-
-
-def _rsc_backward(ctx, dweights, _dids, dscores, _dcutoff):
-    logits, ids = ctx.saved_tensors
-    score_func, route_norm, route_scale = ctx.cfg
-    dlogits = None
-    if ctx.needs_input_grad[0]:
-        dlogits = _O.router_select_bwd(logits, ids, dweights, dscores, score_func, route_norm, route_scale,
-                                       SELECT_TOPK)
-    return (dlogits,) + (None,) * 5
-
-
-_autograd("router_select_cutoff_fwd", _rsc_backward, _rsc_setup)
-
-
-def _rms_setup(ctx, inputs, output):
-    x, weight, _eps = inputs
-    ctx.save_for_backward(x, weight, output[1])
-    ctx.set_materialize_grads(False)
-
-
-def _rms_backward(ctx, dy, _drstd):
-    x, weight, rstd = ctx.saved_tensors
-    need = ctx.needs_input_grad
-    if dy is None or not (need[0] or need[1]):
-        return None, None, None
-    dx, dw = _O.rms_norm_bwd(dy, x, weight, rstd, need[0], need[1])
-    return (dx if need[0] else None), (dw if need[1] else None), None
-
-
-_autograd("rms_norm_fwd", _rms_backward, _rms_setup)
-
-
-def _bl_setup(ctx, inputs, output):
-    scores, _map, pad = inputs
-    ctx.save_for_backward(scores, output, pad)
-
-
-def _bl_backward(ctx, grad):
-    scores, out, pad = ctx.saved_tensors
-    ds = _O.balance_loss_bwd(scores, out[1:], pad, grad[0:1]) if ctx.needs_input_grad[0] else None
-    return ds, None, None
-
-
-_autograd("balance_loss_fwd", _bl_backward, _bl_setup)
-
-
-# -- row gather: backward sums the K row gradients of every token
-def _pr_setup(ctx, inputs, output):
-    x, row_of_slot, _sor, _total, top_k, _cap = inputs
-    ctx.save_for_backward(row_of_slot)
-    ctx.shape = (x.shape[0], top_k)
-
-
-def _pr_backward(ctx, drows):
-    (row_of_slot,) = ctx.saved_tensors
-    dx = _O.permute_rows_bwd(drows, row_of_slot, ctx.shape[0], ctx.shape[1]) if ctx.needs_input_grad[0] else None
-    return dx, None, None, None, None, None
-
-
-_autograd("permute_rows_fwd", _pr_backward, _pr_setup)
-
-
-# -- combine: dY = weights * dout per row, dWeights = <y row, dout row>
-def _cb_setup(ctx, inputs, output):
-    y, weights, row_of_slot, slot_of_row, total_rows, _T, top_k, _round = inputs
-    ctx.save_for_backward(y, weights, row_of_slot, slot_of_row, total_rows)
-    ctx.top_k = top_k
-
-
-def _cb_backward(ctx, dout):
-    y, weights, row_of_slot, slot_of_row, total_rows = ctx.saved_tensors
-    dy, dw = _O.combine_bwd(dout, y, weights, row_of_slot, slot_of_row, total_rows, ctx.top_k)
-    need = ctx.needs_input_grad
-    return ((dy if need[0] else None), (dw.to(weights.dtype) if need[1] else None)) + (None,) * 6
-
-
-_autograd("combine_fwd", _cb_backward, _cb_setup)
-
-
-# -- one grouped linear map (the reference's GroupedExperts._grouped_mm)
-def _gl_setup(ctx, inputs, output):
-    x, w, so, sc, te, tr, nt, zero_fill = inputs
-    ctx.save_for_backward(x, w, so, sc, te, tr, nt)
-    ctx.zero_fill = zero_fill
-    ctx.set_materialize_grads(False)
-
-
-def _gl_backward(ctx, dy):
-    x, w, so, sc, te, tr, nt = ctx.saved_tensors
-    need = ctx.needs_input_grad
-    if dy is None or not (need[0] or need[1]):
-        return (None,) * 8
-    dx, dw = _O.grouped_linear_bwd(dy, x, w, so, sc, te, tr, nt, need[0], need[1], ctx.zero_fill)
-    return ((dx if need[0] else None), (dw if need[1] else None)) + (None,) * 6
-
-
-_autograd("grouped_linear_fwd", _gl_backward, _gl_setup)
+# Each differentiable operator's backward is the hand-written kernel for that stage (linear.py:133-151 is
+# the gate's formula).  The formulas are C++ autograd nodes registered for the operators' Autograd key in
+# csrc/torch_autograd.cpp: they call the backward operators through the dispatcher, so the fake kernels
+# above serve tracing in both directions, and they run on the engine's thread without the interpreter
+# lock.
 
 
 # ====================================================================== router
