@@ -235,3 +235,38 @@ def test_protocol_fallback_matches_the_fused_path_on_the_device(dtype, Dg, Fg, t
         assert metric(v, u) < tol, f"{name}: protocol path vs fused path {metric(v, u)}"
         if r is not None:
             assert metric(v, r) < tol, f"{name}: protocol path vs oracle {metric(v, r)}"
+
+
+def test_own_dispatcher_check_gives_a_tracing_compiler_the_eager_answer():
+    """RoutedExperts decides between the fused kernels and the protocol calls by looking at the
+    dispatcher's four seam methods, instance patches included; a tracing compiler must reach the same
+    decision (it cannot read an instance dictionary, and mis-evaluates hasattr on a bound method)."""
+    from torchllmtuner_amd import moe
+    from torchllmtuner_amd.moe import experts as X
+
+    class Probe(torch.nn.Module):
+        def __init__(self, dispatcher):
+            super().__init__()
+            self.dispatcher = dispatcher
+
+        def forward(self, x):
+            return x + 1 if X._is_own_dispatcher(self.dispatcher) else x - 1
+
+    class Other:
+        def dispatch(self, *a, **k):
+            raise AssertionError
+
+    def free_function(*a, **k):
+        raise AssertionError
+
+    cases = {"plain": None, "function on the instance": free_function, "method of another object": Other().dispatch}
+    for name, patch in cases.items():
+        d = moe.LocalTokenDispatcher(8, 2)
+        if patch is not None:
+            d.dispatch = patch
+        probe = Probe(d)
+        want = 1.0 if patch is None else -1.0
+        assert probe(torch.zeros(1)).item() == want, name
+        torch._dynamo.reset()
+        traced = torch.compile(probe, backend="eager", fullgraph=True)
+        assert traced(torch.zeros(1)).item() == want, name

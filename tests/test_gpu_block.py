@@ -937,3 +937,37 @@ def test_partial_gradient_requests_give_the_same_gradients_and_skip_the_rest(dty
                 assert got[name] is None, (case, name)
             else:
                 assert got[name] is not None and torch.equal(got[name], want), (case, name)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,D,F,shared_F", [(torch.float32, 64, 96, None), (torch.bfloat16, 384, 384, None),
+                                                (torch.bfloat16, 384, 384, 384)])
+def test_whole_block_traces_as_one_graph_and_equals_eager(dtype, D, F, shared_F):
+    """The block under torch.compile(backend="aot_eager", fullgraph=True) -- one graph, forward and
+    backward through the operators' fake kernels and autograd nodes -- gives the eager step bit for bit:
+    output, every gradient, and the counters the block commits.  (The reference traces its experts this
+    way, tests/unit_tests/cpu/test_expert_compile_segments.py:13-40; here the whole block does.)"""
+    print(f"block under torch.compile {dtype} D={D} F={F} shared={shared_F}", flush=True)
+    T, E, K = 300, 8, 2
+    spec = R.RouterSpec(E, K, score_func="sigmoid", route_norm=True)
+    p = make_params(E, D, F, dtype, seed=3, std=0.1, shared_F=shared_F)
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(T, D, generator=g).to(dtype).to(DEV)
+    gout = torch.randn(T, D, generator=g).to(dtype).to(DEV)
+
+    def run(compiled):
+        block = build_block(p, spec, D, F, dtype, DEV)
+        block.train()
+        block.overlap_shared_experts = False  # (a traced block runs on one stream: the same summation order)
+        fn = torch.compile(block, backend="aot_eager", fullgraph=True) if compiled else block
+        xin = x.clone().requires_grad_()
+        out = fn(xin)
+        out.backward(gout)
+        return [out.detach(), xin.grad] + [q.grad for q in block.parameters()] + [block.tokens_per_expert_E.clone()]
+
+    torch._dynamo.reset()
+    eager, traced = run(False), run(True)
+    assert len(eager) == len(traced)
+    for i, (a, b) in enumerate(zip(eager, traced)):
+        assert a is not None and b is not None and torch.equal(a, b), i
+    assert eager[-1].sum() == T * K

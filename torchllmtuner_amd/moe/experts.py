@@ -18,6 +18,7 @@ from __future__ import annotations
 
 from contextlib import AbstractContextManager, nullcontext
 from dataclasses import dataclass
+import types
 from typing import Protocol
 
 import torch
@@ -258,9 +259,16 @@ def _is_own_dispatcher(dispatcher) -> bool:
         _OWN_DISPATCHER_CLASSES[seams] = own
     if not own:
         return False
-    # methods patched onto the instance count as overrides too
-    d = getattr(dispatcher, "__dict__", None)
-    return not d or not ("dispatch" in d or "combine" in d or "plan" in d or "_permute_tokens" in d)
+    # methods patched onto the instance count as overrides too: what the instance hands out must be the
+    # class's function bound to it (written so that a tracing compiler can follow it: no instance dictionary)
+    dispatch, combine, plan, permute = (dispatcher.dispatch, dispatcher.combine, dispatcher.plan,
+                                        dispatcher._permute_tokens)
+    return (
+        isinstance(dispatch, types.MethodType) and dispatch.__func__ is cls.dispatch
+        and isinstance(combine, types.MethodType) and combine.__func__ is cls.combine
+        and isinstance(plan, types.MethodType) and plan.__func__ is cls.plan
+        and isinstance(permute, types.MethodType) and permute.__func__ is cls._permute_tokens
+    )
 
 
 _OWN_DISPATCHER_CLASSES: dict = {}  # a class's four seam methods -> whether they are this package's own

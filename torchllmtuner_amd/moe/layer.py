@@ -194,7 +194,10 @@ class MoE(nn.Module):
         elif self.shared_experts is not None:
             out_TD = out_TD + self.shared_experts(tokens)
         # Commit this block's observations only after both expert paths succeeded.
-        if self.training and not in_checkpoint_recompute.get():
+        # (a tracing compiler runs this once and replays the graph, recomputation included, without
+        # re-entering the module: there is no recompute pass to skip, and it cannot read the context
+        # variable)
+        if self.training and (torch.compiler.is_compiling() or not in_checkpoint_recompute.get()):
             with torch.no_grad():
                 if padding_mask is None:
                     valid_counts_E = num_tokens_per_expert_E  # int32; add_ promotes inside its one kernel

@@ -125,6 +125,10 @@ class LocalTokenDispatcher:
         ids = topk_expert_ids_TK
         lo, hi = self._local_range()
         layout = (self.num_experts, lo, hi, self._align())
+        if torch.compiler.is_compiling():
+            # no memo under a tracing compiler: it would keep traced tensors in module state, and a
+            # tensor's version counter is not a value the trace can branch on
+            return ops.permute_plan(ids, self.num_experts, lo, hi, self._align())
         last = self._last_plan
         if last is not None and last[0]() is ids and last[1] == ids._version and last[3] == layout:
             return last[2]

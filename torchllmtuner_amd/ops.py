@@ -604,8 +604,10 @@ def grouped_linear_bwd(dy_RO, x_RI, w_EOI, plan: PermutePlan, need_dx=True, need
     return _opt(dx, need_dx), _opt(dw, need_dw)
 
 
+@torch.compiler.assume_constant_result
 def combine_bwd_slots(dtype, D, F):
-    """Partials per row of the folded experts+combine backward; 0 when it does not apply."""
+    """Partials per row of the folded experts+combine backward; 0 when it does not apply.  (A pure
+    function of its three constants: a tracing compiler calls it while it traces and keeps the answer.)"""
     if dtype != torch.bfloat16:
         return 0
     return int(_lib.load().mi355_grouped_combine_bwd_slots(_DT[dtype], int(D), int(F)))
