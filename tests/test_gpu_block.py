@@ -971,3 +971,35 @@ def test_whole_block_traces_as_one_graph_and_equals_eager(dtype, D, F, shared_F)
     for i, (a, b) in enumerate(zip(eager, traced)):
         assert a is not None and b is not None and torch.equal(a, b), i
     assert eager[-1].sum() == T * K
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kw", [dict(dispatcher="padded", pad_multiple=128), dict(dispatcher="share", local=(2, 6)),
+                                dict(load_balance_coeff=1e-3)], ids=["padded", "local-share", "expert-bias"])
+def test_traced_block_with_the_other_dispatchers_and_the_expert_bias_equals_eager(kw):
+    """The same one-graph trace for the padded layout, one rank's share of the experts, and a block that
+    carries the load-balancing bias and its counters."""
+    print(f"block under torch.compile {kw}", flush=True)
+    dtype, D, F, T, E, K = torch.bfloat16, 384, 384, 300, 8, 2
+    spec = R.RouterSpec(E, K, score_func="softmax", route_norm=False)
+    p = make_params(E, D, F, dtype, seed=3, std=0.1)
+    if kw.get("dispatcher") == "share":
+        for name in ("w1_EFD", "w3_EFD", "w2_EDF"):
+            setattr(p, name, getattr(p, name)[2:6].clone())
+    if "load_balance_coeff" in kw:
+        p.expert_bias_E = torch.linspace(-0.1, 0.1, E)
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(T, D, generator=g).to(dtype).to(DEV)
+    gout = torch.randn(T, D, generator=g).to(dtype).to(DEV)
+
+    def run(compiled):
+        block = build_block(p, spec, D, F, dtype, DEV, **kw)
+        block.train()
+        fn = torch.compile(block, backend="aot_eager", fullgraph=True) if compiled else block
+        xin = x.clone().requires_grad_()
+        fn(xin).backward(gout)
+        return [xin.grad] + [q.grad for q in block.parameters()] + [block.tokens_per_expert_E.clone()]
+
+    torch._dynamo.reset()
+    for i, (a, b) in enumerate(zip(run(False), run(True))):
+        assert (a is None and b is None) or torch.equal(a, b), i
