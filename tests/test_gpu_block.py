@@ -1003,3 +1003,69 @@ def test_traced_block_with_the_other_dispatchers_and_the_expert_bias_equals_eage
     torch._dynamo.reset()
     for i, (a, b) in enumerate(zip(run(False), run(True))):
         assert (a is None and b is None) or torch.equal(a, b), i
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,D,F", [(torch.float32, 64, 96), (torch.bfloat16, 384, 384)])
+def test_second_backward_through_a_kept_graph_and_checkpointed_recomputation(dtype, D, F):
+    """The autograd nodes keep what they saved when the graph is kept: a second backward pass gives the
+    same gradients again (accumulated: exactly twice the first).  Under torch.utils.checkpoint the block
+    is run again inside the backward pass: the same output gradient reaches the same kernels, so input
+    and weight gradients equal the plain run's bit for bit."""
+    from torch.utils.checkpoint import checkpoint
+
+    T, E, K = 150, 8, 2
+    spec = R.RouterSpec(E, K, score_func="softmax", route_norm=True)
+    p = make_params(E, D, F, dtype, seed=9, std=0.1, shared_F=F)
+    g = torch.Generator().manual_seed(21)
+    x = torch.randn(T, D, generator=g).to(dtype).to(DEV)
+    gout = torch.randn(T, D, generator=g).to(dtype).to(DEV)
+
+    def grads_of(block, xin):
+        return [xin.grad.clone()] + [q.grad.clone() for q in block.parameters()]
+
+    block = build_block(p, spec, D, F, dtype, DEV)
+    block.train()
+    block.overlap_shared_experts = False
+    xin = x.clone().requires_grad_()
+    out = block(xin)
+    out.backward(gout, retain_graph=True)
+    once = grads_of(block, xin)
+    out.backward(gout)
+    twice = grads_of(block, xin)
+    for a, b in zip(once, twice):
+        assert torch.equal(b.float(), 2 * a.float()) or rel_max(b.float(), 2 * a.float()) < 1e-2  # bf16 accumulation rounds
+
+    block2 = build_block(p, spec, D, F, dtype, DEV)
+    block2.train()
+    block2.overlap_shared_experts = False
+    xin2 = x.clone().requires_grad_()
+    checkpoint(block2, xin2, use_reentrant=False).backward(gout)
+    for a, b in zip(once, grads_of(block2, xin2)):
+        assert torch.equal(a, b)
+    # the replay stops at the last tensor the backward needs, before the block commits its counters at the
+    # end of forward (layer.py:246-309 commits last for the same reason): one pass is counted.  A wrapper
+    # that replays whole forwards sets the reference's context variable (models/common/aux_loss.py:42-43)
+    # and has the replay skipped, below.
+    assert block2.tokens_per_expert_E.sum() == T * K
+
+    from contextlib import contextmanager, nullcontext
+
+    from torchllmtuner_amd.moe.layer import in_checkpoint_recompute
+
+    @contextmanager
+    def replaying():
+        token = in_checkpoint_recompute.set(True)
+        try:
+            yield
+        finally:
+            in_checkpoint_recompute.reset(token)
+
+    block3 = build_block(p, spec, D, F, dtype, DEV)
+    block3.train()
+    block3.overlap_shared_experts = False
+    xin3 = x.clone().requires_grad_()
+    checkpoint(block3, xin3, use_reentrant=False, context_fn=lambda: (nullcontext(), replaying())).backward(gout)
+    for a, b in zip(once, grads_of(block3, xin3)):
+        assert torch.equal(a, b)
+    assert block3.tokens_per_expert_E.sum() == T * K
